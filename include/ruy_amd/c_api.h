@@ -1,0 +1,212 @@
+/* C ABI of the gfx950 (MI355X) implementation of ruy's matrix-multiplication
+ * hot path.
+ *
+ * This is the drop-in boundary: everything above it (the `ruy::Mul` templates
+ * in include/ruy/, the Python mirror in ruy_amd/) only flattens its arguments
+ * into the plain structs below and calls these functions. Nothing in the
+ * signatures depends on C++, torch or HIP types; a HIP stream is passed as an
+ * opaque `void*`.
+ *
+ * Every entry point cites the piece of the reference (google/ruy) that it
+ * replaces, as file:line into the reference tree.
+ *
+ * All functions return 0 on success and a non-zero RUYAMD_E_* code on failure
+ * unless stated otherwise; `ruyamd_ctx_last_error` gives the message of the
+ * last failure on a context. There is no CPU fallback: if no gfx950 device is
+ * usable, `ruyamd_ctx_create` fails.
+ */
+#ifndef RUY_AMD_C_API_H_
+#define RUY_AMD_C_API_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RUYAMD_API __attribute__((visibility("default")))
+
+/* Storage order of a matrix. Values are those of ruy::Order
+ * (ruy/matrix.h:29). */
+enum {
+  RUYAMD_ORDER_COL_MAJOR = 0,
+  RUYAMD_ORDER_ROW_MAJOR = 1,
+};
+
+/* Scalar type ids. 1..4 are the ids ruy's own kernels use
+ * (RUY_ASM_TYPE_ID_*, ruy/kernel_common.h:66-69); 5 and 6 are added for the
+ * floating-point types. */
+enum {
+  RUYAMD_DTYPE_U8 = 1,
+  RUYAMD_DTYPE_I8 = 2,
+  RUYAMD_DTYPE_I16 = 3,
+  RUYAMD_DTYPE_I32 = 4,
+  RUYAMD_DTYPE_F32 = 5,
+  RUYAMD_DTYPE_F64 = 6,
+};
+
+/* Values of ruy::CachePolicy (ruy/matrix.h:117-122). */
+enum {
+  RUYAMD_CACHE_NEVER = 0,
+  RUYAMD_CACHE_IF_LARGE_SPEEDUP = 1,
+  RUYAMD_CACHE_IF_SIGNIFICANT_SPEEDUP = 2,
+  RUYAMD_CACHE_ALWAYS = 3,
+};
+
+/* Values of ruy::ChannelDimension (ruy/mul_params.h:31-36). */
+enum {
+  RUYAMD_CHANNEL_ROW = 0,
+  RUYAMD_CHANNEL_COL = 1,
+};
+
+/* Bits of the path mask. The low four bits keep the values of ruy::Path's
+ * architecture-independent paths (ruy/path.h:55-69) so that callers' masks
+ * keep compiling; only RUYAMD_PATH_GFX950 ever executes. */
+enum {
+  RUYAMD_PATH_NONE = 0,
+  RUYAMD_PATH_STANDARD_CPP = 0x1,
+  RUYAMD_PATH_GFX950 = 0x10,
+};
+
+/* Error codes. */
+enum {
+  RUYAMD_OK = 0,
+  RUYAMD_E_INVALID = 1,     /* malformed descriptor / illegal parameter combo */
+  RUYAMD_E_UNSUPPORTED = 2, /* type tuple that ruy::Mul does not define */
+  RUYAMD_E_HIP = 3,         /* a HIP runtime call failed */
+  RUYAMD_E_NO_PATH = 4,     /* the enabled-path mask excludes gfx950 */
+  RUYAMD_E_NO_DEVICE = 5,   /* no usable gfx950 device */
+};
+
+/* Which device kernel served the last ruyamd_mul call (diagnostics/tests). */
+enum {
+  RUYAMD_KERNEL_NONE = 0,
+  RUYAMD_KERNEL_GENERIC = 1,   /* one output per lane, any type/layout */
+  RUYAMD_KERNEL_I8_MFMA = 2,   /* v_mfma_i32_32x32x32_i8 GEMM */
+  RUYAMD_KERNEL_F32_MFMA = 3,  /* v_mfma_f32_32x32x2_f32 GEMM */
+  RUYAMD_KERNEL_I8_GEMV = 4,   /* wavefront-reduction skinny kernel, cols<=8 */
+  RUYAMD_KERNEL_I8I16_MFMA = 5,/* int8 x int16 as two int8 MFMA planes */
+  RUYAMD_KERNEL_F32_GEMV = 6,  /* fp32 skinny kernel */
+};
+
+/* Type-erased, non-owning matrix view: the fields of ruy::Matrix<T>
+ * (ruy/matrix.h:132-167) / ruy::EMat (ruy/mat.h:236-242).
+ * Element (r, c) lives at data[r * rs + c * cs] with (rs, cs) = (1, stride)
+ * for column-major and (stride, 1) for row-major (ruy/matrix.h:188-199);
+ * `stride` is in elements. `data` may be a device pointer (the measured path)
+ * or a host pointer (staged through device memory by the library). */
+typedef struct ruyamd_mat {
+  void* data;
+  int32_t rows;
+  int32_t cols;
+  int32_t stride;
+  int32_t zero_point;
+  uint8_t order;
+  uint8_t dtype;
+  uint8_t cache_policy;
+  uint8_t reserved;
+} ruyamd_mat;
+
+/* The fields of ruy::MulParams<AccumScalar, DstScalar>
+ * (ruy/mul_params.h:97-214, storage :219-297). The clamp bounds are DstScalar
+ * values widened to double, which is exact for every supported DstScalar.
+ * `bias` has AccumScalar elements. The per-channel arrays are both either
+ * NULL (use the scalar multiplier) or non-NULL. */
+typedef struct ruyamd_mul_params {
+  const void* bias;
+  const int32_t* multiplier_fixedpoint_perchannel;
+  const int32_t* multiplier_exponent_perchannel;
+  int32_t multiplier_fixedpoint;
+  int32_t multiplier_exponent;
+  double clamp_min;
+  double clamp_max;
+  uint8_t accum_dtype;
+  uint8_t channel_dimension;
+  uint8_t perchannel_buffers_capacity_rounding_log2;
+  uint8_t reserved;
+} ruyamd_mul_params;
+
+typedef struct ruyamd_ctx ruyamd_ctx;
+
+/* Replaces ruy::Context::Context / ~Context (ruy/context.cc:29-30,
+ * ruy/ctx_impl.h:57-82): per-caller state = HIP stream, device workspace,
+ * prepacked-matrix cache, last used path, knobs. Not thread-safe, like
+ * ruy::Context (ruy/ruy.h:82-95): one context per calling thread. */
+RUYAMD_API int ruyamd_ctx_create(ruyamd_ctx** out);
+RUYAMD_API void ruyamd_ctx_destroy(ruyamd_ctx* ctx);
+
+/* Replaces ruy::Mul (ruy/ruy.h:36-48,96-102) and everything below it:
+ * MulFrontEnd (ruy/frontend.h:80-95), PreparePackedMatrices
+ * (ruy/prepare_packed_matrices.cc:70-95), TrMul (ruy/trmul.cc:309-422),
+ * RunPack (ruy/pack.h:135-151) and RunKernel (ruy/kernel.h:57-139).
+ * Computes dst = epilogue(lhs * rhs) with ReferenceMul's arithmetic
+ * (ruy/reference_mul.h:29-52). By default dst is complete when the call
+ * returns. */
+RUYAMD_API int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs,
+                          const ruyamd_mat* rhs,
+                          const ruyamd_mul_params* params,
+                          const ruyamd_mat* dst);
+
+/* Stream control. By default a context owns a stream and every ruyamd_mul
+ * synchronises it before returning, which is ruy::Mul's contract
+ * (ruy/thread_pool.cc:239 waits for all workers). `ruyamd_ctx_set_stream`
+ * makes the context launch on a caller-owned hipStream_t (NULL = the legacy
+ * default stream); `ruyamd_ctx_set_synchronous(ctx, 0)` makes calls whose
+ * operands are all device-resident return after enqueueing. */
+RUYAMD_API int ruyamd_ctx_set_stream(ruyamd_ctx* ctx, void* hip_stream);
+RUYAMD_API int ruyamd_ctx_set_synchronous(ruyamd_ctx* ctx, int synchronous);
+RUYAMD_API int ruyamd_ctx_synchronize(ruyamd_ctx* ctx);
+
+/* ruy::Context accessors (ruy/context.h:45-96, ruy/ctx.cc:67-178). The
+ * thread-count, tuning and strategy knobs are stored and returned but have no
+ * effect on the single-stream device path. */
+RUYAMD_API int ruyamd_ctx_last_used_path(const ruyamd_ctx* ctx);
+RUYAMD_API int ruyamd_ctx_get_runtime_enabled_paths(ruyamd_ctx* ctx);
+RUYAMD_API void ruyamd_ctx_set_runtime_enabled_paths(ruyamd_ctx* ctx,
+                                                     int paths);
+RUYAMD_API int ruyamd_ctx_max_num_threads(const ruyamd_ctx* ctx);
+RUYAMD_API void ruyamd_ctx_set_max_num_threads(ruyamd_ctx* ctx, int value);
+RUYAMD_API int ruyamd_ctx_explicit_tuning(const ruyamd_ctx* ctx);
+RUYAMD_API void ruyamd_ctx_set_explicit_tuning(ruyamd_ctx* ctx, int value);
+RUYAMD_API int ruyamd_ctx_num_threads_strategy(const ruyamd_ctx* ctx);
+RUYAMD_API void ruyamd_ctx_set_num_threads_strategy(ruyamd_ctx* ctx,
+                                                    int value);
+RUYAMD_API int ruyamd_ctx_performance_advisory(const ruyamd_ctx* ctx,
+                                               int advisory);
+
+/* Prepacked-matrix cache (ruy/prepacked_cache.h:45-127,
+ * ruy/context.h:83-88). Count and byte accounting follow
+ * PrepackedCache::MatrixCount / BuffersBytes (ruy/prepacked_cache.h:104-107);
+ * `set_cache_max_bytes` plays the role of PrepackedCache's constructor
+ * argument (ruy/prepacked_cache.h:98-99) and clears the cache. */
+RUYAMD_API void ruyamd_ctx_clear_prepacked_cache(ruyamd_ctx* ctx);
+RUYAMD_API int ruyamd_ctx_cache_matrix_count(const ruyamd_ctx* ctx);
+RUYAMD_API int64_t ruyamd_ctx_cache_buffers_bytes(const ruyamd_ctx* ctx);
+RUYAMD_API void ruyamd_ctx_set_cache_max_bytes(ruyamd_ctx* ctx,
+                                               int64_t max_bytes);
+
+/* Diagnostics. */
+RUYAMD_API const char* ruyamd_ctx_last_error(const ruyamd_ctx* ctx);
+RUYAMD_API int ruyamd_ctx_last_kernel(const ruyamd_ctx* ctx);
+/* Restricts dispatch to the generic kernel when `force` is non-zero
+ * (differential testing of the tuned kernels against the simple one, the
+ * role of ruy's kInternalStandardCppVariant paths, ruy/kernel.h:150-169). */
+RUYAMD_API void ruyamd_ctx_force_generic_kernel(ruyamd_ctx* ctx, int force);
+
+/* detail::MultiplyByQuantizedMultiplier (ruy/apply_multiplier.cc:48-65)
+ * evaluated ON THE DEVICE for n inputs: out[i] = MBQM(x[i], m[i], e[i]).
+ * All pointers are device or host pointers like matrix data. Exists so the
+ * requantizer's known-answer tests run against the device arithmetic. */
+RUYAMD_API int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x,
+                                       const int32_t* m, const int32_t* e,
+                                       int32_t* out, int64_t n);
+
+/* Library version string. */
+RUYAMD_API const char* ruyamd_version(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* RUY_AMD_C_API_H_ */

@@ -1,0 +1,121 @@
+/* TEST INFRASTRUCTURE — NOT PART OF THE PRODUCT.
+ *
+ * CPU restatement of the arithmetic of ruy::Mul, used only as the checker in
+ * tests/, in the smoke test and as the "port" CPU-baseline leg of bench.py.
+ * The shipped library never links, loads or calls anything in this directory.
+ *
+ * The structs deliberately have the same field order and types as
+ * ruyamd_mat / ruyamd_mul_params in include/ruy_amd/c_api.h so that a test
+ * can hand one descriptor to both the device library and this checker; the
+ * definitions are repeated here so the checker builds on its own.
+ *
+ * What follows which part of the reference:
+ *   oracle_mbqm        detail::MultiplyByQuantizedMultiplier
+ *                      ruy/apply_multiplier.cc:48-65
+ *   oracle_mul         ReferenceMul  ruy/reference_mul.h:29-52
+ *                      (element addressing ruy/matrix.h:188-199,
+ *                       multiplier selection ruy/apply_multiplier.h:67-79)
+ *   oracle_validate    ValidateZeroPoints  ruy/validate.h:40-75
+ *   oracle_pack_sums   generic PackImpl::Run  ruy/pack.h:105-132 with the
+ *                      uint8->int8 conversion of ruy/pack_common.h:36-58
+ *   oracle_mul_packed  the expanded accumulator form of the StandardCpp
+ *                      kernel  ruy/kernel.h:174-241
+ *
+ * Pinning (what each function is checked against, in tests/):
+ *   oracle_mbqm       - all 32 known answers of
+ *                       ruy/apply_multiplier_test.cc:39-93 and the 5 of
+ *                       :105-124; exact rational floor(x*m/2^(31-e)+1/2) with
+ *                       Python big integers on random and extreme inputs.
+ *   oracle_mul        - the saturation known answers of
+ *                       ruy/test_overflow_dst_zero_point.cc:47-125; the six
+ *                       hand-computable cases of example/example.cc:21-192;
+ *                       numpy int64 matmul of (l-zl)(r-zr) reduced mod 2^32;
+ *                       invariance under storage order / stride / transposed
+ *                       problem; stock ruy (oracle/_ref, Path::kStandardCpp and
+ *                       ReferenceMul) when that build is present.
+ *   oracle_pack_sums,
+ *   oracle_mul_packed - identity with oracle_mul (ruy/kernel.h:224-232 is
+ *                       algebraically reference_mul.h:38 mod 2^32).
+ */
+#ifndef RUY_AMD_ORACLE_REF_MUL_H_
+#define RUY_AMD_ORACLE_REF_MUL_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ORACLE_COL_MAJOR = 0, ORACLE_ROW_MAJOR = 1 };
+enum {
+  ORACLE_U8 = 1,
+  ORACLE_I8 = 2,
+  ORACLE_I16 = 3,
+  ORACLE_I32 = 4,
+  ORACLE_F32 = 5,
+  ORACLE_F64 = 6
+};
+enum { ORACLE_CHANNEL_ROW = 0, ORACLE_CHANNEL_COL = 1 };
+
+typedef struct oracle_mat {
+  void* data;
+  int32_t rows;
+  int32_t cols;
+  int32_t stride;
+  int32_t zero_point;
+  uint8_t order;
+  uint8_t dtype;
+  uint8_t cache_policy;
+  uint8_t reserved;
+} oracle_mat;
+
+typedef struct oracle_mul_params {
+  const void* bias;
+  const int32_t* multiplier_fixedpoint_perchannel;
+  const int32_t* multiplier_exponent_perchannel;
+  int32_t multiplier_fixedpoint;
+  int32_t multiplier_exponent;
+  double clamp_min;
+  double clamp_max;
+  uint8_t accum_dtype;
+  uint8_t channel_dimension;
+  uint8_t perchannel_buffers_capacity_rounding_log2;
+  uint8_t reserved;
+} oracle_mul_params;
+
+/* ruy/apply_multiplier.cc:48-65. Requires e >= -31. */
+int32_t oracle_mbqm(int32_t x, int32_t m, int e);
+
+/* ruy/validate.h:40-75 plus the static type constraints of
+ * ruy/mul_params.h:219-297. Returns 0 when (lhs, rhs, params, dst) is a legal
+ * ruy::Mul call. */
+int oracle_validate(const oracle_mat* lhs, const oracle_mat* rhs,
+                    const oracle_mul_params* params, const oracle_mat* dst);
+
+/* ruy/reference_mul.h:29-52. Returns 0 on success, non-zero if the call is not
+ * legal. `*overflow` (may be NULL) is set to 1 if any exact integer
+ * accumulator (before the multiplier) left the int32 range, i.e. the int32
+ * result relied on wrap-around. Uses OpenMP over dst rows when built with it. */
+int oracle_mul(const oracle_mat* lhs, const oracle_mat* rhs,
+               const oracle_mul_params* params, const oracle_mat* dst,
+               int* overflow);
+
+/* ruy/pack.h:105-132 for an integer source: `src` is the matrix whose COLUMNS
+ * are packed (the transposed LHS, or the RHS), `depth_padded` >= src->rows and
+ * `cols_padded` >= src->cols give the packed size, `packed` receives the
+ * column-major int8/int16 packed values (uint8 minus 128; padding = packed
+ * zero point), `sums` one int32 per packed column. */
+int oracle_pack_sums(const oracle_mat* src, int depth_padded, int cols_padded,
+                     void* packed, int32_t* sums);
+
+/* ruy/kernel.h:174-241: integer Mul computed from packed operands and sums
+ * with the expanded zero-point form. Must equal oracle_mul. */
+int oracle_mul_packed(const oracle_mat* lhs, const oracle_mat* rhs,
+                      const oracle_mul_params* params, const oracle_mat* dst,
+                      int depth_round);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RUY_AMD_ORACLE_REF_MUL_H_ */
