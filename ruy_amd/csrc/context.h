@@ -1,0 +1,66 @@
+// Per-caller state behind ruyamd_ctx: the counterpart of ruy::CtxImpl
+// (ruy/ctx_impl.h:57-82) for a device: a stream, a grow-only device workspace
+// that replaces the bump allocator (ruy/allocator.h:56-97), the
+// prepacked-matrix cache, and the knobs ruy::Context exposes.
+#ifndef RUY_AMD_CSRC_CONTEXT_H_
+#define RUY_AMD_CSRC_CONTEXT_H_
+
+#include <hip/hip_runtime.h>
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "internal.h"
+#include "prepacked_cache.h"
+
+namespace ruyamd {
+
+// Device scratch memory handed out by bumping a pointer; everything is
+// released together at the start of the next call (ruy's
+// Allocator::FreeAll, ruy/frontend.cc:34). If a call outgrows the current
+// block an extra block is taken, and the next Reset replaces all blocks with
+// one that is large enough.
+class Workspace {
+ public:
+  ~Workspace();
+  // 256-byte aligned device memory valid until the next Reset; nullptr on
+  // allocation failure.
+  void* Alloc(std::size_t bytes);
+  // Call only when no kernel still uses the previous call's scratch.
+  void Reset();
+  std::size_t capacity() const;
+
+ private:
+  struct Block {
+    char* base;
+    std::size_t size;
+    std::size_t used;
+  };
+  std::vector<Block> blocks_;
+};
+
+}  // namespace ruyamd
+
+struct ruyamd_ctx {
+  int device = 0;
+  hipStream_t own_stream = nullptr;
+  hipStream_t stream = nullptr;
+  bool synchronous = true;
+  bool pending_async = false;  // work enqueued by an asynchronous call
+  int last_used_path = RUYAMD_PATH_NONE;
+  int runtime_enabled_paths = RUYAMD_PATH_NONE;  // kNone = not decided yet
+  int max_num_threads = 1;
+  int explicit_tuning = 0;        // ruy::Tuning::kAuto
+  int num_threads_strategy = 0;   // ruy::NumThreadsStrategy::kDefault
+  int performance_advisories = 0;
+  int last_kernel = RUYAMD_KERNEL_NONE;
+  bool force_generic = false;
+  std::string last_error;
+  ruyamd::Workspace workspace;
+  std::unique_ptr<ruyamd::PrepackedCache> cache;
+  // Host staging of the destination: copies to perform after the kernel.
+  int multiprocessor_count = 0;
+};
+
+#endif  // RUY_AMD_CSRC_CONTEXT_H_

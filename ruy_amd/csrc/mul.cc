@@ -1,0 +1,271 @@
+// ruyamd_mul: the front end and dispatcher. It stands where the reference has
+// MulFrontEnd (ruy/frontend.h:45-95), CreateTrMulParams
+// (ruy/create_trmul_params.h:403-480), PreparePackedMatrices
+// (ruy/prepare_packed_matrices.cc:38-95) and TrMul (ruy/trmul.cc:309-422):
+// validate, choose the path, make operands device-resident, consult the
+// prepacked cache, pick one kernel, launch it on the context's stream.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <limits>
+#include <string>
+
+#include "context.h"
+#include "internal.h"
+#include "plan.h"
+
+namespace ruyamd {
+namespace {
+
+int Fail(ruyamd_ctx* ctx, int code, const std::string& msg) {
+  ctx->last_error = msg;
+  return code;
+}
+
+int TypeLowest(int dtype) {
+  switch (dtype) {
+    case RUYAMD_DTYPE_U8:
+      return 0;
+    case RUYAMD_DTYPE_I8:
+      return -128;
+    case RUYAMD_DTYPE_I16:
+      return -32768;
+    default:
+      return std::numeric_limits<int32_t>::lowest();
+  }
+}
+
+// The static type constraints of ruy::MulParams (ruy/mul_params.h:219-297),
+// the shape agreement ruy::Mul assumes, and ValidateZeroPoints
+// (ruy/validate.h:40-75). The reference checks the latter only in debug
+// builds; a C ABI cannot rely on that, so they are errors here.
+int Validate(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
+             const ruyamd_mul_params* p, const ruyamd_mat* dst) {
+  if (!lhs || !rhs || !p || !dst) return Fail(ctx, RUYAMD_E_INVALID, "null argument");
+  const ruyamd_mat* mats[3] = {lhs, rhs, dst};
+  const char* names[3] = {"lhs", "rhs", "dst"};
+  for (int s = 0; s < 3; ++s) {
+    const ruyamd_mat* m = mats[s];
+    if (m->rows < 0 || m->cols < 0) return Fail(ctx, RUYAMD_E_INVALID, std::string(names[s]) + ": negative size");
+    if (m->order != RUYAMD_ORDER_COL_MAJOR && m->order != RUYAMD_ORDER_ROW_MAJOR)
+      return Fail(ctx, RUYAMD_E_INVALID, std::string(names[s]) + ": bad order");
+    if (!DtypeSize(m->dtype)) return Fail(ctx, RUYAMD_E_INVALID, std::string(names[s]) + ": bad dtype");
+    const int inner = m->order == RUYAMD_ORDER_COL_MAJOR ? m->rows : m->cols;
+    if (m->stride < inner) return Fail(ctx, RUYAMD_E_INVALID, std::string(names[s]) + ": stride smaller than the contiguous dimension");
+    if (m->rows > 0 && m->cols > 0 && !m->data)
+      return Fail(ctx, RUYAMD_E_INVALID, std::string(names[s]) + ": null data");
+    if (m->cache_policy > RUYAMD_CACHE_ALWAYS) return Fail(ctx, RUYAMD_E_INVALID, std::string(names[s]) + ": bad cache policy");
+  }
+  if (lhs->cols != rhs->rows || dst->rows != lhs->rows || dst->cols != rhs->cols)
+    return Fail(ctx, RUYAMD_E_INVALID, "shape mismatch: need lhs MxK, rhs KxN, dst MxN");
+  if (p->channel_dimension > RUYAMD_CHANNEL_COL) return Fail(ctx, RUYAMD_E_INVALID, "bad channel dimension");
+  const bool fp = IsFloating(dst->dtype);
+  if (fp) {
+    if (!IsFloating(p->accum_dtype) || !IsFloating(lhs->dtype) || !IsFloating(rhs->dtype))
+      return Fail(ctx, RUYAMD_E_UNSUPPORTED, "floating-point destination needs floating-point operands and accumulator");
+    if (DtypeSize(dst->dtype) > DtypeSize(p->accum_dtype))
+      return Fail(ctx, RUYAMD_E_UNSUPPORTED, "destination wider than accumulator");
+    if (lhs->zero_point || rhs->zero_point || dst->zero_point)
+      return Fail(ctx, RUYAMD_E_INVALID, "floating-point matrices need zero_point == 0");
+    if (p->multiplier_fixedpoint_perchannel || p->multiplier_exponent_perchannel)
+      return Fail(ctx, RUYAMD_E_INVALID, "multiplier set on a floating-point Mul");
+  } else {
+    if (p->accum_dtype != RUYAMD_DTYPE_I32)
+      return Fail(ctx, RUYAMD_E_UNSUPPORTED, "integer destination needs an int32 accumulator");
+    if (lhs->dtype > RUYAMD_DTYPE_I16 || rhs->dtype > RUYAMD_DTYPE_I16)
+      return Fail(ctx, RUYAMD_E_UNSUPPORTED, "integer operands must be uint8, int8 or int16");
+    const bool has16 = lhs->dtype == RUYAMD_DTYPE_I16 || rhs->dtype == RUYAMD_DTYPE_I16;
+    if (has16 && (lhs->zero_point || rhs->zero_point || dst->zero_point))
+      return Fail(ctx, RUYAMD_E_INVALID, "int16 operands need all zero points == 0");
+    if (!(lhs->dtype == RUYAMD_DTYPE_U8 && rhs->dtype == RUYAMD_DTYPE_U8) &&
+        lhs->zero_point == TypeLowest(lhs->dtype) && rhs->zero_point == TypeLowest(rhs->dtype))
+      return Fail(ctx, RUYAMD_E_INVALID, "both source zero points at the type minimum");
+    if ((p->multiplier_fixedpoint_perchannel != nullptr) != (p->multiplier_exponent_perchannel != nullptr))
+      return Fail(ctx, RUYAMD_E_INVALID, "per-channel multiplier needs both arrays");
+    if (dst->dtype == RUYAMD_DTYPE_I32 && p->multiplier_fixedpoint_perchannel)
+      return Fail(ctx, RUYAMD_E_INVALID, "multiplier set on a raw int32 destination");
+    if (dst->dtype != RUYAMD_DTYPE_I32 && !p->multiplier_fixedpoint_perchannel &&
+        p->multiplier_exponent < -31)
+      return Fail(ctx, RUYAMD_E_INVALID, "multiplier_exponent below -31");  // ruy/apply_multiplier.cc:51
+  }
+  return RUYAMD_OK;
+}
+
+bool IsDevicePointer(const void* p) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+    (void)hipGetLastError();  // unregistered host memory
+    return false;
+  }
+  return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged ||
+         attr.type == hipMemoryTypeArray;
+}
+
+int64_t StorageElements(const ruyamd_mat& m) {
+  const int64_t inner = m.order == RUYAMD_ORDER_COL_MAJOR ? m.rows : m.cols;
+  const int64_t outer = m.order == RUYAMD_ORDER_COL_MAJOR ? m.cols : m.rows;
+  if (inner == 0 || outer == 0) return 0;
+  return (outer - 1) * m.stride + inner;
+}
+
+// Makes `bytes` of possibly-host memory readable on the device.
+const void* StageIn(ruyamd_ctx* ctx, const void* p, std::size_t bytes, bool* staged_any, bool* ok) {
+  if (!p || bytes == 0 || IsDevicePointer(p)) return p;
+  void* d = ctx->workspace.Alloc(bytes);
+  if (!d || hipMemcpyAsync(d, p, bytes, hipMemcpyHostToDevice, ctx->stream) != hipSuccess) {
+    *ok = false;
+    return nullptr;
+  }
+  *staged_any = true;
+  return d;
+}
+
+DevMat ToDevMat(const ruyamd_mat& m, const void* device_data) {
+  DevMat d;
+  d.data = const_cast<void*>(device_data);
+  d.rows = m.rows;
+  d.cols = m.cols;
+  d.rs = m.order == RUYAMD_ORDER_COL_MAJOR ? 1 : m.stride;
+  d.cs = m.order == RUYAMD_ORDER_ROW_MAJOR ? 1 : m.stride;
+  d.dtype = m.dtype;
+  d.zero_point = m.zero_point;
+  return d;
+}
+
+int32_t ClampToInt32(double v) {
+  if (v >= 2147483647.0) return std::numeric_limits<int32_t>::max();
+  if (v <= -2147483648.0) return std::numeric_limits<int32_t>::lowest();
+  return static_cast<int32_t>(v);
+}
+
+}  // namespace
+}  // namespace ruyamd
+
+using namespace ruyamd;
+
+extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
+                          const ruyamd_mul_params* p, const ruyamd_mat* dst) {
+  if (!ctx) return RUYAMD_E_INVALID;
+  ctx->performance_advisories = 0;  // ruy/frontend.h:86 clears them per call
+  if (int rc = Validate(ctx, lhs, rhs, p, dst)) return rc;
+
+  // ruy/ctx.cc:175-178: most significant of (compiled & enabled). The only
+  // compiled path of this library is gfx950.
+  const int enabled = ruyamd_ctx_get_runtime_enabled_paths(ctx);
+  if (!(enabled & RUYAMD_PATH_GFX950)) {
+    ctx->last_used_path = RUYAMD_PATH_NONE;
+    return Fail(ctx, RUYAMD_E_NO_PATH,
+                "runtime-enabled paths exclude gfx950 and this library has no CPU path");
+  }
+  ctx->last_used_path = RUYAMD_PATH_GFX950;
+  ctx->last_kernel = RUYAMD_KERNEL_NONE;
+
+  if (hipSetDevice(ctx->device) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "hipSetDevice failed");
+  if (dst->rows == 0 || dst->cols == 0) return RUYAMD_OK;
+
+  // The previous call's scratch may still be in use by an asynchronous launch.
+  if (ctx->pending_async && ctx->workspace.capacity() > 0) {
+    // Stream order protects reuse: every user of the scratch was enqueued on
+    // ctx->stream before anything this call enqueues.
+  }
+  ctx->workspace.Reset();
+
+  bool staged = false, ok = true;
+  const int channels = p->channel_dimension == RUYAMD_CHANNEL_ROW ? dst->rows : dst->cols;
+  const void* lhs_d = StageIn(ctx, lhs->data, StorageElements(*lhs) * DtypeSize(lhs->dtype), &staged, &ok);
+  const void* rhs_d = StageIn(ctx, rhs->data, StorageElements(*rhs) * DtypeSize(rhs->dtype), &staged, &ok);
+  const void* bias_d = StageIn(ctx, p->bias, std::size_t(channels) * DtypeSize(p->accum_dtype), &staged, &ok);
+  const void* mf_d = StageIn(ctx, p->multiplier_fixedpoint_perchannel, std::size_t(channels) * 4, &staged, &ok);
+  const void* me_d = StageIn(ctx, p->multiplier_exponent_perchannel, std::size_t(channels) * 4, &staged, &ok);
+  if (!ok) return Fail(ctx, RUYAMD_E_HIP, "staging host operands to the device failed");
+
+  // Destination: device memory is written in place; host memory gets a device
+  // image with the same stride that is copied back row by row (column by
+  // column), so the padding between them is never touched.
+  const bool dst_on_device = IsDevicePointer(dst->data);
+  void* dst_d = dst->data;
+  const std::size_t dst_elt = DtypeSize(dst->dtype);
+  if (!dst_on_device) {
+    dst_d = ctx->workspace.Alloc(StorageElements(*dst) * dst_elt);
+    if (!dst_d) return Fail(ctx, RUYAMD_E_HIP, "device allocation for the destination failed");
+  }
+
+  MulCall call;
+  call.lhs = ToDevMat(*lhs, lhs_d);
+  call.rhs = ToDevMat(*rhs, rhs_d);
+  call.dst = ToDevMat(*dst, dst_d);
+  call.lhs_src_key = lhs->data;
+  call.rhs_src_key = rhs->data;
+  call.lhs_cache_policy = lhs->cache_policy;
+  call.rhs_cache_policy = rhs->cache_policy;
+  call.accum_dtype = p->accum_dtype;
+  Epilogue& ep = call.ep;
+  ep.bias = bias_d;
+  ep.mult_fixedpoint = static_cast<const int32_t*>(mf_d);
+  ep.mult_exponent = static_cast<const int32_t*>(me_d);
+  ep.mult_fixedpoint_scalar = p->multiplier_fixedpoint;
+  ep.mult_exponent_scalar = p->multiplier_exponent;
+  ep.dst_zero_point = dst->zero_point;
+  ep.channel_is_col = p->channel_dimension == RUYAMD_CHANNEL_COL;
+  const bool fp = IsFloating(dst->dtype);
+  ep.requantize = !fp && dst->dtype != RUYAMD_DTYPE_I32;
+  if (fp) {
+    ep.clamp_min_f = static_cast<float>(p->clamp_min);
+    ep.clamp_max_f = static_cast<float>(p->clamp_max);
+    ep.clamp_min_d = p->clamp_min;
+    ep.clamp_max_d = p->clamp_max;
+  } else if (dst->dtype == RUYAMD_DTYPE_I32) {
+    // ruy/mul_params.h:291-293: no clamping of raw accumulators.
+    ep.clamp_min_i = std::numeric_limits<int32_t>::lowest();
+    ep.clamp_max_i = std::numeric_limits<int32_t>::max();
+  } else {
+    ep.clamp_min_i = ClampToInt32(p->clamp_min);
+    ep.clamp_max_i = ClampToInt32(p->clamp_max);
+  }
+
+  std::string err;
+  const int rc = RunMul(ctx, &call, &err);
+  if (rc != RUYAMD_OK) return Fail(ctx, rc, err);
+
+  if (!dst_on_device) {
+    const std::size_t inner = dst->order == RUYAMD_ORDER_COL_MAJOR ? dst->rows : dst->cols;
+    const std::size_t outer = dst->order == RUYAMD_ORDER_COL_MAJOR ? dst->cols : dst->rows;
+    const std::size_t pitch = std::size_t(dst->stride) * dst_elt;
+    if (hipMemcpy2DAsync(dst->data, pitch, dst_d, pitch, inner * dst_elt, outer,
+                         hipMemcpyDeviceToHost, ctx->stream) != hipSuccess)
+      return Fail(ctx, RUYAMD_E_HIP, "copying the destination back to the host failed");
+    staged = true;
+  }
+  if (ctx->synchronous || staged) {
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess)
+      return Fail(ctx, RUYAMD_E_HIP, std::string("kernel execution failed: ") + hipGetErrorString(hipGetLastError()));
+    ctx->pending_async = false;
+  } else {
+    ctx->pending_async = true;
+  }
+  return RUYAMD_OK;
+}
+
+extern "C" int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x, const int32_t* m,
+                                       const int32_t* e, int32_t* out, int64_t n) {
+  if (!ctx || n < 0) return RUYAMD_E_INVALID;
+  if (n == 0) return RUYAMD_OK;
+  if (!x || !m || !e || !out) return Fail(ctx, RUYAMD_E_INVALID, "null argument");
+  if (hipSetDevice(ctx->device) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "hipSetDevice failed");
+  ctx->workspace.Reset();
+  bool staged = false, ok = true;
+  const std::size_t bytes = std::size_t(n) * 4;
+  const int32_t* xd = static_cast<const int32_t*>(StageIn(ctx, x, bytes, &staged, &ok));
+  const int32_t* md = static_cast<const int32_t*>(StageIn(ctx, m, bytes, &staged, &ok));
+  const int32_t* ed = static_cast<const int32_t*>(StageIn(ctx, e, bytes, &staged, &ok));
+  if (!ok) return Fail(ctx, RUYAMD_E_HIP, "staging failed");
+  const bool out_dev = IsDevicePointer(out);
+  int32_t* od = out_dev ? out : static_cast<int32_t*>(ctx->workspace.Alloc(bytes));
+  if (!od) return Fail(ctx, RUYAMD_E_HIP, "device allocation failed");
+  if (LaunchApplyMultiplier(ctx->stream, xd, md, ed, od, n) != hipSuccess)
+    return Fail(ctx, RUYAMD_E_HIP, "launch failed");
+  if (!out_dev && hipMemcpyAsync(out, od, bytes, hipMemcpyDeviceToHost, ctx->stream) != hipSuccess)
+    return Fail(ctx, RUYAMD_E_HIP, "copy back failed");
+  if (hipStreamSynchronize(ctx->stream) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "kernel execution failed");
+  return RUYAMD_OK;
+}

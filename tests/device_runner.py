@@ -1,0 +1,72 @@
+"""Runs a workloads.Problem through the C ABI (ruyamd_mul) on the GPU."""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from ruy_amd import _structs as S
+from ruy_amd import api
+
+_TORCH = {S.U8: torch.uint8, S.I8: torch.int8, S.I16: torch.int16, S.I32: torch.int32,
+          S.F32: torch.float32, S.F64: torch.float64}
+
+
+def to_dev(arr):
+    return torch.from_numpy(np.ascontiguousarray(arr)).cuda()
+
+
+class DeviceProblem:
+    """Device-resident copy of a Problem: tensors + the two descriptor structs."""
+
+    def __init__(self, problem, dst_fill=0x5A):
+        p = problem
+        self.problem = p
+        self.lhs_t = to_dev(p.lhs.storage)
+        self.rhs_t = to_dev(p.rhs.storage)
+        d = p.dst
+        fill = np.full(max(d.n_storage, 1), 0, dtype=d.storage.dtype)
+        fill.view(np.uint8)[:] = dst_fill
+        self.dst_t = to_dev(fill)
+        self.bias_t = to_dev(p.bias) if p.bias is not None else None
+        self.mf_t = self.me_t = None
+        if p.multiplier_fixedpoint_perchannel is not None:
+            self.mf_t = to_dev(p.multiplier_fixedpoint_perchannel)
+            self.me_t = to_dev(p.multiplier_exponent_perchannel)
+        self.lhs_s = p.lhs.struct(self.lhs_t.data_ptr())
+        self.rhs_s = p.rhs.struct(self.rhs_t.data_ptr())
+        self.dst_s = p.dst.struct(self.dst_t.data_ptr())
+        self.par_s = p.params_struct(
+            self.bias_t.data_ptr() if self.bias_t is not None else None,
+            self.mf_t.data_ptr() if self.mf_t is not None else None,
+            self.me_t.data_ptr() if self.me_t is not None else None)
+        torch.cuda.synchronize()
+
+    def run(self, ctx):
+        rc = api.lib.ruyamd_mul(ctx._h, C.byref(self.lhs_s), C.byref(self.rhs_s),
+                                C.byref(self.par_s), C.byref(self.dst_s))
+        ctx._check(rc)
+
+    def result(self):
+        torch.cuda.synchronize()
+        return self.dst_t.cpu().numpy()
+
+
+def device_mul(ctx, problem, dst_fill=0x5A):
+    """dst storage (numpy, same layout as problem.dst) computed on the GPU from
+    device-resident operands; untouched elements keep the fill byte."""
+    dp = DeviceProblem(problem, dst_fill)
+    dp.run(ctx)
+    return dp.result()
+
+
+def host_pointer_mul(ctx, problem, dst_fill=0x5A):
+    """Same call with host pointers for every buffer (the library stages them)."""
+    p = problem
+    d = p.dst
+    out = np.full(max(d.n_storage, 1), 0, dtype=d.storage.dtype)
+    out.view(np.uint8)[:] = dst_fill
+    l, r, ds = p.lhs.struct(), p.rhs.struct(), p.dst.struct(out.ctypes.data)
+    ps = p.params_struct()
+    rc = api.lib.ruyamd_mul(ctx._h, C.byref(l), C.byref(r), C.byref(ps), C.byref(ds))
+    ctx._check(rc)
+    return out

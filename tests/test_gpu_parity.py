@@ -1,0 +1,210 @@
+"""Parity of the device path (through the C ABI) against the CPU checker.
+
+Integer results must be bit-identical; fp32 results from the generic kernel are
+bit-identical too (it keeps the reference's ascending-k, unfused arithmetic),
+results from the MFMA kernels must be within 1e-5 relative Frobenius error.
+"""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+import cases
+import oracle_lib as O
+from ruy_amd import _structs as S
+from ruy_amd import workloads as W
+from test_oracle import (MBQM_KATS, SATURATION_CASES, example_problems, mbqm_random_cases,
+                         saturation_problem)
+
+pytestmark = pytest.mark.gpu
+
+REL_FROBENIUS_TOL = 1e-5
+
+
+def announce(*what):
+    print("[case]", *what, flush=True)
+    sys.stdout.flush()
+
+
+def compare(problem, got, want, exact_fp=False):
+    if problem.dst.dtype in (S.F32, S.F64) and not exact_fp:
+        g = O.dense_of(problem, got).astype(np.float64)
+        w = O.dense_of(problem, want).astype(np.float64)
+        denom = max(np.linalg.norm(w), 1e-30)
+        err = np.linalg.norm(g - w) / denom
+        assert err <= REL_FROBENIUS_TOL, (problem.name, err)
+        # and padding untouched
+        mask = np.ones(got.shape, bool)
+    else:
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "%s: %d mismatches, first at %d: got %r want %r" % (
+            problem.name, bad.size, bad[0], got[bad[0]], want[bad[0]])
+
+
+def run_both(ctx, problem, fill=0x5A):
+    import device_runner as D
+    want = O.oracle_mul(problem)
+    # give the checker's untouched elements the same fill pattern
+    filled = np.zeros_like(want)
+    filled.view(np.uint8)[:] = fill
+    d = problem.dst
+    if d.rows and d.cols:
+        it = want.itemsize
+        strides = (it, d.stride * it) if d.order == S.ORDER_COL_MAJOR else (d.stride * it, it)
+        np.lib.stride_tricks.as_strided(filled, (d.rows, d.cols), strides)[...] = \
+            np.lib.stride_tricks.as_strided(want, (d.rows, d.cols), strides)
+    got = D.device_mul(ctx, problem, fill)
+    return got, filled
+
+
+def test_requantizer_known_answers_on_device(device_ctx):
+    import torch
+    kats = MBQM_KATS + [(x, m, e, O.oracle.oracle_mbqm(x, m, e)) for x, m, e in mbqm_random_cases(4000, 23)]
+    x = torch.tensor([k[0] for k in kats], dtype=torch.int32).cuda()
+    m = torch.tensor([k[1] for k in kats], dtype=torch.int32).cuda()
+    e = torch.tensor([k[2] for k in kats], dtype=torch.int32).cuda()
+    out = torch.zeros_like(x)
+    torch.cuda.synchronize()
+    device_ctx.apply_multiplier(x, m, e, out, len(kats))
+    got = out.cpu().numpy()
+    want = np.array([k[3] for k in kats], np.int32)
+    assert (got == want).all()
+    # host pointers take the staged route
+    xh, mh, eh = (np.array([k[i] for k in kats], np.int32) for i in range(3))
+    oh = np.zeros(len(kats), np.int32)
+    device_ctx.apply_multiplier(xh, mh, eh, oh, len(kats))
+    assert (oh == want).all()
+
+
+@pytest.mark.parametrize("dst_dtype,cols,zp", SATURATION_CASES)
+def test_saturation_known_answers_on_device(device_ctx, dst_dtype, cols, zp):
+    import device_runner as D
+    p, want = saturation_problem(dst_dtype, cols, zp)
+    got = D.device_mul(device_ctx, p)
+    assert (got[:cols] == want).all()
+
+
+def test_example_cases_on_device(device_ctx):
+    import device_runner as D
+    for p, want in example_problems():
+        announce("example", p.name)
+        got = O.dense_of(p, D.device_mul(device_ctx, p))
+        assert (got == np.array(want)).all(), (p.name, got)
+        got = O.dense_of(p, D.host_pointer_mul(device_ctx, p))
+        assert (got == np.array(want)).all(), (p.name, "host pointers", got)
+
+
+def sweep_shapes():
+    return ([(s, s, s) for s in cases.SQUARE_SIZES] + cases.MISC_SHAPES + cases.DEEP_SHAPES +
+            cases.SHALLOW_SHAPES + cases.NARROW_SHAPES + cases.GEMV_SHAPES[::5] +
+            [(5, 5001, 1), (8193, 17, 1)])
+
+
+@pytest.mark.parametrize("tup", cases.TYPE_TUPLES, ids=cases.tuple_name)
+@pytest.mark.parametrize("force_generic", [True, False], ids=["generic", "tuned"])
+def test_reference_shape_sweep(device_ctx, tup, force_generic):
+    """The reference's test_fast shape list (ruy/test_fast.cc:31-107), each with
+    a random storage-order combination, padded strides half of the time, and
+    TestSet-style random parameters (ruy/test.h:1718-1783)."""
+    rng = np.random.default_rng(4242 + cases.TYPE_TUPLES.index(tup))
+    device_ctx.force_generic_kernel(force_generic)
+    try:
+        for shape in sweep_shapes():
+            orders = cases.ALL_ORDERS[int(rng.integers(8))]
+            strided = bool(rng.integers(2))
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=strided,
+                                 name="%s %s %s strided=%s" % (cases.tuple_name(tup), shape, orders, strided))
+            announce(p.name, "generic" if force_generic else "tuned")
+            got, want = run_both(device_ctx, p)
+            # The generic kernel keeps the reference's fp evaluation order.
+            compare(p, got, want, exact_fp=force_generic)
+    finally:
+        device_ctx.force_generic_kernel(False)
+
+
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.U8),
+                                 (S.F32, S.F32, S.F32, S.F32), (S.I8, S.I16, S.I32, S.I16),
+                                 (S.I8, S.I8, S.I32, S.I32)], ids=cases.tuple_name)
+def test_all_orders_with_padded_strides(device_ctx, tup):
+    """TestLinearAllOrders (ruy/test.h:2306-2325): all 8 order combinations with
+    stride = minimum + 1, on shapes that cross the tile sizes of the kernels."""
+    rng = np.random.default_rng(99)
+    for shape in [(65, 130, 33), (256, 192, 128), (40, 4096, 50), (17, 65, 300)]:
+        for orders in cases.ALL_ORDERS:
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=True,
+                                 name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
+
+
+def test_host_pointer_operands(device_ctx):
+    """Host pointers for every buffer (what a drop-in caller of the reference
+    passes): staged by the library, padding of a strided dst left alone."""
+    import device_runner as D
+    rng = np.random.default_rng(5)
+    for tup in [(S.I8, S.I8, S.I32, S.I8), (S.F32, S.F32, S.F32, S.F32), (S.U8, S.U8, S.I32, S.I16)]:
+        p = W.random_problem(rng, *tup, 37, 91, 23, 1, 0, 0, strided=True)
+        want = O.oracle_mul(p, fill=0)
+        got = D.host_pointer_mul(device_ctx, p, dst_fill=0)
+        compare(p, got, want, exact_fp=False)
+        got = D.host_pointer_mul(device_ctx, p, dst_fill=0x77)
+        d = p.dst
+        gaps = [c * d.stride + d.rows for c in range(d.cols - 1)]
+        assert all(got.view(np.uint8).reshape(got.size, -1)[g, 0] == 0x77 for g in gaps)
+
+
+def test_empty_and_degenerate_shapes(device_ctx):
+    import device_runner as D
+    rng = np.random.default_rng(6)
+    for shape in [(0, 5, 3), (4, 5, 0), (4, 0, 3), (1, 1, 1)]:
+        p = W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, *shape, 1, 0, 0)
+        got, want = run_both(device_ctx, p)
+        compare(p, got, want)
+
+
+def test_rejects_what_the_reference_forbids(device_ctx):
+    import device_runner as D
+    from ruy_amd import api
+    p = W.config_int8_gemm(8)
+    p.lhs.zero_point, p.rhs.zero_point = -128, -128
+    with pytest.raises(api.RuyAmdError):
+        D.device_mul(device_ctx, p)
+    p = W.config_int8_int16(8, 8, 8)
+    p.dst.zero_point = 3
+    with pytest.raises(api.RuyAmdError):
+        D.device_mul(device_ctx, p)
+    p = W.config_int8_gemm(8)
+    device_ctx.set_runtime_enabled_paths(api.Path.kStandardCpp)
+    try:
+        with pytest.raises(api.RuyAmdError) as ei:
+            D.device_mul(device_ctx, p)
+        assert ei.value.code == 4
+    finally:
+        device_ctx.set_runtime_enabled_paths(api.Path.kNone)
+    D.device_mul(device_ctx, p)
+    assert device_ctx.last_used_path() == api.Path.kGfx950
+
+
+CONFIG_CASES = [
+    ("C1 int8 256^3", lambda: W.config_int8_gemm(256)),
+    ("C2 fp32 1024^3", lambda: W.config_f32_gemm(1024)),
+    ("C2 fp32 1024^3 relu6", lambda: W.config_f32_gemm(1024, relu6=True)),
+    ("C3 int8 per-channel 1024x1024x196", lambda: W.config_int8_perchannel_conv()),
+    ("C4 int8xint16 2048x2048x512", lambda: W.config_int8_int16()),
+    ("C5 gemv 4096 n1 i32", lambda: W.config_int8_gemv(4096, 1)),
+    ("C5 gemv 4096 n4 i32", lambda: W.config_int8_gemv(4096, 4)),
+    ("C5 gemv 4096 n8 i32", lambda: W.config_int8_gemv(4096, 8)),
+    ("C5 gemv 4096 n1 i8", lambda: W.config_int8_gemv(4096, 1, requant=True)),
+    ("T int8 1024^3", lambda: W.config_int8_gemm(1024, config_id=6)),
+]
+
+
+@pytest.mark.parametrize("name,make", CONFIG_CASES, ids=[c[0] for c in CONFIG_CASES])
+def test_benchmark_configurations(device_ctx, name, make):
+    p = make()
+    announce(name)
+    got, want = run_both(device_ctx, p)
+    compare(p, got, want)
+    announce(name, "kernel:", device_ctx.last_kernel_name())
