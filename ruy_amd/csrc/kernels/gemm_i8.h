@@ -1,0 +1,64 @@
+// Launch interfaces of the int8 kernels and of the pack / sums kernels.
+#ifndef RUY_AMD_CSRC_KERNELS_GEMM_I8_H_
+#define RUY_AMD_CSRC_KERNELS_GEMM_I8_H_
+
+#include <hip/hip_runtime.h>
+
+#include "../internal.h"
+
+namespace ruyamd {
+
+// Operands of the int8 kernels are depth-contiguous int8: row i of `a` (an LHS
+// row) is the K bytes at a + i*lda, column j of `b` (an RHS column) the K bytes
+// at b + j*ldb. Both base pointers and leading dimensions are multiples of 16
+// and K is a multiple of 16; `a_bytes` / `b_bytes` (< 2^31) bound the buffer
+// descriptors, so rows at or past M / N read as zero.
+struct GemmI8Args {
+  const int8_t* a = nullptr;
+  const int8_t* b = nullptr;
+  uint32_t a_bytes = 0;
+  uint32_t b_bytes = 0;
+  int32_t lda = 0;
+  int32_t ldb = 0;
+  int32_t M = 0;
+  int32_t N = 0;
+  int32_t K = 0;
+  Epilogue ep;
+  // The destination must be column-major (dst.rs == 1): callers swap the
+  // operands for a row-major one. dst_elt is its element size; dst_vector_ok
+  // says that base and column pitch are 16-byte aligned so that 16-byte stores
+  // may be used.
+  DevMat dst;
+  int32_t dst_elt = 1;
+  int32_t dst_vector_ok = 0;
+};
+
+hipError_t LaunchGemmI8(hipStream_t stream, const GemmI8Args& args, int num_cus);
+
+// A matrix seen as `count` depth-vectors of length K: vector c, depth k is
+// data[c * stride_c + k * stride_k] (elements of `dtype`, uint8 or int8).
+struct PackSource {
+  const void* data = nullptr;
+  int64_t stride_c = 0;
+  int64_t stride_k = 0;
+  int32_t count = 0;
+  int32_t K = 0;
+  int32_t dtype = 0;
+};
+
+// The device form of the reference's Pack (ruy/pack.h:105-132 with the
+// uint8 -> int8 conversion of ruy/pack_common.h:36-58): writes vector c as int8
+// at dst + c*ld (depth-contiguous, zero-filled from K up to ld) and, when
+// `sums` is non-null, sums[c] = sum over the K real depth positions of the
+// packed values.
+hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld,
+                        int32_t* sums);
+
+// sums[c] = sum_k data[c*ld + k] for depth-contiguous int8 data with 16-byte
+// aligned base and ld, K a multiple of 16.
+hipError_t LaunchSumsI8(hipStream_t stream, const int8_t* data, int32_t ld, int32_t count,
+                        int32_t K, int32_t* sums);
+
+}  // namespace ruyamd
+
+#endif  // RUY_AMD_CSRC_KERNELS_GEMM_I8_H_

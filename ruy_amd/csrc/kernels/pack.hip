@@ -1,0 +1,170 @@
+// Pack and sums kernels: the device counterpart of the reference's packing
+// stage (generic ruy/pack.h:105-132; AVX-512 ruy/pack_avx512.cc:840-1098).
+// Packing re-lays an operand out as depth-contiguous int8 vectors (the operand
+// order of the int8 matrix instructions), converts uint8 to int8 by flipping
+// the top bit (ruy/pack_common.h:36-58), zero-fills the depth padding, and
+// produces the per-vector int32 sums that the zero-point correction needs.
+// Operands that already have that layout are used in place and only summed.
+#include <hip/hip_runtime.h>
+
+#include "../internal.h"
+#include "gemm_i8.h"
+
+namespace ruyamd {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kTileC = 64;  // vectors per block
+constexpr int kTileK = 64;  // depth bytes per step
+constexpr int kPitch = kTileK + 4;  // LDS row pitch in bytes (breaks bank alignment)
+
+__device__ __forceinline__ int WaveSum(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+__global__ void ZeroI32Kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// Block = 256 threads = one 64-vector x (k_span) slab, walked 64 depth bytes at
+// a time through LDS so that both the read (along the source's contiguous
+// dimension) and the write (along depth) are coalesced.
+__global__ __launch_bounds__(256) void PackI8Kernel(PackSource src, int8_t* dst, int32_t ld,
+                                                   int32_t* sums, int k_span) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kPitch];
+  const int tid = threadIdx.x;
+  const int c0 = blockIdx.x * kTileC;
+  const int k_begin = blockIdx.y * k_span;
+  const int k_end = min(k_begin + k_span, ld);  // includes the zero-filled padding
+  const uint8_t* s = static_cast<const uint8_t*>(src.data);
+  const uint32_t flip = src.dtype == RUYAMD_DTYPE_U8 ? 0x80808080u : 0u;
+  const bool depth_contiguous = src.stride_k == 1;
+  // writer role: vector wc, 16-byte granule wg of the 64-byte step
+  const int wc = tid >> 2;
+  const int wg = tid & 3;
+  int32_t sum = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += kTileK) {
+    if (depth_contiguous) {
+      const int tx = tid & 63;  // depth
+      const int k = k0 + tx;
+#pragma unroll 4
+      for (int cc = tid >> 6; cc < kTileC; cc += 4) {
+        const int c = c0 + cc;
+        uint8_t v = 0;
+        if (c < src.count && k < src.K) v = s[c * src.stride_c + k];
+        tile[cc * kPitch + tx] = v;
+      }
+    } else {
+      const int tx = tid & 63;  // vector
+      const int c = c0 + tx;
+#pragma unroll 4
+      for (int kk = tid >> 6; kk < kTileK; kk += 4) {
+        const int k = k0 + kk;
+        uint8_t v = 0;
+        if (c < src.count && k < src.K) v = s[c * src.stride_c + k * src.stride_k];
+        tile[tx * kPitch + kk] = v;
+      }
+    }
+    __syncthreads();
+    const int c = c0 + wc;
+    const int k = k0 + wg * 16;
+    if (c < src.count && k < ld) {
+      const uint32_t* row = reinterpret_cast<const uint32_t*>(tile + wc * kPitch + wg * 16);
+      v4i out;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        // Padding bytes were stored as 0 and must stay 0: flip only real ones.
+        uint32_t w = row[d];
+        const int kd = k + 4 * d;
+        if (flip) {
+          uint32_t mask = kd + 4 <= src.K ? 0xffffffffu
+                          : kd >= src.K  ? 0u
+                                         : (0xffffffffu >> (8 * (kd + 4 - src.K)));
+          w ^= flip & mask;
+        }
+        out[d] = static_cast<int>(w);
+        sum = __builtin_amdgcn_sdot4(static_cast<int>(w), 0x01010101, sum, false);
+      }
+      *reinterpret_cast<v4i*>(dst + int64_t(c) * ld + k) = out;
+    }
+    __syncthreads();
+  }
+  if (sums) {
+    // the 4 granule-writers of a vector are adjacent lanes
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    const int c = c0 + wc;
+    if (wg == 0 && c < src.count) {
+      if (gridDim.y == 1)
+        sums[c] = sum;
+      else
+        atomicAdd(&sums[c], sum);
+    }
+  }
+}
+
+// One wave per vector, 16 bytes per lane per step.
+__global__ __launch_bounds__(256) void SumsI8Kernel(const int8_t* data, int32_t ld, int32_t count,
+                                                   int32_t K, int32_t* sums) {
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (c >= count) return;
+  const int8_t* row = data + int64_t(c) * ld;
+  int32_t s0 = 0, s1 = 0;
+  int k = lane * 16;
+  for (; k + 1024 < K; k += 2048) {
+    const v4i x = *reinterpret_cast<const v4i*>(row + k);
+    const v4i y = *reinterpret_cast<const v4i*>(row + k + 1024);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      s0 = __builtin_amdgcn_sdot4(x[d], 0x01010101, s0, false);
+      s1 = __builtin_amdgcn_sdot4(y[d], 0x01010101, s1, false);
+    }
+  }
+  for (; k < K; k += 1024) {
+    const v4i x = *reinterpret_cast<const v4i*>(row + k);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) s0 = __builtin_amdgcn_sdot4(x[d], 0x01010101, s0, false);
+  }
+  const int32_t total = WaveSum(s0 + s1);
+  if (lane == 0) sums[c] = total;
+}
+
+}  // namespace
+
+hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld,
+                        int32_t* sums) {
+  if (src.count == 0 || ld == 0) return hipSuccess;
+  const int blocks_c = (src.count + kTileC - 1) / kTileC;
+  // Split the depth when there are too few vector slabs to fill the device.
+  int k_split = 1;
+  const int k_steps = (ld + kTileK - 1) / kTileK;
+  if (blocks_c < 512 && k_steps > 8) {
+    k_split = min((512 + blocks_c - 1) / blocks_c, k_steps / 8);
+    if (k_split < 1) k_split = 1;
+  }
+  const int steps_per = (k_steps + k_split - 1) / k_split;
+  const int k_span = steps_per * kTileK;
+  k_split = (k_steps + steps_per - 1) / steps_per;
+  if (sums && k_split > 1) {
+    hipLaunchKernelGGL(ZeroI32Kernel, dim3((src.count + 255) / 256), dim3(256), 0, stream, sums,
+                       src.count);
+  }
+  hipLaunchKernelGGL(PackI8Kernel, dim3(blocks_c, k_split), dim3(256), 0, stream, src, dst, ld, sums,
+                     k_span);
+  return hipGetLastError();
+}
+
+hipError_t LaunchSumsI8(hipStream_t stream, const int8_t* data, int32_t ld, int32_t count, int32_t K,
+                        int32_t* sums) {
+  if (count == 0) return hipSuccess;
+  hipLaunchKernelGGL(SumsI8Kernel, dim3((count + 3) / 4), dim3(256), 0, stream, data, ld, count, K,
+                     sums);
+  return hipGetLastError();
+}
+
+}  // namespace ruyamd

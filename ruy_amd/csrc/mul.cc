@@ -172,8 +172,8 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
 
   bool staged = false, ok = true;
   const int channels = p->channel_dimension == RUYAMD_CHANNEL_ROW ? dst->rows : dst->cols;
-  const void* lhs_d = StageIn(ctx, lhs->data, StorageElements(*lhs) * DtypeSize(lhs->dtype), &staged, &ok);
-  const void* rhs_d = StageIn(ctx, rhs->data, StorageElements(*rhs) * DtypeSize(rhs->dtype), &staged, &ok);
+  // The two source matrices are staged lazily by the dispatcher (a cache hit
+  // needs no copy); the small per-channel vectors are staged now.
   const void* bias_d = StageIn(ctx, p->bias, std::size_t(channels) * DtypeSize(p->accum_dtype), &staged, &ok);
   const void* mf_d = StageIn(ctx, p->multiplier_fixedpoint_perchannel, std::size_t(channels) * 4, &staged, &ok);
   const void* me_d = StageIn(ctx, p->multiplier_exponent_perchannel, std::size_t(channels) * 4, &staged, &ok);
@@ -191,8 +191,12 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
   }
 
   MulCall call;
-  call.lhs = ToDevMat(*lhs, lhs_d);
-  call.rhs = ToDevMat(*rhs, rhs_d);
+  call.lhs = ToDevMat(*lhs, lhs->data);
+  call.rhs = ToDevMat(*rhs, rhs->data);
+  if (lhs->data && !IsDevicePointer(lhs->data))
+    call.lhs_host_bytes = StorageElements(*lhs) * DtypeSize(lhs->dtype);
+  if (rhs->data && !IsDevicePointer(rhs->data))
+    call.rhs_host_bytes = StorageElements(*rhs) * DtypeSize(rhs->dtype);
   call.dst = ToDevMat(*dst, dst_d);
   call.lhs_src_key = lhs->data;
   call.rhs_src_key = rhs->data;
@@ -226,6 +230,7 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
   std::string err;
   const int rc = RunMul(ctx, &call, &err);
   if (rc != RUYAMD_OK) return Fail(ctx, rc, err);
+  staged = staged || call.staged_any;
 
   if (!dst_on_device) {
     const std::size_t inner = dst->order == RUYAMD_ORDER_COL_MAJOR ? dst->rows : dst->cols;

@@ -1,8 +1,238 @@
 #include "plan.h"
 
+#include <cstdint>
+
+#include "kernels/gemm_i8.h"
+
 namespace ruyamd {
+namespace {
+
+// The skinny-kernel limit; it also plays the role of the "kernel width" in the
+// cache-policy heuristics (ruy/prepare_packed_matrices.cc:38-66), so that
+// kCacheIfLargeSpeedup means "the other side is narrow enough for the
+// bandwidth-bound kernel".
+constexpr int kSkinnyWidth = 8;
+
+bool Is8Bit(int dtype) { return dtype == RUYAMD_DTYPE_U8 || dtype == RUYAMD_DTYPE_I8; }
+
+int32_t RoundUp(int32_t x, int32_t m) { return (x + m - 1) / m * m; }
+
+// ruy/prepare_packed_matrices.cc:38-66
+bool ShouldCache(int cache_policy, int other_width) {
+  switch (cache_policy) {
+    case RUYAMD_CACHE_ALWAYS:
+      return true;
+    case RUYAMD_CACHE_IF_LARGE_SPEEDUP:
+      return other_width <= kSkinnyWidth;
+    case RUYAMD_CACHE_IF_SIGNIFICANT_SPEEDUP:
+      return other_width <= 4 * kSkinnyWidth;
+    default:
+      return false;
+  }
+}
+
+// One side of an 8-bit multiplication, ready for the int8 kernels.
+struct Operand8 {
+  const int8_t* data = nullptr;
+  int32_t ld = 0;
+  const int32_t* sums = nullptr;
+  int32_t zero_point = 0;  // of the int8 form (uint8 zero point minus 128)
+  uint32_t bytes = 0;
+};
+
+// Prepares one side: from the cache, in place, or packed into the workspace.
+// `src` views the side as `count` depth vectors (LHS rows / RHS columns).
+int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point, bool need_sums,
+                    int cache_policy, const void* src_key, int other_width, Operand8* out,
+                    std::string* err) {
+  // View of the side as `count` depth vectors; its data pointer is only valid
+  // on the device after EnsureOnDevice.
+  auto view = [&]() {
+    const DevMat& m = side == 0 ? call->lhs : call->rhs;
+    return side == 0 ? PackSource{m.data, m.rs, m.cs, m.rows, m.cols, m.dtype}
+                     : PackSource{m.data, m.cs, m.rs, m.cols, m.rows, m.dtype};
+  };
+  PackSource src = view();
+  const int32_t K = src.K;
+  const int32_t ld = RoundUp(K > 0 ? K : 1, 16);
+  const bool is_u8 = src.dtype == RUYAMD_DTYPE_U8;
+  out->zero_point = is_u8 ? zero_point - 128 : zero_point;
+  const uint64_t packed_bytes = uint64_t(src.count) * ld;
+  if (packed_bytes >= (uint64_t(1) << 31)) {
+    *err = "operand larger than 2 GiB is not supported by the int8 kernels";
+    return RUYAMD_E_UNSUPPORTED;
+  }
+
+  if (ShouldCache(cache_policy, other_width)) {
+    PackedMatrix pm;
+    pm.element_size = 1;
+    pm.is_floating_point = false;
+    pm.layout.rows = ld;
+    pm.layout.cols = src.count;
+    pm.layout.stride = ld;
+    pm.layout.order = 0;
+    pm.layout.kernel_order = 0;
+    pm.layout.kernel_rows = 16;
+    pm.layout.kernel_cols = 1;
+    pm.zero_point = out->zero_point;
+    const auto action = ctx->cache->Get(src_key, &pm);
+    if (!pm.data) {
+      *err = "device allocation for a cached packed matrix failed";
+      return RUYAMD_E_HIP;
+    }
+    if (action == PrepackedCache::Action::kInsertedNewEntry) {
+      if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
+      src = view();
+      if (LaunchPackI8(ctx->stream, src, static_cast<int8_t*>(pm.data), ld, pm.sums) != hipSuccess) {
+        *err = "pack kernel launch failed";
+        return RUYAMD_E_HIP;
+      }
+    }
+    out->data = static_cast<const int8_t*>(pm.data);
+    out->ld = ld;
+    out->sums = pm.sums;
+    out->bytes = static_cast<uint32_t>(packed_bytes);
+    return RUYAMD_OK;
+  }
+
+  if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
+  src = view();
+  // In place: already int8, depth-contiguous, 16-byte aligned base and pitch,
+  // depth a multiple of 16, and small enough for a buffer descriptor.
+  const uint64_t extent = src.count > 0 ? uint64_t(src.count - 1) * uint64_t(src.stride_c) + K : 0;
+  const bool direct = !is_u8 && src.stride_k == 1 && K % 16 == 0 && K > 0 &&
+                      (reinterpret_cast<uintptr_t>(src.data) & 15) == 0 &&
+                      (src.stride_c % 16 == 0 || src.count == 1) && extent < (uint64_t(1) << 31);
+  if (direct) {
+    out->data = static_cast<const int8_t*>(src.data);
+    out->ld = src.count == 1 ? ld : static_cast<int32_t>(src.stride_c);
+    out->bytes = static_cast<uint32_t>(extent);
+    if (need_sums) {
+      int32_t* sums = static_cast<int32_t*>(ctx->workspace.Alloc(std::size_t(src.count) * 4));
+      if (!sums) {
+        *err = "workspace allocation failed";
+        return RUYAMD_E_HIP;
+      }
+      if (LaunchSumsI8(ctx->stream, out->data, out->ld, src.count, K, sums) != hipSuccess) {
+        *err = "sums kernel launch failed";
+        return RUYAMD_E_HIP;
+      }
+      out->sums = sums;
+    }
+    return RUYAMD_OK;
+  }
+
+  int8_t* packed = static_cast<int8_t*>(ctx->workspace.Alloc(packed_bytes ? packed_bytes : 16));
+  int32_t* sums = need_sums ? static_cast<int32_t*>(ctx->workspace.Alloc(std::size_t(src.count) * 4)) : nullptr;
+  if (!packed || (need_sums && !sums)) {
+    *err = "workspace allocation failed";
+    return RUYAMD_E_HIP;
+  }
+  if (LaunchPackI8(ctx->stream, src, packed, ld, sums) != hipSuccess) {
+    *err = "pack kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  out->data = packed;
+  out->ld = ld;
+  out->sums = sums;
+  out->bytes = static_cast<uint32_t>(packed_bytes);
+  return RUYAMD_OK;
+}
+
+int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
+  const DevMat& lhs = call->lhs;
+  const DevMat& rhs = call->rhs;
+  const int M = lhs.rows, K = lhs.cols, N = rhs.cols;
+  const int32_t lzp = lhs.dtype == RUYAMD_DTYPE_U8 ? lhs.zero_point - 128 : lhs.zero_point;
+  const int32_t rzp = rhs.dtype == RUYAMD_DTYPE_U8 ? rhs.zero_point - 128 : rhs.zero_point;
+  Operand8 a, b;
+  // Row sums of one side are needed iff the other side's zero point is not 0
+  // (ruy/kernel.h:219-232).
+  if (int rc = PrepareOperand8(ctx, call, 0, lhs.zero_point, rzp != 0, call->lhs_cache_policy,
+                               call->lhs_src_key, N, &a, err))
+    return rc;
+  if (int rc = PrepareOperand8(ctx, call, 1, rhs.zero_point, lzp != 0, call->rhs_cache_policy,
+                               call->rhs_src_key, M, &b, err))
+    return rc;
+  GemmI8Args args;
+  args.K = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
+  args.ep = call->ep;
+  args.ep.zp_product_depth =
+      static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
+  const DevMat& dst = call->dst;
+  if (dst.rs == 1) {
+    args.a = a.data;
+    args.b = b.data;
+    args.a_bytes = a.bytes;
+    args.b_bytes = b.bytes;
+    args.lda = a.ld;
+    args.ldb = b.ld;
+    args.M = M;
+    args.N = N;
+    args.ep.lhs_sums = a.sums;
+    args.ep.rhs_sums = b.sums;
+    args.ep.lhs_zero_point = lzp;
+    args.ep.rhs_zero_point = rzp;
+    args.dst = dst;
+  } else {
+    // Row-major destination: compute dst^T = rhs^T * lhs^T, which is
+    // column-major in the same memory, with the channel dimension flipped
+    // (ruy/create_trmul_params.h:471-479).
+    args.a = b.data;
+    args.b = a.data;
+    args.a_bytes = b.bytes;
+    args.b_bytes = a.bytes;
+    args.lda = b.ld;
+    args.ldb = a.ld;
+    args.M = N;
+    args.N = M;
+    args.ep.lhs_sums = b.sums;
+    args.ep.rhs_sums = a.sums;
+    args.ep.lhs_zero_point = rzp;
+    args.ep.rhs_zero_point = lzp;
+    args.ep.channel_is_col = !call->ep.channel_is_col;
+    args.dst = dst;
+    args.dst.rows = dst.cols;
+    args.dst.cols = dst.rows;
+    args.dst.rs = 1;
+    args.dst.cs = dst.rs;
+  }
+  args.dst_elt = DtypeSize(dst.dtype);
+  args.dst_vector_ok = (reinterpret_cast<uintptr_t>(args.dst.data) & 15) == 0 &&
+                       (args.dst.cs * args.dst_elt) % 16 == 0;
+  if (LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count) != hipSuccess) {
+    *err = "int8 MFMA kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  ctx->last_kernel = RUYAMD_KERNEL_I8_MFMA;
+  return RUYAMD_OK;
+}
+
+}  // namespace
+
+int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
+  DevMat& m = side == 0 ? call->lhs : call->rhs;
+  std::size_t& bytes = side == 0 ? call->lhs_host_bytes : call->rhs_host_bytes;
+  if (bytes == 0) return RUYAMD_OK;
+  void* d = ctx->workspace.Alloc(bytes);
+  if (!d || hipMemcpyAsync(d, m.data, bytes, hipMemcpyHostToDevice, ctx->stream) != hipSuccess) {
+    *err = "staging a host operand to the device failed";
+    return RUYAMD_E_HIP;
+  }
+  m.data = d;
+  bytes = 0;
+  call->staged_any = true;
+  return RUYAMD_OK;
+}
 
 int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
+  const DevMat& lhs = call->lhs;
+  const DevMat& rhs = call->rhs;
+  if (!ctx->force_generic) {
+    if (Is8Bit(lhs.dtype) && Is8Bit(rhs.dtype)) return RunInt8(ctx, call, err);
+  }
+  if (int rc = EnsureOnDevice(ctx, call, 0, err)) return rc;
+  if (int rc = EnsureOnDevice(ctx, call, 1, err)) return rc;
   if (LaunchGeneric(ctx->stream, call->lhs, call->rhs, call->ep, call->dst, call->accum_dtype) != hipSuccess) {
     *err = "generic kernel launch failed";
     return RUYAMD_E_HIP;

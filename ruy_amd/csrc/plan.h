@@ -19,7 +19,17 @@ struct MulCall {
   int lhs_cache_policy = 0;
   int rhs_cache_policy = 0;
   int accum_dtype = 0;
+  // Source operands given as host pointers are copied to the device only when
+  // a kernel is about to read them, so a prepacked-cache hit costs no transfer.
+  // While *_host_bytes is non-zero, lhs.data / rhs.data is still the host
+  // pointer; EnsureOnDevice replaces it with a device copy.
+  std::size_t lhs_host_bytes = 0;
+  std::size_t rhs_host_bytes = 0;
+  bool staged_any = false;
 };
+
+// Makes call->lhs (side 0) or call->rhs (side 1) device-resident.
+int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err);
 
 // Chooses a kernel, prepares packed operands and sums as needed (through the
 // context's cache when the cache policy says so), and enqueues the launch on
