@@ -10,13 +10,17 @@
 // operand order of v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive
 // depth bytes of row/column l%32, at depth offset 16*(l/32).
 //
-// Work decomposition: one workgroup per BM x BN destination tile, waves in a
-// WAVES_M x WAVES_N grid, each wave owning WM x WN blocks of 32x32. The depth
-// is walked in steps of 64 bytes through a double-buffered LDS stage; global
-// reads are 16-byte buffer loads (rows past the end of the matrix read as
-// zero through the buffer descriptor's bounds check), LDS rows are 64 bytes
-// with the four 16-byte granules XOR-swizzled by (row/4)%4 so that the
-// 16-lane groups of a ds_read_b128 touch all 64 banks.
+// Work decomposition: one workgroup (4 waves, 2 x 2) per BM x BN destination
+// tile, each wave owning WM x WN blocks of 32x32. The depth is walked in steps
+// of BK = 128 bytes (one full 128-byte cache line per row, so every line is
+// fetched from L2 exactly once) through a ring of LDS stages that is filled by
+// buffer_load_dwordx4 ... lds (global memory straight into LDS, no registers),
+// a whole step or more ahead of the matrix instructions. Rows past the end of
+// a matrix and depth granules past K read as zero through the buffer
+// descriptor's bounds check. The 16-byte granules of an LDS row are
+// XOR-swizzled by the row number so that a ds_read_b128 of 16 consecutive rows
+// touches all 64 banks; since a direct-to-LDS load places lane l at
+// base + 16*l, the swizzle is applied to the global address each lane fetches.
 #include <hip/hip_runtime.h>
 
 #include "../epilogue.h"
@@ -29,35 +33,85 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kBK = 64;                 // depth bytes per LDS stage
 constexpr int kGranule = 16;            // bytes per lane per load
-constexpr int kGranulesPerRow = kBK / kGranule;
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records we accept
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t MakeRsrc(const void* p, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+// Buffer descriptor words for a raw (stride 0) buffer of `bytes` bytes.
+__device__ __forceinline__ v4i MakeRsrc(const void* p, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  v4i r;
+  r[0] = __builtin_amdgcn_readfirstlane(static_cast<int>(a & 0xffffffffu));
+  r[1] = __builtin_amdgcn_readfirstlane(static_cast<int>((a >> 32) & 0xffffu));
+  r[2] = __builtin_amdgcn_readfirstlane(static_cast<int>(bytes));
+  r[3] = 0x00020000;
+  return r;
 }
 
-// Byte offset inside one LDS stage of granule g of tile row r.
+// 16 bytes per lane from buffer offset `voffset` straight into LDS at
+// lds_base + 16*lane (lds_base wave-uniform). Tracked by vmcnt. The compiler
+// does not know this instruction writes LDS, which is the point: it would
+// otherwise drain vmcnt to zero before every LDS read. M0 is not used by
+// anything else in these kernels.
+__device__ __forceinline__ void LoadToLds16(uint32_t lds_base, uint32_t voffset, v4i rsrc) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, 0 offen lds"
+      :
+      : "s"(lds_base), "v"(voffset), "s"(rsrc)
+      : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void WaitVmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// Swizzle term of tile row r: the granule stored in slot s of the row is
+// s ^ Swizzle(r). Chosen so that 16 consecutive rows at one granule index map
+// to 16 different 16-byte bank groups (256 bytes = all 64 banks).
+template <int BK>
+__device__ __forceinline__ int Swizzle(int r) {
+  static_assert(BK == 64 || BK == 128, "");
+  return BK == 64 ? ((r >> 2) & 3) : ((r >> 1) & 7);
+}
+
+// Byte offset inside one operand tile of granule g of tile row r.
+template <int BK>
 __device__ __forceinline__ int LdsOffset(int r, int g) {
-  return r * kBK + ((g ^ ((r >> 2) & 3)) << 4);
+  return r * BK + ((g ^ Swizzle<BK>(r)) << 4);
 }
 
-template <int WAVES_M, int WAVES_N, int WM, int WN>
+template <int WM, int WN, int BK, int STAGES>
 struct Cfg {
-  static constexpr int kBM = WAVES_M * WM * 32;
-  static constexpr int kBN = WAVES_N * WN * 32;
-  static constexpr int kThreads = 64 * WAVES_M * WAVES_N;
-  static constexpr int kAGranules = kBM * kGranulesPerRow / kThreads;  // per thread per stage
-  static constexpr int kBGranules = kBN * kGranulesPerRow / kThreads;
-  static constexpr int kStageBytes = (kBM + kBN) * kBK;
-  static_assert(kBM * kGranulesPerRow % kThreads == 0, "");
-  static_assert(kBN * kGranulesPerRow % kThreads == 0, "");
+  static constexpr int kBM = 2 * WM * 32;
+  static constexpr int kBN = 2 * WN * 32;
+  static constexpr int kBK = BK;
+  static constexpr int kThreads = 256;
+  static constexpr int kStages = STAGES;
+  static constexpr int kKSteps = BK / 32;           // matrix-instruction depth steps per stage
+  static constexpr int kGranulesPerRow = BK / kGranule;
+  static constexpr int kRowsPerLoad = 64 / kGranulesPerRow;  // tile rows one wave-level load covers
+  static constexpr int kALoads = kBM / kRowsPerLoad / 4;     // per wave per stage
+  static constexpr int kBLoads = kBN / kRowsPerLoad / 4;
+  static constexpr int kLoadsPerStage = kALoads + kBLoads;
+  static constexpr int kStageBytes = (kBM + kBN) * BK;
+  static constexpr int kEpilogueBytes = 4 * 32 * (WM * 32 + 4) * 4;
+  static constexpr int kLdsBytes =
+      kStages * kStageBytes > kEpilogueBytes ? kStages * kStageBytes : kEpilogueBytes;
 };
 
-template <int WAVES_M, int WAVES_N, int WM, int WN>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Args args) {
-  using C = Cfg<WAVES_M, WAVES_N, WM, WN>;
+// (hi(x*m) + 2^(s-1)) >> s with s = (31 - e) - 32 >= 1: MultiplyByQuantizedMultiplier
+// when the total shift is at least 33, where the low product word cannot
+// influence the floor.
+__device__ __forceinline__ int32_t RequantHigh(int32_t x, int32_t m, int s) {
+  return (__mulhi(x, m) + (1 << (s - 1))) >> s;
+}
+
+template <int WM, int WN, int BK, int STAGES>
+__global__ __launch_bounds__(256) void GemmI8Kernel(GemmI8Args args) {
+  using C = Cfg<WM, WN, BK, STAGES>;
+  constexpr int kBK = BK;
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
   // ---- which tile: XCD-aware, grouped ordering ----
@@ -82,46 +136,85 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Arg
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wave_m = wave / WAVES_N;
-  const int wave_n = wave % WAVES_N;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave >> 1;
+  const int wave_n = wave & 1;
 
-  const __amdgpu_buffer_rsrc_t a_rsrc = MakeRsrc(args.a, args.a_bytes);
-  const __amdgpu_buffer_rsrc_t b_rsrc = MakeRsrc(args.b, args.b_bytes);
+  const v4i a_rsrc = MakeRsrc(args.a, args.a_bytes);
+  const v4i b_rsrc = MakeRsrc(args.b, args.b_bytes);
+  // The 32-bit LDS address of the dynamic shared array (what M0 wants).
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 
-  // ---- global -> LDS assignment: granule q = tid + i*kThreads of the tile ----
-  uint32_t a_goff[C::kAGranules];  // byte offset of (row, granule 0-of-this-thread) at depth 0
-  int a_loff[C::kAGranules];
-  int a_k[C::kAGranules];
+  // ---- global -> LDS assignment ----
+  // Load i of this wave fills LDS 16-byte slots [chunk*64, chunk*64+64) of the
+  // tile; slot p holds tile row p / granules-per-row, granule
+  // (p % granules-per-row) ^ Swizzle(row).
+  const int K = args.K;
+  uint32_t a_goff[C::kALoads];
+  int a_k[C::kALoads];
 #pragma unroll
-  for (int i = 0; i < C::kAGranules; ++i) {
-    const int q = tid + i * C::kThreads;
-    const int r = q / kGranulesPerRow;
-    const int g = q % kGranulesPerRow;
+  for (int i = 0; i < C::kALoads; ++i) {
+    const int chunk = wave * C::kALoads + i;
+    const int r = chunk * C::kRowsPerLoad + lane / C::kGranulesPerRow;
+    const int g = (lane % C::kGranulesPerRow) ^ Swizzle<BK>(r);
     const int row = m0 + r;
     a_goff[i] = row < args.M ? uint32_t(row) * uint32_t(args.lda) + g * kGranule : kOutOfRange;
-    a_loff[i] = LdsOffset(r, g);
     a_k[i] = g * kGranule;
   }
-  uint32_t b_goff[C::kBGranules];
-  int b_loff[C::kBGranules];
-  int b_k[C::kBGranules];
+  uint32_t b_goff[C::kBLoads];
+  int b_k[C::kBLoads];
 #pragma unroll
-  for (int i = 0; i < C::kBGranules; ++i) {
-    const int q = tid + i * C::kThreads;
-    const int r = q / kGranulesPerRow;
-    const int g = q % kGranulesPerRow;
+  for (int i = 0; i < C::kBLoads; ++i) {
+    const int chunk = wave * C::kBLoads + i;
+    const int r = chunk * C::kRowsPerLoad + lane / C::kGranulesPerRow;
+    const int g = (lane % C::kGranulesPerRow) ^ Swizzle<BK>(r);
     const int col = n0 + r;
     b_goff[i] = col < args.N ? uint32_t(col) * uint32_t(args.ldb) + g * kGranule : kOutOfRange;
-    b_loff[i] = C::kBM * kBK + LdsOffset(r, g);
     b_k[i] = g * kGranule;
   }
+  // Issues the loads of depth step kt into ring slot kt % kStages. Steps past
+  // the end of the depth are issued too (they fetch zeros) so that the number
+  // of loads in flight, which the vmcnt waits count, never depends on K.
+  auto issue = [&](int kt) {
+    const int kbase = kt * kBK;
+    const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
+#pragma unroll
+    for (int i = 0; i < C::kALoads; ++i) {
+      const uint32_t off = (kbase + a_k[i] < K) ? a_goff[i] + kbase : kOutOfRange;
+      LoadToLds16(stage + (wave * C::kALoads + i) * 1024, off, a_rsrc);
+    }
+#pragma unroll
+    for (int i = 0; i < C::kBLoads; ++i) {
+      const uint32_t off = (kbase + b_k[i] < K) ? b_goff[i] + kbase : kOutOfRange;
+      LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, off, b_rsrc);
+    }
+  };
 
-  // ---- LDS -> MFMA fragment addresses (byte offsets inside a stage) ----
-  // Fragment for 32x32 block `bm`, depth sub-step ks in {0,1}: lane reads row
-  // wave_m*WM*32 + bm*32 + lane%32, granule ks*2 + lane/32.
+  // ---- LDS -> MFMA fragments ----
+  // Fragment of 32x32 block b, depth sub-step ks: lane reads tile row
+  // b*32 + lane%32, granule ks*2 + lane/32.
   const int frag_row = lane & 31;
   const int frag_half = lane >> 5;
+  int a_foff[C::kKSteps], b_foff[C::kKSteps];  // byte offsets inside a stage, block 0 of this wave
+#pragma unroll
+  for (int ks = 0; ks < C::kKSteps; ++ks) {
+    // Blocks are 32 rows apart, which leaves the swizzle term unchanged.
+    a_foff[ks] = LdsOffset<BK>(wave_m * WM * 32 + frag_row, ks * 2 + frag_half);
+    b_foff[ks] = C::kBM * kBK + LdsOffset<BK>(wave_n * WN * 32 + frag_row, ks * 2 + frag_half);
+  }
+  struct Frags {
+    v4i a[WM];
+    v4i b[WN];
+  };
+  auto read_frags = [&](int kt, int ks, Frags& f) {
+    const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+      f.a[i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * 32 * kBK);
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+      f.b[j] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * 32 * kBK);
+  };
 
   v16i acc[WM][WN];
 #pragma unroll
@@ -130,69 +223,47 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Arg
     for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+  auto mma = [&](const Frags& f) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+  };
 
-  const int K = args.K;
   const int k_tiles = (K + kBK - 1) / kBK;
 
-  v4i a_stage[C::kAGranules];
-  v4i b_stage[C::kBGranules];
-
-  auto load_global = [&](int kt) {
-    const int kbase = kt * kBK;
+  // ---- software pipeline ----
+  // Fragments are double-buffered in registers: while the matrix instructions
+  // of depth sub-step ks run, the fragments of sub-step ks+1 are read from LDS.
+  // At the last sub-step of ring step kt the next fragments belong to step
+  // kt+1: wait until its loads have landed, barrier (after which every wave has
+  // also finished reading step kt, so its ring slot is free), issue the loads
+  // of step kt+kStages into that slot, then read fragments (kt+1, 0).
 #pragma unroll
-    for (int i = 0; i < C::kAGranules; ++i) {
-      const uint32_t off = (kbase + a_k[i] < K) ? a_goff[i] + kbase : kOutOfRange;
-      a_stage[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, off, 0, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < C::kBGranules; ++i) {
-      const uint32_t off = (kbase + b_k[i] < K) ? b_goff[i] + kbase : kOutOfRange;
-      b_stage[i] = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, off, 0, 0);
-    }
-  };
-  auto store_lds = [&](int buf) {
-    char* base = lds + buf * C::kStageBytes;
-#pragma unroll
-    for (int i = 0; i < C::kAGranules; ++i) *reinterpret_cast<v4i*>(base + a_loff[i]) = a_stage[i];
-#pragma unroll
-    for (int i = 0; i < C::kBGranules; ++i) *reinterpret_cast<v4i*>(base + b_loff[i]) = b_stage[i];
-  };
-
-  if (k_tiles > 0) {
-    load_global(0);
-    store_lds(0);
-  }
+  for (int s = 0; s < C::kStages; ++s) issue(s);
+  WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
   __syncthreads();
-
+  Frags f[2];
+  read_frags(0, 0, f[0]);
   for (int kt = 0; kt < k_tiles; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < k_tiles) load_global(kt + 1);
-    const char* a_base = lds + buf * C::kStageBytes;
-    const char* b_base = a_base + C::kBM * kBK;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      v4i a_frag[WM];
-      v4i b_frag[WN];
-      const int g = ks * 2 + frag_half;
-#pragma unroll
-      for (int i = 0; i < WM; ++i) {
-        const int r = (wave_m * WM + i) * 32 + frag_row;
-        a_frag[i] = *reinterpret_cast<const v4i*>(a_base + LdsOffset(r, g));
+    for (int ks = 0; ks < C::kKSteps; ++ks) {
+      if (ks + 1 < C::kKSteps) {
+        read_frags(kt, ks + 1, f[(ks + 1) & 1]);
+      } else {
+        WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
+        __syncthreads();
+        issue(kt + C::kStages);
+        read_frags(kt + 1, 0, f[0]);
       }
-#pragma unroll
-      for (int j = 0; j < WN; ++j) {
-        const int r = (wave_n * WN + j) * 32 + frag_row;
-        b_frag[j] = *reinterpret_cast<const v4i*>(b_base + LdsOffset(r, g));
-      }
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_frag[i], b_frag[j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(f[ks & 1]);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (kt + 1 < k_tiles) store_lds(buf ^ 1);
-    __syncthreads();
   }
+  WaitVmcnt<0>();
+  __syncthreads();  // every wave is done with the operand ring
 
   // ---- fused write-back ----
   // The destination is column-major here (rows contiguous; the host swaps the
@@ -202,7 +273,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Arg
   // one column of blocks (WM*32 rows x 32 columns) at a time through its own
   // LDS region, after which a lane owns 16 consecutive rows of one column and
   // writes them with one vector store per 16 bytes.
-  __syncthreads();  // every wave is done with the operand stages
   constexpr int kRows = WM * 32;
   constexpr int kPitch = kRows + 4;  // ints; keeps the b128 writes conflict-free
   int* region = reinterpret_cast<int*>(lds) + wave * (32 * kPitch);
@@ -212,6 +282,37 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Arg
   const int elt = args.dst_elt;
   char* dst_base = static_cast<char*>(args.dst.data);
   const int64_t ldd = args.dst.cs;
+  const int chunk = lane % kChunksPerCol;
+  const int i0 = m0 + wave_m * kRows + chunk * 16;
+  const bool row_channel = !ep.channel_is_col;
+  const bool per_channel = ep.mult_fixedpoint != nullptr;
+
+  // Everything that depends only on the destination row is the same for all
+  // columns this lane will write: gather it once.
+  uint32_t row_add[16];
+  int32_t row_m[16], row_e[16];
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int i = i0 + q;
+    uint32_t add = static_cast<uint32_t>(ep.zp_product_depth);
+    int32_t m = ep.mult_fixedpoint_scalar, e = ep.mult_exponent_scalar;
+    if (i < args.M) {
+      if (ep.bias && row_channel) add += static_cast<uint32_t>(static_cast<const int32_t*>(ep.bias)[i]);
+      if (ep.rhs_zero_point)
+        add -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[i]);
+      if (per_channel && row_channel) {
+        m = ep.mult_fixedpoint[i];
+        e = ep.mult_exponent[i];
+      }
+    }
+    row_add[q] = add;
+    row_m[q] = m;
+    row_e[q] = e;
+  }
+  // Wave-uniform fast requantization: scalar multiplier with exponent <= -2.
+  const bool uniform_high = ep.requantize && !per_channel && ep.mult_exponent_scalar <= -2;
+  const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
+
 #pragma unroll
   for (int bj = 0; bj < WN; ++bj) {
 #pragma unroll
@@ -228,8 +329,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Arg
       }
     }
     __builtin_amdgcn_wave_barrier();
-    const int chunk = lane % kChunksPerCol;
-    const int i0 = m0 + wave_m * kRows + chunk * 16;
     for (int pass = 0; pass < 32 / kColsPerPass; ++pass) {
       const int c = pass * kColsPerPass + lane / kChunksPerCol;
       const int j = n0 + (wave_n * WN + bj) * 32 + c;
@@ -244,11 +343,33 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Arg
         vals[4 * q + 2] = w[2];
         vals[4 * q + 3] = w[3];
       }
-      const bool full = i0 + 16 <= args.M;
+      uint32_t col_add = 0;
+      int32_t col_m = 0, col_e = 0;
+      if (ep.bias && !row_channel) col_add += static_cast<uint32_t>(static_cast<const int32_t*>(ep.bias)[j]);
+      if (ep.lhs_zero_point)
+        col_add -= static_cast<uint32_t>(ep.lhs_zero_point) * static_cast<uint32_t>(ep.rhs_sums[j]);
+      if (per_channel && !row_channel) {
+        col_m = ep.mult_fixedpoint[j];
+        col_e = ep.mult_exponent[j];
+      }
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        if (full || i0 + q < args.M) vals[q] = FinishInt<true>(vals[q], i0 + q, j, ep);
+        int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + row_add[q] + col_add);
+        if (ep.requantize) {
+          if (uniform_high) {
+            v = RequantHigh(v, ep.mult_fixedpoint_scalar, high_shift);
+          } else {
+            const int32_t m = (per_channel && !row_channel) ? col_m : row_m[q];
+            const int e = (per_channel && !row_channel) ? col_e : row_e[q];
+            v = MultiplyByQuantizedMultiplier(v, m, e);
+          }
+        }
+        v = static_cast<int32_t>(static_cast<uint32_t>(v) + static_cast<uint32_t>(ep.dst_zero_point));
+        v = v > ep.clamp_max_i ? ep.clamp_max_i : v;
+        v = v < ep.clamp_min_i ? ep.clamp_min_i : v;
+        vals[q] = v;
       }
+      const bool full = i0 + 16 <= args.M;
       char* out = dst_base + (int64_t(j) * ldd + i0) * elt;
       if (full && args.dst_vector_ok) {
         if (elt == 1) {
@@ -294,16 +415,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void GemmI8Kernel(GemmI8Arg
   }
 }
 
-template <int WAVES_M, int WAVES_N, int WM, int WN>
+template <int WM, int WN, int BK, int STAGES>
 hipError_t Launch(hipStream_t stream, const GemmI8Args& args) {
-  using C = Cfg<WAVES_M, WAVES_N, WM, WN>;
+  using C = Cfg<WM, WN, BK, STAGES>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
   const int tiles_n = (args.N + C::kBN - 1) / C::kBN;
   const int total = tiles_m * tiles_n;
   const int grid = ((total + 7) / 8) * 8;
-  const size_t epilogue_bytes = size_t(WAVES_M * WAVES_N) * 32 * (WM * 32 + 4) * 4;
-  const size_t lds_bytes = 2 * C::kStageBytes > epilogue_bytes ? 2 * C::kStageBytes : epilogue_bytes;
-  auto kernel = GemmI8Kernel<WAVES_M, WAVES_N, WM, WN>;
+  const size_t lds_bytes = C::kLdsBytes;
+  auto kernel = GemmI8Kernel<WM, WN, BK, STAGES>;
   static bool attr_set = false;
   if (!attr_set && lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -323,9 +443,9 @@ int GemmI8TileCount(const GemmI8Args& args, int bm, int bn) {
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmI8Args& args, int num_cus) {
   // Largest tile that still gives every CU something to do.
-  if (GemmI8TileCount(args, 256, 256) >= num_cus) return Launch<2, 2, 4, 4>(stream, args);
-  if (GemmI8TileCount(args, 128, 128) >= num_cus) return Launch<2, 2, 2, 2>(stream, args);
-  return Launch<2, 2, 1, 1>(stream, args);
+  if (GemmI8TileCount(args, 256, 256) >= num_cus) return Launch<4, 4, 128, 2>(stream, args);
+  if (GemmI8TileCount(args, 128, 128) >= num_cus) return Launch<2, 2, 128, 3>(stream, args);
+  return Launch<1, 1, 128, 4>(stream, args);
 }
 
 }  // namespace ruyamd
