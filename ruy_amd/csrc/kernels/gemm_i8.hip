@@ -96,7 +96,11 @@ struct Cfg {
   static constexpr int kBLoads = kBN / kRowsPerLoad / 4;
   static constexpr int kLoadsPerStage = kALoads + kBLoads;
   static constexpr int kStageBytes = (kBM + kBN) * BK;
-  static constexpr int kEpilogueBytes = 4 * 32 * (WM * 32 + 4) * 4;
+  // The write-back stages kEpilogueBlockCols columns of 32x32 blocks per wave
+  // at a time, each column of WM*32 ints padded by 4.
+  static constexpr int kEpilogueBlockCols = WN >= 2 ? WN / 2 : 1;
+  static constexpr int kEpiloguePitch = WM * 32 + 4;
+  static constexpr int kEpilogueBytes = 4 * kEpilogueBlockCols * 32 * kEpiloguePitch * 4;
   static constexpr int kLdsBytes =
       kStages * kStageBytes > kEpilogueBytes ? kStages * kStageBytes : kEpilogueBytes;
 };
@@ -175,19 +179,22 @@ __global__ __launch_bounds__(256) void GemmI8Kernel(GemmI8Args args) {
   // Issues the loads of depth step kt into ring slot kt % kStages. Steps past
   // the end of the depth are issued too (they fetch zeros) so that the number
   // of loads in flight, which the vmcnt waits count, never depends on K.
-  auto issue = [&](int kt) {
+  // Load number n (0 .. kLoadsPerStage-1) of depth step kt: A loads first.
+  auto issue_one = [&](int kt, int n) {
     const int kbase = kt * kBK;
     const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
-#pragma unroll
-    for (int i = 0; i < C::kALoads; ++i) {
-      const uint32_t off = (kbase + a_k[i] < K) ? a_goff[i] + kbase : kOutOfRange;
-      LoadToLds16(stage + (wave * C::kALoads + i) * 1024, off, a_rsrc);
-    }
-#pragma unroll
-    for (int i = 0; i < C::kBLoads; ++i) {
+    if (n < C::kALoads) {
+      const uint32_t off = (kbase + a_k[n] < K) ? a_goff[n] + kbase : kOutOfRange;
+      LoadToLds16(stage + (wave * C::kALoads + n) * 1024, off, a_rsrc);
+    } else {
+      const int i = n - C::kALoads;
       const uint32_t off = (kbase + b_k[i] < K) ? b_goff[i] + kbase : kOutOfRange;
       LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, off, b_rsrc);
     }
+  };
+  auto issue = [&](int kt) {
+#pragma unroll
+    for (int n = 0; n < C::kLoadsPerStage; ++n) issue_one(kt, n);
   };
 
   // ---- LDS -> MFMA fragments ----
@@ -251,15 +258,30 @@ __global__ __launch_bounds__(256) void GemmI8Kernel(GemmI8Args args) {
     for (int ks = 0; ks < C::kKSteps; ++ks) {
       if (ks + 1 < C::kKSteps) {
         read_frags(kt, ks + 1, f[(ks + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(f[ks & 1]);
+        __builtin_amdgcn_sched_barrier(0);
       } else {
         WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
         __syncthreads();
-        issue(kt + C::kStages);
         read_frags(kt + 1, 0, f[0]);
+        // The loads of step kt+kStages are issued one at a time between the
+        // matrix instructions of this sub-step, so the matrix pipe keeps
+        // running while the addresses are generated.
+        const Frags& g = f[ks & 1];
+        constexpr int kMmas = WM * WN;
+#pragma unroll
+        for (int n = 0; n < kMmas; ++n) {
+          __builtin_amdgcn_sched_barrier(0);
+          acc[n / WN][n % WN] =
+              __builtin_amdgcn_mfma_i32_32x32x32_i8(g.a[n / WN], g.b[n % WN], acc[n / WN][n % WN], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int l = n * C::kLoadsPerStage / kMmas; l < (n + 1) * C::kLoadsPerStage / kMmas; ++l)
+            issue_one(kt + C::kStages, l);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
-      mma(f[ks & 1]);
-      __builtin_amdgcn_sched_barrier(0);
     }
   }
   WaitVmcnt<0>();
@@ -274,8 +296,9 @@ __global__ __launch_bounds__(256) void GemmI8Kernel(GemmI8Args args) {
   // LDS region, after which a lane owns 16 consecutive rows of one column and
   // writes them with one vector store per 16 bytes.
   constexpr int kRows = WM * 32;
-  constexpr int kPitch = kRows + 4;  // ints; keeps the b128 writes conflict-free
-  int* region = reinterpret_cast<int*>(lds) + wave * (32 * kPitch);
+  constexpr int kPitch = C::kEpiloguePitch;  // ints; keeps the b128 writes conflict-free
+  constexpr int kHalfCols = C::kEpilogueBlockCols * 32;  // columns staged at a time
+  int* region = reinterpret_cast<int*>(lds) + wave * (kHalfCols * kPitch);
   constexpr int kChunksPerCol = kRows / 16;
   constexpr int kColsPerPass = 64 / kChunksPerCol;
   const Epilogue& ep = args.ep;
@@ -289,49 +312,67 @@ __global__ __launch_bounds__(256) void GemmI8Kernel(GemmI8Args args) {
 
   // Everything that depends only on the destination row is the same for all
   // columns this lane will write: gather it once.
+  // Rows past the end are clamped to the last row (their results are never
+  // stored) so that the loads below carry no per-lane branches and can all be
+  // in flight together.
   uint32_t row_add[16];
   int32_t row_m[16], row_e[16];
+  int row_idx[16];
 #pragma unroll
   for (int q = 0; q < 16; ++q) {
-    const int i = i0 + q;
-    uint32_t add = static_cast<uint32_t>(ep.zp_product_depth);
-    int32_t m = ep.mult_fixedpoint_scalar, e = ep.mult_exponent_scalar;
-    if (i < args.M) {
-      if (ep.bias && row_channel) add += static_cast<uint32_t>(static_cast<const int32_t*>(ep.bias)[i]);
-      if (ep.rhs_zero_point)
-        add -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[i]);
-      if (per_channel && row_channel) {
-        m = ep.mult_fixedpoint[i];
-        e = ep.mult_exponent[i];
-      }
+    row_idx[q] = min(i0 + q, args.M - 1);
+    row_add[q] = static_cast<uint32_t>(ep.zp_product_depth);
+    row_m[q] = ep.mult_fixedpoint_scalar;
+    row_e[q] = ep.mult_exponent_scalar;
+  }
+  if (ep.bias && row_channel) {
+    const int32_t* bias = static_cast<const int32_t*>(ep.bias);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) row_add[q] += static_cast<uint32_t>(bias[row_idx[q]]);
+  }
+  if (ep.rhs_zero_point) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      row_add[q] -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[row_idx[q]]);
+  }
+  if (per_channel && row_channel) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      row_m[q] = ep.mult_fixedpoint[row_idx[q]];
+      row_e[q] = ep.mult_exponent[row_idx[q]];
     }
-    row_add[q] = add;
-    row_m[q] = m;
-    row_e[q] = e;
   }
   // Wave-uniform fast requantization: scalar multiplier with exponent <= -2.
   const bool uniform_high = ep.requantize && !per_channel && ep.mult_exponent_scalar <= -2;
   const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
 
+  // The accumulators go to LDS in straight-line code (their register indices
+  // must be compile-time constants); everything after that is a compact loop,
+  // which keeps the kernel's code well inside the instruction cache.
 #pragma unroll
-  for (int bj = 0; bj < WN; ++bj) {
+  for (int half = 0; half < WN / C::kEpilogueBlockCols; ++half) {
 #pragma unroll
-    for (int bi = 0; bi < WM; ++bi) {
+    for (int bjj = 0; bjj < C::kEpilogueBlockCols; ++bjj) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        v4i w;
-        w[0] = acc[bi][bj][4 * q + 0];
-        w[1] = acc[bi][bj][4 * q + 1];
-        w[2] = acc[bi][bj][4 * q + 2];
-        w[3] = acc[bi][bj][4 * q + 3];
-        const int r = bi * 32 + 8 * q + 4 * frag_half;
-        *reinterpret_cast<v4i*>(region + frag_row * kPitch + r) = w;
+      for (int bi = 0; bi < WM; ++bi) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v16i& a = acc[bi][half * C::kEpilogueBlockCols + bjj];
+          v4i w;
+          w[0] = a[4 * q + 0];
+          w[1] = a[4 * q + 1];
+          w[2] = a[4 * q + 2];
+          w[3] = a[4 * q + 3];
+          const int r = bi * 32 + 8 * q + 4 * frag_half;
+          *reinterpret_cast<v4i*>(region + (bjj * 32 + frag_row) * kPitch + r) = w;
+        }
       }
     }
     __builtin_amdgcn_wave_barrier();
-    for (int pass = 0; pass < 32 / kColsPerPass; ++pass) {
-      const int c = pass * kColsPerPass + lane / kChunksPerCol;
-      const int j = n0 + (wave_n * WN + bj) * 32 + c;
+#pragma unroll 1
+    for (int pass = 0; pass < kHalfCols / kColsPerPass; ++pass) {
+      const int c = pass * kColsPerPass + lane / kChunksPerCol;  // column inside the staged half
+      const int j = n0 + (wave_n * WN + half * C::kEpilogueBlockCols) * 32 + c;
       if (j >= args.N || i0 >= args.M) continue;
       int32_t vals[16];
       const v4i* src = reinterpret_cast<const v4i*>(region + c * kPitch + chunk * 16);
@@ -353,18 +394,25 @@ __global__ __launch_bounds__(256) void GemmI8Kernel(GemmI8Args args) {
         col_e = ep.mult_exponent[j];
       }
 #pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + row_add[q] + col_add);
-        if (ep.requantize) {
-          if (uniform_high) {
-            v = RequantHigh(v, ep.mult_fixedpoint_scalar, high_shift);
-          } else {
-            const int32_t m = (per_channel && !row_channel) ? col_m : row_m[q];
-            const int e = (per_channel && !row_channel) ? col_e : row_e[q];
-            v = MultiplyByQuantizedMultiplier(v, m, e);
-          }
+      for (int q = 0; q < 16; ++q)
+        vals[q] = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + row_add[q] + col_add);
+      // One wave-uniform branch per pass, straight-line code per element.
+      if (uniform_high) {
+        const int32_t m = ep.mult_fixedpoint_scalar;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) vals[q] = RequantHigh(vals[q], m, high_shift);
+      } else if (ep.requantize) {
+        if (per_channel && !row_channel) {
+#pragma unroll
+          for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], col_m, col_e);
+        } else {
+#pragma unroll
+          for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], row_m[q], row_e[q]);
         }
-        v = static_cast<int32_t>(static_cast<uint32_t>(v) + static_cast<uint32_t>(ep.dst_zero_point));
+      }
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
         v = v > ep.clamp_max_i ? ep.clamp_max_i : v;
         v = v < ep.clamp_min_i ? ep.clamp_min_i : v;
         vals[q] = v;
