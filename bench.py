@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of the ruy::Mul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one ruyamd_mul call (through the C ABI) on seeded synthetic operands
+that are already resident in HBM. The headline workload is the int8 GEMM
+M=N=K=8192 with the full fused epilogue (zero points, int32 bias, fixed-point
+requantization to int8, clamp); the same run also measures the int8 GEMV
+M=K=16384, N=1 (prepacked-cache LHS, raw int32 destination) and reports it in
+the "gemv" object. One JSON line is printed:
+
+  value     = 2*M*N*K / step time (the reference's own operation count,
+              ruy/benchmark.cc:199-200), wall clock around K steps
+  roofline  = the dominant kernel against MI355X's published dense int8 MFMA
+              peak (GEMM) or HBM peak (GEMV); its duration is measured with HIP
+              events around each launch on the launch stream
+  cpu_baseline = the stock reference library (built from its own sources into
+              oracle/_ref) timed on this machine's host cores on a bounded
+              slice of the same workload; falls back to the C restatement
+              ("port") when that build is not present.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix peak, TOP/s
+HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E peak, GB/s
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="all", choices=["all", "gemm", "gemv"])
+    ap.add_argument("--size", type=int, default=8192, help="M=N=K of the int8 GEMM")
+    ap.add_argument("--gemv-size", type=int, default=16384, help="M=K of the int8 GEMV")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def device_problem(problem):
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import device_runner
+    return device_runner.DeviceProblem(problem, dst_fill=0)
+
+
+def time_steps(run, steps, warmup, ctx):
+    import torch
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    ctx.kernel_timing()  # drop the warm-up launches
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms, launches = ctx.kernel_timing()
+    return wall / steps, (kernel_ms / launches if launches else None)
+
+
+def load_traffic(name):
+    """Measured HBM bytes per launch, recorded from rocprofv3 --pmc runs."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(name)
+    except (OSError, ValueError):
+        return None
+
+
+def cpu_baseline_gemm(problem, n_slice):
+    """Stock ruy on the host cores over the first n_slice RHS columns."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as O
+    from ruy_amd import workloads as W
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    sub = W.Problem(problem.name, problem.lhs,
+                    W.HostMatrix(problem.rhs.dtype, problem.K, n_slice, problem.rhs.order,
+                                 stride=problem.rhs.stride, zero_point=problem.rhs.zero_point,
+                                 storage=problem.rhs.storage),
+                    W.HostMatrix(problem.dst.dtype, problem.M, n_slice, problem.dst.order,
+                                 zero_point=problem.dst.zero_point),
+                    problem.accum_dtype, bias=problem.bias,
+                    multiplier_fixedpoint=problem.multiplier_fixedpoint,
+                    multiplier_exponent=problem.multiplier_exponent,
+                    clamp_min=problem.clamp_min, clamp_max=problem.clamp_max)
+    ops = 2.0 * sub.M * sub.N * sub.K
+    sample = "first %d of %d rhs columns (M=%d, K=%d)" % (n_slice, problem.N, sub.M, sub.K)
+    if O.stock is not None:
+        l, r, d = sub.lhs.struct(), sub.rhs.struct(), sub.dst.struct()
+        p = sub.params_struct()
+        lat, used = C.c_double(0), C.c_int(0)
+        rc = O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, cores,
+                                         2.0, 2, C.byref(lat), C.byref(used))
+        if rc == 0 and lat.value > 0:
+            return {"value": ops / lat.value / 1e12, "unit": "TOP/s", "cores": cores,
+                    "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
+    t0 = time.perf_counter()
+    O.oracle_mul(sub)
+    dt = time.perf_counter() - t0
+    return {"value": ops / dt / 1e12, "unit": "TOP/s", "cores": cores, "kind": "port",
+            "sample": sample + ", C restatement with OpenMP"}
+
+
+def cpu_baseline_gemv(problem):
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as O
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    nbytes = problem.algorithmic_bytes()
+    sample = "full %dx%d weight, N=%d, LHS kAlwaysCache (warm)" % (problem.M, problem.K, problem.N)
+    if O.stock is not None:
+        l, r, d = problem.lhs.struct(), problem.rhs.struct(), problem.dst.struct()
+        p = problem.params_struct()
+        lat, used = C.c_double(0), C.c_int(0)
+        rc = O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, cores,
+                                         1.0, 3, C.byref(lat), C.byref(used))
+        if rc == 0 and lat.value > 0:
+            return {"value": nbytes / lat.value / 1e9, "unit": "GB/s", "cores": cores,
+                    "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
+    t0 = time.perf_counter()
+    O.oracle_mul(problem)
+    dt = time.perf_counter() - t0
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": sample + ", C restatement with OpenMP"}
+
+
+def bench_gemm(ctx, args):
+    from ruy_amd import workloads as W
+    n = args.size
+    problem = W.config_int8_gemm(n, config_id=6, name="int8_gemm_%d" % n)
+    dp = device_problem(problem)
+    dp.run(ctx)
+    kernel = ctx.last_kernel_name()
+    step_s, kernel_ms = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx)
+    ops = float(problem.ops())
+    out = {
+        "value": ops / step_s / 1e12,
+        "ms_per_step": step_s * 1e3,
+        "kernel": kernel,
+        "roofline": {
+            "bound": "mfma",
+            "achieved": ops / (kernel_ms * 1e-3) / 1e12 if kernel_ms else None,
+            "peak": INT8_MFMA_PEAK_TOPS,
+            "unit": "TOP/s",
+            "frac": ops / (kernel_ms * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS if kernel_ms else None,
+            "traffic": load_traffic("int8_gemm_%d" % n),
+            "kernel_ms": kernel_ms,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_gemm(problem, min(n, 512))
+    return problem, out
+
+
+def bench_gemv(ctx, args):
+    """int8 GEMV with a prepacked-cache LHS. The 256 MiB weight is about the
+    size of the 256 MB Infinity Cache, so the step rotates over four distinct
+    weight matrices (each its own cache entry) to keep the reads cold."""
+    import torch
+    from ruy_amd import workloads as W
+    n = args.gemv_size
+    rotate = 4
+    ctx.set_cache_max_bytes(rotate * (n * n + 4 * n) + (1 << 20))
+    problems = [W.config_int8_gemv(n, 1, weight_seed=i) for i in range(rotate)]
+    dps = [device_problem(p) for p in problems]
+    for dp in dps:
+        dp.run(ctx)  # packs into the cache
+    kernel = ctx.last_kernel_name()
+    state = {"i": 0}
+
+    def run():
+        dps[state["i"] % rotate].run(ctx)
+        state["i"] += 1
+
+    step_s, kernel_ms = time_steps(run, args.steps * 4, args.warmup * 4, ctx)
+    nbytes = float(problems[0].algorithmic_bytes())
+    out = {
+        "metric": "int8 GEMV M=K=%d N=1 algorithmic HBM GB/s" % n,
+        "value": nbytes / step_s / 1e9,
+        "unit": "GB/s",
+        "ms_per_step": step_s * 1e3,
+        "kernel": kernel,
+        "algorithmic_bytes": nbytes,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": nbytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if kernel_ms else None,
+            "traffic": load_traffic("int8_gemv_%d_n1" % n),
+            "kernel_ms": kernel_ms,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_gemv(problems[0])
+    del dps
+    ctx.clear_prepacked_cache()
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path "
+              "(the Mul hot path shards by destination block without any exchange); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from ruy_amd import api
+    ctx = api.Context()
+    # Launch on torch's current stream, return after enqueueing, time the kernels.
+    ctx.set_stream(torch.cuda.current_stream().cuda_stream)
+    ctx.set_synchronous(False)
+    ctx.set_kernel_timing(True)
+
+    line = {
+        "metric": "int8 TOPS @%d^3 (+ GEMV HBM GB/s in 'gemv'), vs MI355X roofline and host-CPU ruy" % args.size,
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic (SplitMix64-seeded uniform int8, random int32 bias)",
+    }
+    if args.workload in ("all", "gemm"):
+        problem, g = bench_gemm(ctx, args)
+        line.update({"value": g["value"], "ms_per_step": g["ms_per_step"],
+                     "roofline": g["roofline"]})
+        if "cpu_baseline" in g:
+            line["cpu_baseline"] = g["cpu_baseline"]
+        line["config"] = {
+            "workload": "int8xint8->int8 GEMM M=N=K=%d, LHS row-major zp 0, RHS col-major zp -3, "
+                        "dst col-major zp 5, int32 bias, multiplier 1395864371*2^-8, clamp [-128,127]" % args.size,
+            "kernel": g["kernel"],
+            "operands": "device-resident",
+        }
+    if args.workload in ("all", "gemv"):
+        gv = bench_gemv(ctx, args)
+        if args.workload == "gemv":
+            line.update({"metric": gv["metric"], "unit": "GB/s", "value": gv["value"],
+                         "ms_per_step": gv["ms_per_step"], "roofline": gv["roofline"],
+                         "config": {"workload": gv["metric"], "kernel": gv["kernel"]}})
+            if "cpu_baseline" in gv:
+                line["cpu_baseline"] = gv["cpu_baseline"]
+        else:
+            line["gemv"] = gv
+    ctx.close()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

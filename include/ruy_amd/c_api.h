@@ -194,6 +194,17 @@ RUYAMD_API int ruyamd_ctx_last_kernel(const ruyamd_ctx* ctx);
  * role of ruy's kInternalStandardCppVariant paths, ruy/kernel.h:150-169). */
 RUYAMD_API void ruyamd_ctx_force_generic_kernel(ruyamd_ctx* ctx, int force);
 
+/* Timing of the main device kernel of each call, for roofline measurements.
+ * While enabled, every ruyamd_mul brackets the launch of its dominant kernel
+ * (the GEMM / GEMV kernel, not the pack or sums helpers) with HIP events on
+ * the context's stream. `ruyamd_ctx_kernel_timing` synchronises the stream,
+ * returns the summed elapsed milliseconds and the number of launches since the
+ * last query, and resets both. No counterpart in the reference, whose
+ * benchmark times whole calls (ruy/test.h:2082-2136). */
+RUYAMD_API int ruyamd_ctx_set_kernel_timing(ruyamd_ctx* ctx, int enable);
+RUYAMD_API int ruyamd_ctx_kernel_timing(ruyamd_ctx* ctx, double* total_ms,
+                                        int64_t* launches);
+
 /* detail::MultiplyByQuantizedMultiplier (ruy/apply_multiplier.cc:48-65)
  * evaluated ON THE DEVICE for n inputs: out[i] = MBQM(x[i], m[i], e[i]).
  * All pointers are device or host pointers like matrix data. Exists so the

@@ -48,6 +48,8 @@ PROTOTYPES = {
     "ruyamd_ctx_force_generic_kernel": (None, [_ctx, C.c_int]),
     "ruyamd_apply_multiplier": (C.c_int, [_ctx, C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_int64]),
+    "ruyamd_ctx_set_kernel_timing": (C.c_int, [_ctx, C.c_int]),
+    "ruyamd_ctx_kernel_timing": (C.c_int, [_ctx, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
     "ruyamd_version": (C.c_char_p, []),
 }
 

@@ -320,6 +320,15 @@ class Context:
     def force_generic_kernel(self, flag):
         lib.ruyamd_ctx_force_generic_kernel(self._h, int(flag))
 
+    def set_kernel_timing(self, flag):
+        self._check(lib.ruyamd_ctx_set_kernel_timing(self._h, int(flag)))
+
+    def kernel_timing(self):
+        """(total milliseconds, launches) of the dominant kernel since the last query."""
+        ms, n = C.c_double(0), C.c_int64(0)
+        self._check(lib.ruyamd_ctx_kernel_timing(self._h, C.byref(ms), C.byref(n)))
+        return ms.value, n.value
+
     def apply_multiplier(self, x, m, e, out, n):
         self._check(lib.ruyamd_apply_multiplier(
             self._h, _address(x), _address(m), _address(e), _address(out), n))

@@ -59,6 +59,22 @@ void Workspace::Reset() {
 
 using ruyamd::PrepackedCache;
 
+bool ruyamd_ctx::TimingBegin() {
+  if (!kernel_timing) return false;
+  std::pair<hipEvent_t, hipEvent_t> ev;
+  if (!timing_pool.empty()) {
+    ev = timing_pool.back();
+    timing_pool.pop_back();
+  } else {
+    if (hipEventCreate(&ev.first) != hipSuccess || hipEventCreate(&ev.second) != hipSuccess) return false;
+  }
+  (void)hipEventRecord(ev.first, stream);
+  timing_pending.push_back(ev);
+  return true;
+}
+
+void ruyamd_ctx::TimingEnd() { (void)hipEventRecord(timing_pending.back().second, stream); }
+
 namespace {
 
 void* DeviceAlloc(std::size_t bytes) {
@@ -117,6 +133,11 @@ void ruyamd_ctx_destroy(ruyamd_ctx* ctx) {
   if (!ctx) return;
   (void)hipStreamSynchronize(ctx->stream);
   ctx->cache.reset();
+  for (auto* v : {&ctx->timing_pending, &ctx->timing_pool})
+    for (auto& ev : *v) {
+      (void)hipEventDestroy(ev.first);
+      (void)hipEventDestroy(ev.second);
+    }
   if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
   delete ctx;
 }
@@ -190,6 +211,28 @@ int64_t ruyamd_ctx_cache_buffers_bytes(const ruyamd_ctx* ctx) { return ctx->cach
 void ruyamd_ctx_set_cache_max_bytes(ruyamd_ctx* ctx, int64_t max_bytes) {
   (void)hipStreamSynchronize(ctx->stream);
   ctx->cache->SetMaxBuffersBytes(static_cast<std::ptrdiff_t>(max_bytes));
+}
+
+int ruyamd_ctx_set_kernel_timing(ruyamd_ctx* ctx, int enable) {
+  if (!ctx) return RUYAMD_E_INVALID;
+  ctx->kernel_timing = enable != 0;
+  return RUYAMD_OK;
+}
+
+int ruyamd_ctx_kernel_timing(ruyamd_ctx* ctx, double* total_ms, int64_t* launches) {
+  if (!ctx || !total_ms || !launches) return RUYAMD_E_INVALID;
+  if (hipStreamSynchronize(ctx->stream) != hipSuccess) return RUYAMD_E_HIP;
+  double sum = 0;
+  for (auto& ev : ctx->timing_pending) {
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, ev.first, ev.second) != hipSuccess) return RUYAMD_E_HIP;
+    sum += ms;
+    ctx->timing_pool.push_back(ev);
+  }
+  *total_ms = sum;
+  *launches = static_cast<int64_t>(ctx->timing_pending.size());
+  ctx->timing_pending.clear();
+  return RUYAMD_OK;
 }
 
 const char* ruyamd_ctx_last_error(const ruyamd_ctx* ctx) {

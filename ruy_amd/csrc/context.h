@@ -9,6 +9,7 @@
 
 #include <memory>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "internal.h"
@@ -59,8 +60,14 @@ struct ruyamd_ctx {
   std::string last_error;
   ruyamd::Workspace workspace;
   std::unique_ptr<ruyamd::PrepackedCache> cache;
-  // Host staging of the destination: copies to perform after the kernel.
   int multiprocessor_count = 0;
+  // Optional timing of the dominant kernel of each call.
+  bool kernel_timing = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pending;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pool;
+  // Brackets for the dispatcher: Begin returns false if timing is off.
+  bool TimingBegin();
+  void TimingEnd();
 };
 
 #endif  // RUY_AMD_CSRC_CONTEXT_H_

@@ -200,7 +200,10 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.dst_elt = DtypeSize(dst.dtype);
   args.dst_vector_ok = (reinterpret_cast<uintptr_t>(args.dst.data) & 15) == 0 &&
                        (args.dst.cs * args.dst_elt) % 16 == 0;
-  if (LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count) != hipSuccess) {
+  const bool timed = ctx->TimingBegin();
+  const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
+  if (timed) ctx->TimingEnd();
+  if (launched != hipSuccess) {
     *err = "int8 MFMA kernel launch failed";
     return RUYAMD_E_HIP;
   }
