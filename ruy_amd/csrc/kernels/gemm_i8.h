@@ -35,6 +35,29 @@ struct GemmI8Args {
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmI8Args& args, int num_cus);
 
+// Skinny multiplication: `rows` wide-side vectors against narrow_count <= 8
+// narrow-side vectors, all depth-contiguous int8 with the same alignment rules
+// as GemmI8Args. `swapped` = 0: the wide side is the LHS (rows of dst), the
+// narrow side the RHS columns; 1: the wide side is the RHS (columns of dst) and
+// the narrow side the LHS rows. `ep` and `dst` are those of the original call
+// (any destination strides).
+struct GemvI8Args {
+  const int8_t* wide = nullptr;
+  const int8_t* narrow = nullptr;
+  uint32_t wide_bytes = 0;
+  uint32_t narrow_bytes = 0;
+  int32_t ld_wide = 0;
+  int32_t ld_narrow = 0;
+  int32_t rows = 0;
+  int32_t narrow_count = 0;
+  int32_t K = 0;
+  int32_t swapped = 0;
+  Epilogue ep;
+  DevMat dst;
+};
+
+hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args);
+
 // A matrix seen as `count` depth-vectors of length K: vector c, depth k is
 // data[c * stride_c + k * stride_k] (elements of `dtype`, uint8 or int8).
 struct PackSource {

@@ -154,11 +154,44 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   if (int rc = PrepareOperand8(ctx, call, 1, rhs.zero_point, lzp != 0, call->rhs_cache_policy,
                                call->rhs_src_key, M, &b, err))
     return rc;
+  const int32_t zp_product_depth =
+      static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
+  if (N <= kSkinnyWidth || M <= kSkinnyWidth) {
+    // Bandwidth-bound shapes: stream the wide side once, no matrix instructions.
+    GemvI8Args g;
+    g.swapped = !(N <= kSkinnyWidth && (M > kSkinnyWidth || M >= N));
+    const Operand8& wide = g.swapped ? b : a;
+    const Operand8& narrow = g.swapped ? a : b;
+    g.wide = wide.data;
+    g.narrow = narrow.data;
+    g.wide_bytes = wide.bytes;
+    g.narrow_bytes = narrow.bytes;
+    g.ld_wide = wide.ld;
+    g.ld_narrow = narrow.ld;
+    g.rows = g.swapped ? N : M;
+    g.narrow_count = g.swapped ? M : N;
+    g.K = RoundUp(K, 16);
+    g.ep = call->ep;
+    g.ep.lhs_sums = a.sums;
+    g.ep.rhs_sums = b.sums;
+    g.ep.lhs_zero_point = lzp;
+    g.ep.rhs_zero_point = rzp;
+    g.ep.zp_product_depth = zp_product_depth;
+    g.dst = call->dst;
+    const bool timed = ctx->TimingBegin();
+    const hipError_t launched = LaunchGemvI8(ctx->stream, g);
+    if (timed) ctx->TimingEnd();
+    if (launched != hipSuccess) {
+      *err = "int8 skinny kernel launch failed";
+      return RUYAMD_E_HIP;
+    }
+    ctx->last_kernel = RUYAMD_KERNEL_I8_GEMV;
+    return RUYAMD_OK;
+  }
   GemmI8Args args;
   args.K = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
   args.ep = call->ep;
-  args.ep.zp_product_depth =
-      static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
+  args.ep.zp_product_depth = zp_product_depth;
   const DevMat& dst = call->dst;
   if (dst.rs == 1) {
     args.a = a.data;
