@@ -8,21 +8,23 @@
 
 namespace ruyamd {
 
-// Operands of the int8 kernels are depth-contiguous int8: row i of `a` (an LHS
-// row) is the K bytes at a + i*lda, column j of `b` (an RHS column) the K bytes
-// at b + j*ldb. Both base pointers and leading dimensions are multiples of 16
-// and K is a multiple of 16; `a_bytes` / `b_bytes` (< 2^31) bound the buffer
-// descriptors, so rows at or past M / N read as zero.
-struct GemmI8Args {
-  const int8_t* a = nullptr;
-  const int8_t* b = nullptr;
+// Operands of the matrix-core kernels are depth-contiguous: row i of `a` (an
+// LHS row) is the k_bytes bytes at a + i*lda, column j of `b` (an RHS column)
+// the k_bytes bytes at b + j*ldb, with lda / ldb in bytes. Both base pointers
+// and leading dimensions are multiples of 16 and k_bytes is a multiple of 16;
+// `a_bytes` / `b_bytes` (< 2^31) bound the buffer descriptors, so rows at or
+// past M / N read as zero. Elements are int8 (LaunchGemmI8) or fp32
+// (LaunchGemmF32).
+struct GemmArgs {
+  const void* a = nullptr;
+  const void* b = nullptr;
   uint32_t a_bytes = 0;
   uint32_t b_bytes = 0;
   int32_t lda = 0;
   int32_t ldb = 0;
   int32_t M = 0;
   int32_t N = 0;
-  int32_t K = 0;
+  int32_t k_bytes = 0;
   Epilogue ep;
   // The destination must be column-major (dst.rs == 1): callers swap the
   // operands for a row-major one. dst_elt is its element size; dst_vector_ok
@@ -33,7 +35,8 @@ struct GemmI8Args {
   int32_t dst_vector_ok = 0;
 };
 
-hipError_t LaunchGemmI8(hipStream_t stream, const GemmI8Args& args, int num_cus);
+hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
+hipError_t LaunchGemmF32(hipStream_t stream, const GemmArgs& args, int num_cus);
 
 // Skinny multiplication: `rows` wide-side vectors against narrow_count <= 8
 // narrow-side vectors, all depth-contiguous int8 with the same alignment rules
@@ -76,6 +79,10 @@ struct PackSource {
 // packed values.
 hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld,
                         int32_t* sums);
+
+// fp32 counterpart: vector c as floats at dst + c*ld (ld in elements, a
+// multiple of 4), zero-filled from K up to ld. `src.dtype` is fp32.
+hipError_t LaunchPackF32(hipStream_t stream, const PackSource& src, float* dst, int32_t ld);
 
 // sums[c] = sum_k data[c*ld + k] for depth-contiguous int8 data with 16-byte
 // aligned base and ld, K a multiple of 16.

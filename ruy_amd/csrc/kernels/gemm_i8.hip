@@ -1,109 +1,16 @@
-// int8 x int8 -> int32 GEMM on the CDNA4 matrix cores with the whole write-back
-// fused: zero-point correction, bias, fixed-point requantization, destination
-// zero point, clamp, cast. Replaces the reference's 8-bit kernels
-// (ruy/kernel_avx512.cc:55-626, generic form ruy/kernel.h:174-241) and the
-// block scheduling above them (ruy/block_map.cc:339-496, ruy/trmul.cc:78-119).
-//
-// Both operands are "depth-contiguous": LHS row i and RHS column j are each a
-// run of K int8 values (that is how the reference packs them too, as columns
-// of the transposed LHS / of the RHS, ruy/pack.h:105-132). That is exactly the
-// operand order of v_mfma_i32_32x32x32_i8: lane l supplies 16 consecutive
-// depth bytes of row/column l%32, at depth offset 16*(l/32).
-//
-// Work decomposition: one workgroup (4 waves, 2 x 2) per BM x BN destination
-// tile, each wave owning WM x WN blocks of 32x32. The depth is walked in steps
-// of BK = 128 bytes (one full 128-byte cache line per row, so every line is
-// fetched from L2 exactly once) through a ring of LDS stages that is filled by
-// buffer_load_dwordx4 ... lds (global memory straight into LDS, no registers),
-// a whole step or more ahead of the matrix instructions. Rows past the end of
-// a matrix and depth granules past K read as zero through the buffer
-// descriptor's bounds check. The 16-byte granules of an LDS row are
-// XOR-swizzled by the row number so that a ds_read_b128 of 16 consecutive rows
-// touches all 64 banks; since a direct-to-LDS load places lane l at
-// base + 16*l, the swizzle is applied to the global address each lane fetches.
+// int8 x int8 -> int32 instantiation of the tiled matrix-core GEMM: one
+// v_mfma_i32_32x32x32_i8 per 16-byte fragment pair, and the integer write-back
+// of ruy/kernel.h:213-237 (bias, zero-point correction from the operand sums,
+// MultiplyByQuantizedMultiplier, destination zero point, clamp).
 #include <hip/hip_runtime.h>
 
-#include "../epilogue.h"
-#include "../internal.h"
-#include "gemm_i8.h"
+#include "mfma_gemm.h"
 
 namespace ruyamd {
 namespace {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-constexpr int kGranule = 16;            // bytes per lane per load
-constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records we accept
-
-// Buffer descriptor words for a raw (stride 0) buffer of `bytes` bytes.
-__device__ __forceinline__ v4i MakeRsrc(const void* p, uint32_t bytes) {
-  const uint64_t a = reinterpret_cast<uint64_t>(p);
-  v4i r;
-  r[0] = __builtin_amdgcn_readfirstlane(static_cast<int>(a & 0xffffffffu));
-  r[1] = __builtin_amdgcn_readfirstlane(static_cast<int>((a >> 32) & 0xffffu));
-  r[2] = __builtin_amdgcn_readfirstlane(static_cast<int>(bytes));
-  r[3] = 0x00020000;
-  return r;
-}
-
-// 16 bytes per lane from buffer offset `voffset` straight into LDS at
-// lds_base + 16*lane (lds_base wave-uniform). Tracked by vmcnt. The compiler
-// does not know this instruction writes LDS, which is the point: it would
-// otherwise drain vmcnt to zero before every LDS read. M0 is not used by
-// anything else in these kernels.
-__device__ __forceinline__ void LoadToLds16(uint32_t lds_base, uint32_t voffset, v4i rsrc) {
-  asm volatile(
-      "s_mov_b32 m0, %0\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %1, %2, 0 offen lds"
-      :
-      : "s"(lds_base), "v"(voffset), "s"(rsrc)
-      : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void WaitVmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-
-// Swizzle term of tile row r: the granule stored in slot s of the row is
-// s ^ Swizzle(r). Chosen so that 16 consecutive rows at one granule index map
-// to 16 different 16-byte bank groups (256 bytes = all 64 banks).
-template <int BK>
-__device__ __forceinline__ int Swizzle(int r) {
-  static_assert(BK == 64 || BK == 128, "");
-  return BK == 64 ? ((r >> 2) & 3) : ((r >> 1) & 7);
-}
-
-// Byte offset inside one operand tile of granule g of tile row r.
-template <int BK>
-__device__ __forceinline__ int LdsOffset(int r, int g) {
-  return r * BK + ((g ^ Swizzle<BK>(r)) << 4);
-}
-
-template <int WM, int WN, int BK, int STAGES>
-struct Cfg {
-  static constexpr int kBM = 2 * WM * 32;
-  static constexpr int kBN = 2 * WN * 32;
-  static constexpr int kBK = BK;
-  static constexpr int kThreads = 256;
-  static constexpr int kStages = STAGES;
-  static constexpr int kKSteps = BK / 32;           // matrix-instruction depth steps per stage
-  static constexpr int kGranulesPerRow = BK / kGranule;
-  static constexpr int kRowsPerLoad = 64 / kGranulesPerRow;  // tile rows one wave-level load covers
-  static constexpr int kALoads = kBM / kRowsPerLoad / 4;     // per wave per stage
-  static constexpr int kBLoads = kBN / kRowsPerLoad / 4;
-  static constexpr int kLoadsPerStage = kALoads + kBLoads;
-  static constexpr int kStageBytes = (kBM + kBN) * BK;
-  // The write-back stages kEpilogueBlockCols columns of 32x32 blocks per wave
-  // at a time, each column of WM*32 ints padded by 4.
-  static constexpr int kEpilogueBlockCols = WN >= 2 ? WN / 2 : 1;
-  static constexpr int kEpiloguePitch = WM * 32 + 4;
-  static constexpr int kEpilogueBytes = 4 * kEpilogueBlockCols * 32 * kEpiloguePitch * 4;
-  static constexpr int kLdsBytes =
-      kStages * kStageBytes > kEpilogueBytes ? kStages * kStageBytes : kEpilogueBytes;
-};
+using mfma_gemm::v16i;
+using mfma_gemm::v4i;
 
 // (hi(x*m) + 2^(s-1)) >> s with s = (31 - e) - 32 >= 1: MultiplyByQuantizedMultiplier
 // when the total shift is at least 33, where the low product word cannot
@@ -112,388 +19,91 @@ __device__ __forceinline__ int32_t RequantHigh(int32_t x, int32_t m, int s) {
   return (__mulhi(x, m) + (1 << (s - 1))) >> s;
 }
 
-template <int WM, int WN, int BK, int STAGES>
-__global__ __launch_bounds__(256) void GemmI8Kernel(GemmI8Args args) {
-  using C = Cfg<WM, WN, BK, STAGES>;
-  constexpr int kBK = BK;
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-
-  // ---- which tile: XCD-aware, grouped ordering ----
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
-  // run of the tile order so that the tiles resident on one XCD share operand
-  // panels in its L2, and order tiles in bands of kGroupM tile-rows so that the
-  // ~32 workgroups running together on an XCD form a compact 2-D patch.
-  const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
-  const int tiles_n = (args.N + C::kBN - 1) / C::kBN;
-  const int total = tiles_m * tiles_n;
-  const int per_xcd = (total + 7) / 8;
-  const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (t >= total) return;
-  constexpr int kGroupM = 4;
-  const int band = t / (kGroupM * tiles_n);
-  const int band_rows = min(kGroupM, tiles_m - band * kGroupM);
-  const int in_band = t - band * kGroupM * tiles_n;
-  const int tile_m = band * kGroupM + in_band % band_rows;
-  const int tile_n = in_band / band_rows;
-  const int m0 = tile_m * C::kBM;
-  const int n0 = tile_n * C::kBN;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wave_m = wave >> 1;
-  const int wave_n = wave & 1;
-
-  const v4i a_rsrc = MakeRsrc(args.a, args.a_bytes);
-  const v4i b_rsrc = MakeRsrc(args.b, args.b_bytes);
-  // The 32-bit LDS address of the dynamic shared array (what M0 wants).
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
-
-  // ---- global -> LDS assignment ----
-  // Load i of this wave fills LDS 16-byte slots [chunk*64, chunk*64+64) of the
-  // tile; slot p holds tile row p / granules-per-row, granule
-  // (p % granules-per-row) ^ Swizzle(row).
-  const int K = args.K;
-  uint32_t a_goff[C::kALoads];
-  int a_k[C::kALoads];
-#pragma unroll
-  for (int i = 0; i < C::kALoads; ++i) {
-    const int chunk = wave * C::kALoads + i;
-    const int r = chunk * C::kRowsPerLoad + lane / C::kGranulesPerRow;
-    const int g = (lane % C::kGranulesPerRow) ^ Swizzle<BK>(r);
-    const int row = m0 + r;
-    a_goff[i] = row < args.M ? uint32_t(row) * uint32_t(args.lda) + g * kGranule : kOutOfRange;
-    a_k[i] = g * kGranule;
+struct Int8Traits {
+  using Acc = v16i;
+  static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
   }
-  uint32_t b_goff[C::kBLoads];
-  int b_k[C::kBLoads];
-#pragma unroll
-  for (int i = 0; i < C::kBLoads; ++i) {
-    const int chunk = wave * C::kBLoads + i;
-    const int r = chunk * C::kRowsPerLoad + lane / C::kGranulesPerRow;
-    const int g = (lane % C::kGranulesPerRow) ^ Swizzle<BK>(r);
-    const int col = n0 + r;
-    b_goff[i] = col < args.N ? uint32_t(col) * uint32_t(args.ldb) + g * kGranule : kOutOfRange;
-    b_k[i] = g * kGranule;
-  }
-  // Issues the loads of depth step kt into ring slot kt % kStages. Steps past
-  // the end of the depth are issued too (they fetch zeros) so that the number
-  // of loads in flight, which the vmcnt waits count, never depends on K.
-  // Load number n (0 .. kLoadsPerStage-1) of depth step kt: A loads first.
-  auto issue_one = [&](int kt, int n) {
-    const int kbase = kt * kBK;
-    const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
-    if (n < C::kALoads) {
-      const uint32_t off = (kbase + a_k[n] < K) ? a_goff[n] + kbase : kOutOfRange;
-      LoadToLds16(stage + (wave * C::kALoads + n) * 1024, off, a_rsrc);
-    } else {
-      const int i = n - C::kALoads;
-      const uint32_t off = (kbase + b_k[i] < K) ? b_goff[i] + kbase : kOutOfRange;
-      LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, off, b_rsrc);
-    }
-  };
-  auto issue = [&](int kt) {
-#pragma unroll
-    for (int n = 0; n < C::kLoadsPerStage; ++n) issue_one(kt, n);
-  };
+  static __device__ __forceinline__ int Bits(int x) { return x; }
 
-  // ---- LDS -> MFMA fragments ----
-  // Fragment of 32x32 block b, depth sub-step ks: lane reads tile row
-  // b*32 + lane%32, granule ks*2 + lane/32.
-  const int frag_row = lane & 31;
-  const int frag_half = lane >> 5;
-  int a_foff[C::kKSteps], b_foff[C::kKSteps];  // byte offsets inside a stage, block 0 of this wave
-#pragma unroll
-  for (int ks = 0; ks < C::kKSteps; ++ks) {
-    // Blocks are 32 rows apart, which leaves the swizzle term unchanged.
-    a_foff[ks] = LdsOffset<BK>(wave_m * WM * 32 + frag_row, ks * 2 + frag_half);
-    b_foff[ks] = C::kBM * kBK + LdsOffset<BK>(wave_n * WN * 32 + frag_row, ks * 2 + frag_half);
-  }
-  struct Frags {
-    v4i a[WM];
-    v4i b[WN];
-  };
-  auto read_frags = [&](int kt, int ks, Frags& f) {
-    const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-      f.a[i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * 32 * kBK);
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-      f.b[j] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * 32 * kBK);
-  };
-
-  v16i acc[WM][WN];
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-  auto mma = [&](const Frags& f) {
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
-  };
-
-  const int k_tiles = (K + kBK - 1) / kBK;
-
-  // ---- software pipeline ----
-  // Fragments are double-buffered in registers: while the matrix instructions
-  // of depth sub-step ks run, the fragments of sub-step ks+1 are read from LDS.
-  // At the last sub-step of ring step kt the next fragments belong to step
-  // kt+1: wait until its loads have landed, barrier (after which every wave has
-  // also finished reading step kt, so its ring slot is free), issue the loads
-  // of step kt+kStages into that slot, then read fragments (kt+1, 0).
-#pragma unroll
-  for (int s = 0; s < C::kStages; ++s) issue(s);
-  WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
-  __syncthreads();
-  Frags f[2];
-  read_frags(0, 0, f[0]);
-  for (int kt = 0; kt < k_tiles; ++kt) {
-#pragma unroll
-    for (int ks = 0; ks < C::kKSteps; ++ks) {
-      if (ks + 1 < C::kKSteps) {
-        read_frags(kt, ks + 1, f[(ks + 1) & 1]);
-        __builtin_amdgcn_sched_barrier(0);
-        mma(f[ks & 1]);
-        __builtin_amdgcn_sched_barrier(0);
-      } else {
-        WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
-        __syncthreads();
-        read_frags(kt + 1, 0, f[0]);
-        // The loads of step kt+kStages are issued one at a time between the
-        // matrix instructions of this sub-step, so the matrix pipe keeps
-        // running while the addresses are generated.
-        const Frags& g = f[ks & 1];
-        constexpr int kMmas = WM * WN;
-#pragma unroll
-        for (int n = 0; n < kMmas; ++n) {
-          __builtin_amdgcn_sched_barrier(0);
-          acc[n / WN][n % WN] =
-              __builtin_amdgcn_mfma_i32_32x32x32_i8(g.a[n / WN], g.b[n % WN], acc[n / WN][n % WN], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int l = n * C::kLoadsPerStage / kMmas; l < (n + 1) * C::kLoadsPerStage / kMmas; ++l)
-            issue_one(kt + C::kStages, l);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  }
-  WaitVmcnt<0>();
-  __syncthreads();  // every wave is done with the operand ring
-
-  // ---- fused write-back ----
-  // The destination is column-major here (rows contiguous; the host swaps the
-  // operands for a row-major destination). In a 32x32 accumulator block lane l
-  // holds column l%32 and rows 8*(v/4) + 4*(l/32) + v%4, so a lane's values are
-  // scattered along the contiguous dimension. Each wave therefore transposes
-  // one column of blocks (WM*32 rows x 32 columns) at a time through its own
-  // LDS region, after which a lane owns 16 consecutive rows of one column and
-  // writes them with one vector store per 16 bytes.
-  constexpr int kRows = WM * 32;
-  constexpr int kPitch = C::kEpiloguePitch;  // ints; keeps the b128 writes conflict-free
-  constexpr int kHalfCols = C::kEpilogueBlockCols * 32;  // columns staged at a time
-  int* region = reinterpret_cast<int*>(lds) + wave * (kHalfCols * kPitch);
-  constexpr int kChunksPerCol = kRows / 16;
-  constexpr int kColsPerPass = 64 / kChunksPerCol;
-  const Epilogue& ep = args.ep;
-  const int elt = args.dst_elt;
-  char* dst_base = static_cast<char*>(args.dst.data);
-  const int64_t ldd = args.dst.cs;
-  const int chunk = lane % kChunksPerCol;
-  const int i0 = m0 + wave_m * kRows + chunk * 16;
-  const bool row_channel = !ep.channel_is_col;
-  const bool per_channel = ep.mult_fixedpoint != nullptr;
-
-  // Everything that depends only on the destination row is the same for all
-  // columns this lane will write: gather it once.
-  // Rows past the end are clamped to the last row (their results are never
-  // stored) so that the loads below carry no per-lane branches and can all be
-  // in flight together.
-  uint32_t row_add[16];
-  int32_t row_m[16], row_e[16];
-  int row_idx[16];
-#pragma unroll
-  for (int q = 0; q < 16; ++q) {
-    row_idx[q] = min(i0 + q, args.M - 1);
-    row_add[q] = static_cast<uint32_t>(ep.zp_product_depth);
-    row_m[q] = ep.mult_fixedpoint_scalar;
-    row_e[q] = ep.mult_exponent_scalar;
-  }
-  if (ep.bias && row_channel) {
-    const int32_t* bias = static_cast<const int32_t*>(ep.bias);
-#pragma unroll
-    for (int q = 0; q < 16; ++q) row_add[q] += static_cast<uint32_t>(bias[row_idx[q]]);
-  }
-  if (ep.rhs_zero_point) {
-#pragma unroll
-    for (int q = 0; q < 16; ++q)
-      row_add[q] -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[row_idx[q]]);
-  }
-  if (per_channel && row_channel) {
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      row_m[q] = ep.mult_fixedpoint[row_idx[q]];
-      row_e[q] = ep.mult_exponent[row_idx[q]];
-    }
-  }
-  // Wave-uniform fast requantization: scalar multiplier with exponent <= -2.
-  const bool uniform_high = ep.requantize && !per_channel && ep.mult_exponent_scalar <= -2;
-  const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
-
-  // The accumulators go to LDS in straight-line code (their register indices
-  // must be compile-time constants); everything after that is a compact loop,
-  // which keeps the kernel's code well inside the instruction cache.
-#pragma unroll
-  for (int half = 0; half < WN / C::kEpilogueBlockCols; ++half) {
-#pragma unroll
-    for (int bjj = 0; bjj < C::kEpilogueBlockCols; ++bjj) {
-#pragma unroll
-      for (int bi = 0; bi < WM; ++bi) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v16i& a = acc[bi][half * C::kEpilogueBlockCols + bjj];
-          v4i w;
-          w[0] = a[4 * q + 0];
-          w[1] = a[4 * q + 1];
-          w[2] = a[4 * q + 2];
-          w[3] = a[4 * q + 3];
-          const int r = bi * 32 + 8 * q + 4 * frag_half;
-          *reinterpret_cast<v4i*>(region + (bjj * 32 + frag_row) * kPitch + r) = w;
-        }
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll 1
-    for (int pass = 0; pass < kHalfCols / kColsPerPass; ++pass) {
-      const int c = pass * kColsPerPass + lane / kChunksPerCol;  // column inside the staged half
-      const int j = n0 + (wave_n * WN + half * C::kEpilogueBlockCols) * 32 + c;
-      if (j >= args.N || i0 >= args.M) continue;
-      int32_t vals[16];
-      const v4i* src = reinterpret_cast<const v4i*>(region + c * kPitch + chunk * 16);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const v4i w = src[q];
-        vals[4 * q + 0] = w[0];
-        vals[4 * q + 1] = w[1];
-        vals[4 * q + 2] = w[2];
-        vals[4 * q + 3] = w[3];
-      }
-      uint32_t col_add = 0;
-      int32_t col_m = 0, col_e = 0;
-      if (ep.bias && !row_channel) col_add += static_cast<uint32_t>(static_cast<const int32_t*>(ep.bias)[j]);
-      if (ep.lhs_zero_point)
-        col_add -= static_cast<uint32_t>(ep.lhs_zero_point) * static_cast<uint32_t>(ep.rhs_sums[j]);
-      if (per_channel && !row_channel) {
-        col_m = ep.mult_fixedpoint[j];
-        col_e = ep.mult_exponent[j];
-      }
-#pragma unroll
-      for (int q = 0; q < 16; ++q)
-        vals[q] = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + row_add[q] + col_add);
-      // One wave-uniform branch per pass, straight-line code per element.
-      if (uniform_high) {
-        const int32_t m = ep.mult_fixedpoint_scalar;
-#pragma unroll
-        for (int q = 0; q < 16; ++q) vals[q] = RequantHigh(vals[q], m, high_shift);
-      } else if (ep.requantize) {
-        if (per_channel && !row_channel) {
-#pragma unroll
-          for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], col_m, col_e);
-        } else {
-#pragma unroll
-          for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], row_m[q], row_e[q]);
-        }
-      }
+  struct RowState {
+    uint32_t add[16];
+    int32_t m[16];
+    int32_t e[16];
+    __device__ __forceinline__ void Load(const Epilogue& ep, const int (&row_idx)[16]) {
+      const bool row_channel = !ep.channel_is_col;
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
-        v = v > ep.clamp_max_i ? ep.clamp_max_i : v;
-        v = v < ep.clamp_min_i ? ep.clamp_min_i : v;
-        vals[q] = v;
+        add[q] = static_cast<uint32_t>(ep.zp_product_depth);
+        m[q] = ep.mult_fixedpoint_scalar;
+        e[q] = ep.mult_exponent_scalar;
       }
-      const bool full = i0 + 16 <= args.M;
-      char* out = dst_base + (int64_t(j) * ldd + i0) * elt;
-      if (full && args.dst_vector_ok) {
-        if (elt == 1) {
-          v4i w;
+      if (ep.bias && row_channel) {
+        const int32_t* bias = static_cast<const int32_t*>(ep.bias);
 #pragma unroll
-          for (int q = 0; q < 4; ++q)
-            w[q] = (vals[4 * q] & 0xff) | ((vals[4 * q + 1] & 0xff) << 8) |
-                   ((vals[4 * q + 2] & 0xff) << 16) | (vals[4 * q + 3] << 24);
-          *reinterpret_cast<v4i*>(out) = w;
-        } else if (elt == 2) {
+        for (int q = 0; q < 16; ++q) add[q] += static_cast<uint32_t>(bias[row_idx[q]]);
+      }
+      if (ep.rhs_zero_point) {
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            v4i w;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              w[q] = (vals[8 * h + 2 * q] & 0xffff) | (vals[8 * h + 2 * q + 1] << 16);
-            reinterpret_cast<v4i*>(out)[h] = w;
-          }
-        } else {
-#pragma unroll
-          for (int h = 0; h < 4; ++h) {
-            v4i w;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) w[q] = vals[4 * h + q];
-            reinterpret_cast<v4i*>(out)[h] = w;
-          }
-        }
-      } else {
+        for (int q = 0; q < 16; ++q)
+          add[q] -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[row_idx[q]]);
+      }
+      if (ep.mult_fixedpoint && row_channel) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
-          if (i0 + q < args.M) {
-            if (elt == 1)
-              reinterpret_cast<int8_t*>(out)[q] = static_cast<int8_t>(vals[q]);
-            else if (elt == 2)
-              reinterpret_cast<int16_t*>(out)[q] = static_cast<int16_t>(vals[q]);
-            else
-              reinterpret_cast<int32_t*>(out)[q] = vals[q];
-          }
+          m[q] = ep.mult_fixedpoint[row_idx[q]];
+          e[q] = ep.mult_exponent[row_idx[q]];
         }
       }
     }
-    __builtin_amdgcn_wave_barrier();
-  }
-}
+  };
 
-template <int WM, int WN, int BK, int STAGES>
-hipError_t Launch(hipStream_t stream, const GemmI8Args& args) {
-  using C = Cfg<WM, WN, BK, STAGES>;
-  const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
-  const int tiles_n = (args.N + C::kBN - 1) / C::kBN;
-  const int total = tiles_m * tiles_n;
-  const int grid = ((total + 7) / 8) * 8;
-  const size_t lds_bytes = C::kLdsBytes;
-  auto kernel = GemmI8Kernel<WM, WN, BK, STAGES>;
-  static bool attr_set = false;
-  if (!attr_set && lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
-    if (e != hipSuccess) return e;
-    attr_set = true;
+  static __device__ __forceinline__ void Finish(int32_t (&vals)[16], const RowState& rows, int j,
+                                                const Epilogue& ep) {
+    const bool row_channel = !ep.channel_is_col;
+    const bool per_channel = ep.mult_fixedpoint != nullptr;
+    uint32_t col_add = 0;
+    int32_t col_m = 0, col_e = 0;
+    if (ep.bias && !row_channel) col_add += static_cast<uint32_t>(static_cast<const int32_t*>(ep.bias)[j]);
+    if (ep.lhs_zero_point)
+      col_add -= static_cast<uint32_t>(ep.lhs_zero_point) * static_cast<uint32_t>(ep.rhs_sums[j]);
+    if (per_channel && !row_channel) {
+      col_m = ep.mult_fixedpoint[j];
+      col_e = ep.mult_exponent[j];
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      vals[q] = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + rows.add[q] + col_add);
+    // One wave-uniform branch per column, straight-line code per element.
+    // Fast path: scalar multiplier with exponent <= -2.
+    if (ep.requantize && !per_channel && ep.mult_exponent_scalar <= -2) {
+      const int32_t m = ep.mult_fixedpoint_scalar;
+      const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
+#pragma unroll
+      for (int q = 0; q < 16; ++q) vals[q] = RequantHigh(vals[q], m, high_shift);
+    } else if (ep.requantize) {
+      if (per_channel && !row_channel) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], col_m, col_e);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], rows.m[q], rows.e[q]);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
+      v = v > ep.clamp_max_i ? ep.clamp_max_i : v;
+      v = v < ep.clamp_min_i ? ep.clamp_min_i : v;
+      vals[q] = v;
+    }
   }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::kThreads), lds_bytes, stream, args);
-  return hipGetLastError();
-}
+};
 
 }  // namespace
 
-int GemmI8TileCount(const GemmI8Args& args, int bm, int bn) {
-  return ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
-}
-
-hipError_t LaunchGemmI8(hipStream_t stream, const GemmI8Args& args, int num_cus) {
-  // Largest tile that still gives every CU something to do.
-  if (GemmI8TileCount(args, 256, 256) >= num_cus) return Launch<4, 4, 128, 2>(stream, args);
-  if (GemmI8TileCount(args, 128, 128) >= num_cus) return Launch<2, 2, 128, 3>(stream, args);
-  return Launch<1, 1, 128, 4>(stream, args);
+hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
+  return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);
 }
 
 }  // namespace ruyamd

@@ -134,7 +134,51 @@ __global__ __launch_bounds__(256) void SumsI8Kernel(const int8_t* data, int32_t 
   if (lane == 0) sums[c] = total;
 }
 
+// fp32 re-layout: 32 vectors x 32 depth positions per step through LDS, so that
+// reads follow the source's contiguous dimension and writes follow depth.
+// There are no sums and no conversion for floating point
+// (ruy/pack_common.h:100-133).
+__global__ __launch_bounds__(256) void PackF32Kernel(PackSource src, float* dst, int32_t ld) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31;
+  const int ty = threadIdx.x >> 5;  // 0..7
+  const int c0 = blockIdx.x * 32;
+  const float* s = static_cast<const float*>(src.data);
+  const bool depth_contiguous = src.stride_k == 1;
+  for (int k0 = blockIdx.y * 32; k0 < ld; k0 += gridDim.y * 32) {
+#pragma unroll
+    for (int t = ty; t < 32; t += 8) {
+      // (c, k) read so that tx runs along the contiguous source dimension
+      const int c = c0 + (depth_contiguous ? t : tx);
+      const int k = k0 + (depth_contiguous ? tx : t);
+      float v = 0.f;
+      if (c < src.count && k < src.K) v = s[c * src.stride_c + k * src.stride_k];
+      if (depth_contiguous)
+        tile[t][tx] = v;
+      else
+        tile[tx][t] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = ty; t < 32; t += 8) {
+      const int c = c0 + t;
+      const int k = k0 + tx;
+      if (c < src.count && k < ld) dst[int64_t(c) * ld + k] = tile[t][tx];
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace
+
+hipError_t LaunchPackF32(hipStream_t stream, const PackSource& src, float* dst, int32_t ld) {
+  if (src.count == 0 || ld == 0) return hipSuccess;
+  const int blocks_c = (src.count + 31) / 32;
+  int blocks_k = (ld + 31) / 32;
+  if (blocks_k > 64) blocks_k = 64;
+  hipLaunchKernelGGL(PackF32Kernel, dim3(blocks_c, blocks_k), dim3(256), 0, stream, src, dst, ld);
+  return hipGetLastError();
+}
 
 hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld,
                         int32_t* sums) {

@@ -13,6 +13,8 @@ namespace {
 // bandwidth-bound kernel".
 constexpr int kSkinnyWidth = 8;
 
+bool SetupDestination(const MulCall& call, GemmArgs* args);
+
 bool Is8Bit(int dtype) { return dtype == RUYAMD_DTYPE_U8 || dtype == RUYAMD_DTYPE_I8; }
 
 int32_t RoundUp(int32_t x, int32_t m) { return (x + m - 1) / m * m; }
@@ -188,51 +190,24 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     ctx->last_kernel = RUYAMD_KERNEL_I8_GEMV;
     return RUYAMD_OK;
   }
-  GemmI8Args args;
-  args.K = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
-  args.ep = call->ep;
+  GemmArgs args;
+  args.k_bytes = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
+  const bool swap = SetupDestination(*call, &args);
   args.ep.zp_product_depth = zp_product_depth;
-  const DevMat& dst = call->dst;
-  if (dst.rs == 1) {
-    args.a = a.data;
-    args.b = b.data;
-    args.a_bytes = a.bytes;
-    args.b_bytes = b.bytes;
-    args.lda = a.ld;
-    args.ldb = b.ld;
-    args.M = M;
-    args.N = N;
-    args.ep.lhs_sums = a.sums;
-    args.ep.rhs_sums = b.sums;
-    args.ep.lhs_zero_point = lzp;
-    args.ep.rhs_zero_point = rzp;
-    args.dst = dst;
-  } else {
-    // Row-major destination: compute dst^T = rhs^T * lhs^T, which is
-    // column-major in the same memory, with the channel dimension flipped
-    // (ruy/create_trmul_params.h:471-479).
-    args.a = b.data;
-    args.b = a.data;
-    args.a_bytes = b.bytes;
-    args.b_bytes = a.bytes;
-    args.lda = b.ld;
-    args.ldb = a.ld;
-    args.M = N;
-    args.N = M;
-    args.ep.lhs_sums = b.sums;
-    args.ep.rhs_sums = a.sums;
-    args.ep.lhs_zero_point = rzp;
-    args.ep.rhs_zero_point = lzp;
-    args.ep.channel_is_col = !call->ep.channel_is_col;
-    args.dst = dst;
-    args.dst.rows = dst.cols;
-    args.dst.cols = dst.rows;
-    args.dst.rs = 1;
-    args.dst.cs = dst.rs;
-  }
-  args.dst_elt = DtypeSize(dst.dtype);
-  args.dst_vector_ok = (reinterpret_cast<uintptr_t>(args.dst.data) & 15) == 0 &&
-                       (args.dst.cs * args.dst_elt) % 16 == 0;
+  const Operand8& x = swap ? b : a;
+  const Operand8& y = swap ? a : b;
+  args.a = x.data;
+  args.b = y.data;
+  args.a_bytes = x.bytes;
+  args.b_bytes = y.bytes;
+  args.lda = x.ld;
+  args.ldb = y.ld;
+  args.M = swap ? N : M;
+  args.N = swap ? M : N;
+  args.ep.lhs_sums = x.sums;
+  args.ep.rhs_sums = y.sums;
+  args.ep.lhs_zero_point = swap ? rzp : lzp;
+  args.ep.rhs_zero_point = swap ? lzp : rzp;
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
@@ -241,6 +216,134 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     return RUYAMD_E_HIP;
   }
   ctx->last_kernel = RUYAMD_KERNEL_I8_MFMA;
+  return RUYAMD_OK;
+}
+
+// One side of an fp32 multiplication, ready for the fp32 matrix-core kernel.
+struct OperandF32 {
+  const float* data = nullptr;
+  int32_t ld = 0;  // elements
+  uint32_t bytes = 0;
+};
+
+int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy,
+                      const void* src_key, int other_width, OperandF32* out, std::string* err) {
+  auto view = [&]() {
+    const DevMat& m = side == 0 ? call->lhs : call->rhs;
+    return side == 0 ? PackSource{m.data, m.rs, m.cs, m.rows, m.cols, m.dtype}
+                     : PackSource{m.data, m.cs, m.rs, m.cols, m.rows, m.dtype};
+  };
+  PackSource src = view();
+  const int32_t K = src.K;
+  const int32_t ld = RoundUp(K > 0 ? K : 1, 4);
+  const uint64_t packed_bytes = uint64_t(src.count) * ld * 4;
+  if (packed_bytes >= (uint64_t(1) << 31)) {
+    *err = "operand larger than 2 GiB is not supported by the fp32 matrix-core kernel";
+    return RUYAMD_E_UNSUPPORTED;
+  }
+  if (ShouldCache(cache_policy, other_width)) {
+    PackedMatrix pm;
+    pm.element_size = 4;
+    pm.is_floating_point = true;
+    pm.layout.rows = ld;
+    pm.layout.cols = src.count;
+    pm.layout.stride = ld;
+    pm.layout.kernel_rows = 4;
+    pm.layout.kernel_cols = 1;
+    const auto action = ctx->cache->Get(src_key, &pm);
+    if (!pm.data) {
+      *err = "device allocation for a cached packed matrix failed";
+      return RUYAMD_E_HIP;
+    }
+    if (action == PrepackedCache::Action::kInsertedNewEntry) {
+      if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
+      src = view();
+      if (LaunchPackF32(ctx->stream, src, static_cast<float*>(pm.data), ld) != hipSuccess) {
+        *err = "pack kernel launch failed";
+        return RUYAMD_E_HIP;
+      }
+    }
+    out->data = static_cast<const float*>(pm.data);
+    out->ld = ld;
+    out->bytes = static_cast<uint32_t>(packed_bytes);
+    return RUYAMD_OK;
+  }
+  if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
+  src = view();
+  const uint64_t extent = src.count > 0 ? (uint64_t(src.count - 1) * uint64_t(src.stride_c) + K) * 4 : 0;
+  const bool direct = src.stride_k == 1 && K % 4 == 0 && K > 0 &&
+                      (reinterpret_cast<uintptr_t>(src.data) & 15) == 0 &&
+                      (src.stride_c % 4 == 0 || src.count == 1) && extent < (uint64_t(1) << 31);
+  if (direct) {
+    out->data = static_cast<const float*>(src.data);
+    out->ld = src.count == 1 ? ld : static_cast<int32_t>(src.stride_c);
+    out->bytes = static_cast<uint32_t>(extent);
+    return RUYAMD_OK;
+  }
+  float* packed = static_cast<float*>(ctx->workspace.Alloc(packed_bytes ? packed_bytes : 16));
+  if (!packed) {
+    *err = "workspace allocation failed";
+    return RUYAMD_E_HIP;
+  }
+  if (LaunchPackF32(ctx->stream, src, packed, ld) != hipSuccess) {
+    *err = "pack kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  out->data = packed;
+  out->ld = ld;
+  out->bytes = static_cast<uint32_t>(packed_bytes);
+  return RUYAMD_OK;
+}
+
+// Fills the destination-side fields of GemmArgs. The kernels write a
+// column-major destination; a row-major one is computed as dst^T = rhs^T *
+// lhs^T in the same memory with the channel dimension flipped
+// (ruy/create_trmul_params.h:471-479). Returns true if the operands must be
+// swapped.
+bool SetupDestination(const MulCall& call, GemmArgs* args) {
+  const DevMat& dst = call.dst;
+  args->ep = call.ep;
+  const bool swap = dst.rs != 1;
+  args->dst = dst;
+  if (swap) {
+    args->ep.channel_is_col = !call.ep.channel_is_col;
+    args->dst.rows = dst.cols;
+    args->dst.cols = dst.rows;
+    args->dst.rs = 1;
+    args->dst.cs = dst.rs;
+  }
+  args->dst_elt = DtypeSize(dst.dtype);
+  args->dst_vector_ok = (reinterpret_cast<uintptr_t>(args->dst.data) & 15) == 0 &&
+                        (args->dst.cs * args->dst_elt) % 16 == 0;
+  return swap;
+}
+
+int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
+  const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
+  OperandF32 a, b;
+  if (int rc = PrepareOperandF32(ctx, call, 0, call->lhs_cache_policy, call->lhs_src_key, N, &a, err)) return rc;
+  if (int rc = PrepareOperandF32(ctx, call, 1, call->rhs_cache_policy, call->rhs_src_key, M, &b, err)) return rc;
+  GemmArgs args;
+  args.k_bytes = RoundUp(K, 4) * 4;
+  const bool swap = SetupDestination(*call, &args);
+  const OperandF32& x = swap ? b : a;
+  const OperandF32& y = swap ? a : b;
+  args.a = x.data;
+  args.b = y.data;
+  args.a_bytes = x.bytes;
+  args.b_bytes = y.bytes;
+  args.lda = x.ld * 4;
+  args.ldb = y.ld * 4;
+  args.M = swap ? N : M;
+  args.N = swap ? M : N;
+  const bool timed = ctx->TimingBegin();
+  const hipError_t launched = LaunchGemmF32(ctx->stream, args, ctx->multiprocessor_count);
+  if (timed) ctx->TimingEnd();
+  if (launched != hipSuccess) {
+    *err = "fp32 matrix-core kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  ctx->last_kernel = RUYAMD_KERNEL_F32_MFMA;
   return RUYAMD_OK;
 }
 
@@ -266,6 +369,10 @@ int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const DevMat& rhs = call->rhs;
   if (!ctx->force_generic) {
     if (Is8Bit(lhs.dtype) && Is8Bit(rhs.dtype)) return RunInt8(ctx, call, err);
+    if (lhs.dtype == RUYAMD_DTYPE_F32 && rhs.dtype == RUYAMD_DTYPE_F32 &&
+        call->dst.dtype == RUYAMD_DTYPE_F32 && call->accum_dtype == RUYAMD_DTYPE_F32 &&
+        lhs.rows > kSkinnyWidth && rhs.cols > kSkinnyWidth)
+      return RunF32(ctx, call, err);
   }
   if (int rc = EnsureOnDevice(ctx, call, 0, err)) return rc;
   if (int rc = EnsureOnDevice(ctx, call, 1, err)) return rc;
