@@ -23,7 +23,8 @@ struct F32Traits {
     for (int e = 0; e < 4; ++e)
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[e]), __int_as_float(b[e]), acc, 0, 0, 0);
   }
-  static __device__ __forceinline__ int Bits(float x) { return __float_as_int(x); }
+  static constexpr bool kSplitB = false;
+  static __device__ __forceinline__ int Bits(float x, float) { return __float_as_int(x); }
 
   struct RowState {
     float bias[16];

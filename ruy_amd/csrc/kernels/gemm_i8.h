@@ -25,6 +25,9 @@ struct GemmArgs {
   int32_t M = 0;
   int32_t N = 0;
   int32_t k_bytes = 0;
+  // Number of destination columns. Equal to N except for the int16 kernel,
+  // where N counts the rows of the plane-split B operand (64 per 32 columns).
+  int32_t n_logical = 0;
   Epilogue ep;
   // The destination must be column-major (dst.rs == 1): callers swap the
   // operands for a row-major one. dst_elt is its element size; dst_vector_ok
@@ -37,6 +40,8 @@ struct GemmArgs {
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmF32(hipStream_t stream, const GemmArgs& args, int num_cus);
+// int8 x int16: `b` is the int16 operand split by LaunchPackI16Split.
+hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus);
 
 // Skinny multiplication: `rows` wide-side vectors against narrow_count <= 8
 // narrow-side vectors, all depth-contiguous int8 with the same alignment rules
@@ -79,6 +84,15 @@ struct PackSource {
 // packed values.
 hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld,
                         int32_t* sums);
+
+// int16 operand for the int8 matrix cores: each value v is split into
+// hi = v >> 8 (signed) and lo = (v & 0xff) - 128, both int8, so that
+// v = 256*hi + lo + 128. For every group of 32 vectors the 32 hi vectors are
+// written first, then the 32 lo vectors: vector c of plane p lands at
+// dst + ((c/32)*64 + p*32 + c%32) * ld. Vectors past `count` inside the last
+// group and depth past K are zero. The destination holds
+// ceil(count/32)*64 vectors.
+hipError_t LaunchPackI16Split(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld);
 
 // fp32 counterpart: vector c as floats at dst + c*ld (ld in elements, a
 // multiple of 4), zero-filled from K up to ld. `src.dtype` is fp32.

@@ -24,7 +24,8 @@ struct Int8Traits {
   static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
   }
-  static __device__ __forceinline__ int Bits(int x) { return x; }
+  static constexpr bool kSplitB = false;
+  static __device__ __forceinline__ int Bits(int x, int) { return x; }
 
   struct RowState {
     uint32_t add[16];
@@ -100,7 +101,25 @@ struct Int8Traits {
   }
 };
 
+// int8 x int16 (ruy/kernel_avx512.cc:55-626 instantiated for a 16-bit RHS,
+// ruy/kernel_x86.h:62-90): the int16 operand arrives split into a high and a
+// low int8 plane, v = 256*hi + (lo + 128), and each plane is multiplied on
+// the int8 matrix cores. The two accumulators of a destination element
+// combine as 256*acc_hi + acc_lo; the remaining "+128 * sum of the int8
+// row" is the ordinary zero-point correction with an RHS zero point of -128,
+// which the dispatcher sets. Everything is exact modulo 2^32.
+struct Int8SplitTraits : Int8Traits {
+  static constexpr bool kSplitB = true;
+  static __device__ __forceinline__ int Bits(int hi, int lo) {
+    return static_cast<int>(static_cast<uint32_t>(hi) * 256u + static_cast<uint32_t>(lo));
+  }
+};
+
 }  // namespace
+
+hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus) {
+  return mfma_gemm::LaunchBest<Int8SplitTraits>(stream, args, num_cus);
+}
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
   return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);

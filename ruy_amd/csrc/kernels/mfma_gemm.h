@@ -26,7 +26,10 @@
 // base + 16*l, the swizzle is applied to the global address each lane fetches.
 //
 // A Traits type supplies: Acc (16-element accumulator vector), Mma(a, b, acc)
-// for one 16-byte fragment pair, Bits(x) (accumulator element as raw 32 bits),
+// for one 16-byte fragment pair, kSplitB (the B operand holds, for every 32
+// destination columns, 32 high-plane rows followed by 32 low-plane rows whose
+// accumulators are combined), Bits(x, x2) (accumulator element - or combined
+// pair - as raw 32 bits),
 // RowState (per-destination-row write-back parameters, gathered once per lane)
 // and Finish(vals, rows, j, ep), which turns 16 raw accumulators of column j
 // into 16 destination values (as raw 32-bit words).
@@ -97,7 +100,7 @@ __device__ __forceinline__ int LdsOffset(int r, int g) {
   return r * BK + ((g ^ Swizzle<BK>(r)) << 4);
 }
 
-template <int WM, int WN, int BK, int STAGES>
+template <int WM, int WN, int BK, int STAGES, bool SPLIT_B = false>
 struct Cfg {
   static constexpr int kBM = 2 * WM * 32;
   static constexpr int kBN = 2 * WN * 32;
@@ -113,7 +116,11 @@ struct Cfg {
   static constexpr int kStageBytes = (kBM + kBN) * BK;
   // The write-back stages kEpilogueBlockCols columns of 32x32 blocks per wave
   // at a time, each column of WM*32 ints padded by 4.
-  static constexpr int kEpilogueBlockCols = WN >= 2 ? WN / 2 : 1;
+  // With SPLIT_B two adjacent physical block columns (high-byte and low-byte
+  // plane of the same 32 destination columns) combine into one logical column.
+  static constexpr int kLogicalWN = SPLIT_B ? WN / 2 : WN;
+  static_assert(!SPLIT_B || WN % 2 == 0, "");
+  static constexpr int kEpilogueBlockCols = kLogicalWN >= 2 ? kLogicalWN / 2 : 1;
   static constexpr int kEpiloguePitch = WM * 32 + 4;
   static constexpr int kEpilogueBytes = 4 * kEpilogueBlockCols * 32 * kEpiloguePitch * 4;
   static constexpr int kLdsBytes =
@@ -122,7 +129,7 @@ struct Cfg {
 
 template <typename Traits, int WM, int WN, int BK, int STAGES>
 __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
-  using C = Cfg<WM, WN, BK, STAGES>;
+  using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   constexpr int kBK = BK;
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -329,19 +336,22 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // must be compile-time constants); everything after that is a compact loop,
   // which keeps the kernel's code well inside the instruction cache.
 #pragma unroll
-  for (int half = 0; half < WN / C::kEpilogueBlockCols; ++half) {
+  for (int half = 0; half < C::kLogicalWN / C::kEpilogueBlockCols; ++half) {
 #pragma unroll
     for (int bjj = 0; bjj < C::kEpilogueBlockCols; ++bjj) {
 #pragma unroll
       for (int bi = 0; bi < WM; ++bi) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const typename Traits::Acc& a = acc[bi][half * C::kEpilogueBlockCols + bjj];
+          constexpr int kPhys = Traits::kSplitB ? 2 : 1;
+          const int lb = half * C::kEpilogueBlockCols + bjj;  // logical block column
+          const typename Traits::Acc& a = acc[bi][kPhys * lb];
+          const typename Traits::Acc& a2 = acc[bi][kPhys * lb + kPhys - 1];
           v4i w;
-          w[0] = Traits::Bits(a[4 * q + 0]);
-          w[1] = Traits::Bits(a[4 * q + 1]);
-          w[2] = Traits::Bits(a[4 * q + 2]);
-          w[3] = Traits::Bits(a[4 * q + 3]);
+          w[0] = Traits::Bits(a[4 * q + 0], a2[4 * q + 0]);
+          w[1] = Traits::Bits(a[4 * q + 1], a2[4 * q + 1]);
+          w[2] = Traits::Bits(a[4 * q + 2], a2[4 * q + 2]);
+          w[3] = Traits::Bits(a[4 * q + 3], a2[4 * q + 3]);
           const int r = bi * 32 + 8 * q + 4 * frag_half;
           *reinterpret_cast<v4i*>(region + (bjj * 32 + frag_row) * kPitch + r) = w;
         }
@@ -351,8 +361,9 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 #pragma unroll 1
     for (int pass = 0; pass < kHalfCols / kColsPerPass; ++pass) {
       const int c = pass * kColsPerPass + lane / kChunksPerCol;  // column inside the staged half
-      const int j = n0 + (wave_n * WN + half * C::kEpilogueBlockCols) * 32 + c;
-      if (j >= args.N || i0 >= args.M) continue;
+      const int j = (Traits::kSplitB ? n0 / 2 : n0) +
+                    (wave_n * C::kLogicalWN + half * C::kEpilogueBlockCols) * 32 + c;
+      if (j >= args.n_logical || i0 >= args.M) continue;
       int32_t vals[16];
       const v4i* src = reinterpret_cast<const v4i*>(region + c * kPitch + chunk * 16);
 #pragma unroll
@@ -412,7 +423,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 
 template <typename Traits, int WM, int WN, int BK, int STAGES>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
-  using C = Cfg<WM, WN, BK, STAGES>;
+  using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
   const int tiles_n = (args.N + C::kBN - 1) / C::kBN;
   const int total = tiles_m * tiles_n;
@@ -438,8 +449,9 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
 template <typename Traits>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
   if (TileCount(args, 256, 256) >= num_cus) return Launch<Traits, 4, 4, 128, 2>(stream, args);
-  if (TileCount(args, 128, 128) >= num_cus) return Launch<Traits, 2, 2, 128, 3>(stream, args);
-  return Launch<Traits, 1, 1, 128, 4>(stream, args);
+  if (TileCount(args, 128, 128) >= num_cus || Traits::kSplitB) return Launch<Traits, 2, 2, 128, 3>(stream, args);
+  if constexpr (!Traits::kSplitB) return Launch<Traits, 1, 1, 128, 4>(stream, args);
+  return hipErrorInvalidValue;
 }
 
 }  // namespace mfma_gemm

@@ -169,7 +169,64 @@ __global__ __launch_bounds__(256) void PackF32Kernel(PackSource src, float* dst,
   }
 }
 
+// int16 -> two int8 planes. Block = 32 vectors (one group) x a depth span; the
+// 32x32 int16 tile goes through LDS so reads follow the source's contiguous
+// dimension; each thread then emits 4 consecutive depth bytes of one plane.
+__global__ __launch_bounds__(256) void PackI16SplitKernel(PackSource src, int8_t* dst, int32_t ld) {
+  __shared__ int16_t tile[32][33];
+  const int tx = threadIdx.x & 31;
+  const int ty = threadIdx.x >> 5;  // 0..7
+  const int group = blockIdx.x;
+  const int c0 = group * 32;
+  const int16_t* s = static_cast<const int16_t*>(src.data);
+  const bool depth_contiguous = src.stride_k == 1;
+  for (int k0 = blockIdx.y * 32; k0 < ld; k0 += gridDim.y * 32) {
+#pragma unroll
+    for (int t = ty; t < 32; t += 8) {
+      const int c = c0 + (depth_contiguous ? t : tx);
+      const int k = k0 + (depth_contiguous ? tx : t);
+      int16_t v = 0;
+      bool real = c < src.count && k < src.K;
+      if (real) v = s[c * src.stride_c + k * src.stride_k];
+      if (depth_contiguous)
+        tile[t][tx] = v;
+      else
+        tile[tx][t] = v;
+    }
+    __syncthreads();
+    // thread -> (vector cc = tid / 8, depth quad kq = tid % 8), both planes
+    const int cc = threadIdx.x >> 3;
+    const int kq = (threadIdx.x & 7) * 4;
+    if (k0 + kq < ld) {
+      uint32_t hi = 0, lo = 0;
+      const bool real_c = c0 + cc < src.count;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const int k = k0 + kq + d;
+        if (real_c && k < src.K) {
+          const int v = tile[cc][kq + d];
+          hi |= (static_cast<uint32_t>(v >> 8) & 0xffu) << (8 * d);
+          lo |= (static_cast<uint32_t>((v & 0xff) - 128) & 0xffu) << (8 * d);
+        }
+      }
+      int8_t* base = dst + (int64_t(group) * 64 + cc) * ld + k0 + kq;
+      *reinterpret_cast<uint32_t*>(base) = hi;
+      *reinterpret_cast<uint32_t*>(base + int64_t(32) * ld) = lo;
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace
+
+hipError_t LaunchPackI16Split(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld) {
+  if (src.count == 0 || ld == 0) return hipSuccess;
+  const int groups = (src.count + 31) / 32;
+  int blocks_k = (ld + 31) / 32;
+  if (blocks_k > 64) blocks_k = 64;
+  hipLaunchKernelGGL(PackI16SplitKernel, dim3(groups, blocks_k), dim3(256), 0, stream, src, dst, ld);
+  return hipGetLastError();
+}
 
 hipError_t LaunchPackF32(hipStream_t stream, const PackSource& src, float* dst, int32_t ld) {
   if (src.count == 0 || ld == 0) return hipSuccess;

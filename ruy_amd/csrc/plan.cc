@@ -204,6 +204,7 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.ldb = y.ld;
   args.M = swap ? N : M;
   args.N = swap ? M : N;
+  args.n_logical = args.N;
   args.ep.lhs_sums = x.sums;
   args.ep.rhs_sums = y.sums;
   args.ep.lhs_zero_point = swap ? rzp : lzp;
@@ -336,6 +337,7 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.ldb = y.ld * 4;
   args.M = swap ? N : M;
   args.N = swap ? M : N;
+  args.n_logical = args.N;
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmF32(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
@@ -344,6 +346,66 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     return RUYAMD_E_HIP;
   }
   ctx->last_kernel = RUYAMD_KERNEL_F32_MFMA;
+  return RUYAMD_OK;
+}
+
+// int8 x int16 (either side) when the int8 side runs along the destination's
+// contiguous dimension. All zero points are 0 here (ruy/validate.h:51-57).
+int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
+  const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
+  GemmArgs args;
+  const bool swap = SetupDestination(*call, &args);  // true: A side = rhs
+  const int side8 = swap ? 1 : 0;
+  const int side16 = 1 - side8;
+  Operand8 a;
+  if (int rc = PrepareOperand8(ctx, call, side8, 0, /*need_sums=*/true,
+                               side8 == 0 ? call->lhs_cache_policy : call->rhs_cache_policy,
+                               side8 == 0 ? call->lhs_src_key : call->rhs_src_key,
+                               side8 == 0 ? N : M, &a, err))
+    return rc;
+  if (int rc = EnsureOnDevice(ctx, call, side16, err)) return rc;
+  const DevMat& m16 = side16 == 0 ? call->lhs : call->rhs;
+  const PackSource src = side16 == 0 ? PackSource{m16.data, m16.rs, m16.cs, m16.rows, m16.cols, m16.dtype}
+                                     : PackSource{m16.data, m16.cs, m16.rs, m16.cols, m16.rows, m16.dtype};
+  const int32_t ld = RoundUp(K > 0 ? K : 1, 16);
+  const int32_t n_phys = (src.count + 31) / 32 * 64;
+  const uint64_t packed_bytes = uint64_t(n_phys) * ld;
+  if (packed_bytes >= (uint64_t(1) << 31)) {
+    *err = "int16 operand too large for the matrix-core kernel";
+    return RUYAMD_E_UNSUPPORTED;
+  }
+  int8_t* planes = static_cast<int8_t*>(ctx->workspace.Alloc(packed_bytes));
+  if (!planes) {
+    *err = "workspace allocation failed";
+    return RUYAMD_E_HIP;
+  }
+  if (LaunchPackI16Split(ctx->stream, src, planes, ld) != hipSuccess) {
+    *err = "int16 pack kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  args.k_bytes = RoundUp(K, 16);
+  args.a = a.data;
+  args.a_bytes = a.bytes;
+  args.lda = a.ld;
+  args.b = planes;
+  args.b_bytes = static_cast<uint32_t>(packed_bytes);
+  args.ldb = ld;
+  args.M = swap ? N : M;
+  args.N = n_phys;
+  args.n_logical = src.count;
+  args.ep.lhs_sums = a.sums;
+  args.ep.rhs_sums = nullptr;
+  args.ep.lhs_zero_point = 0;
+  args.ep.rhs_zero_point = -128;  // the low plane stores (v & 0xff) - 128
+  args.ep.zp_product_depth = 0;
+  const bool timed = ctx->TimingBegin();
+  const hipError_t launched = LaunchGemmI8I16(ctx->stream, args, ctx->multiprocessor_count);
+  if (timed) ctx->TimingEnd();
+  if (launched != hipSuccess) {
+    *err = "int8 x int16 matrix-core kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  ctx->last_kernel = RUYAMD_KERNEL_I8I16_MFMA;
   return RUYAMD_OK;
 }
 
@@ -369,6 +431,14 @@ int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const DevMat& rhs = call->rhs;
   if (!ctx->force_generic) {
     if (Is8Bit(lhs.dtype) && Is8Bit(rhs.dtype)) return RunInt8(ctx, call, err);
+    {
+      // The int8 side must run along the destination's contiguous dimension.
+      const bool dst_col_major = call->dst.rs == 1;
+      const DevMat& side8 = dst_col_major ? lhs : rhs;
+      const DevMat& side16 = dst_col_major ? rhs : lhs;
+      if (side8.dtype == RUYAMD_DTYPE_I8 && side16.dtype == RUYAMD_DTYPE_I16)
+        return RunI8I16(ctx, call, err);
+    }
     if (lhs.dtype == RUYAMD_DTYPE_F32 && rhs.dtype == RUYAMD_DTYPE_F32 &&
         call->dst.dtype == RUYAMD_DTYPE_F32 && call->accum_dtype == RUYAMD_DTYPE_F32 &&
         lhs.rows > kSkinnyWidth && rhs.cols > kSkinnyWidth)
