@@ -1,0 +1,20 @@
+// ruy::PerformanceAdvisory (ruy/performance_advisory.h:21-38 in the
+// reference). The device kernels mask per-channel buffer accesses instead of
+// reallocating the buffers, so kReallocatedPerChannelBuffer is never raised.
+#ifndef RUY_AMD_INCLUDE_RUY_PERFORMANCE_ADVISORY_H_
+#define RUY_AMD_INCLUDE_RUY_PERFORMANCE_ADVISORY_H_
+
+namespace ruy {
+
+enum class PerformanceAdvisory { kNone = 0, kReallocatedPerChannelBuffer = 0x1 };
+
+inline constexpr PerformanceAdvisory operator|(PerformanceAdvisory p, PerformanceAdvisory q) {
+  return static_cast<PerformanceAdvisory>(static_cast<int>(p) | static_cast<int>(q));
+}
+inline constexpr PerformanceAdvisory operator&(PerformanceAdvisory p, PerformanceAdvisory q) {
+  return static_cast<PerformanceAdvisory>(static_cast<int>(p) & static_cast<int>(q));
+}
+
+}  // namespace ruy
+
+#endif  // RUY_AMD_INCLUDE_RUY_PERFORMANCE_ADVISORY_H_

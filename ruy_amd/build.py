@@ -70,5 +70,26 @@ def build(force=False, verbose=True):
     return LIB
 
 
+def build_cpp_tests(verbose=True):
+    """The two C++ test programs under tests/cpp: the host-only unit test of the
+    prepacked cache and the end-to-end test of the ruy:: headers (needs a GPU to
+    run, not to build)."""
+    tdir = os.path.join(ROOT, "tests", "cpp")
+    cmds = [
+        ["g++", "-std=c++17", "-O1", "-I" + CSRC, os.path.join(tdir, "prepacked_cache_test.cc"),
+         os.path.join(CSRC, "prepacked_cache.cc"), "-o", os.path.join(tdir, "prepacked_cache_test")],
+        ["g++", "-std=c++14", "-O1", "-I" + os.path.join(ROOT, "include"),
+         os.path.join(tdir, "api_test.cc"), "-L" + HERE, "-lruy_amd",
+         "-Wl,-rpath,$ORIGIN/../../ruy_amd", "-o", os.path.join(tdir, "api_test")],
+    ]
+    for cmd in cmds:
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("build failed: %s\n%s%s" % (" ".join(cmd), r.stdout, r.stderr))
+    if verbose:
+        print("built tests/cpp/prepacked_cache_test, tests/cpp/api_test")
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)
+    build_cpp_tests()

@@ -440,8 +440,7 @@ int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
         return RunI8I16(ctx, call, err);
     }
     if (lhs.dtype == RUYAMD_DTYPE_F32 && rhs.dtype == RUYAMD_DTYPE_F32 &&
-        call->dst.dtype == RUYAMD_DTYPE_F32 && call->accum_dtype == RUYAMD_DTYPE_F32 &&
-        lhs.rows > kSkinnyWidth && rhs.cols > kSkinnyWidth)
+        call->dst.dtype == RUYAMD_DTYPE_F32 && call->accum_dtype == RUYAMD_DTYPE_F32)
       return RunF32(ctx, call, err);
   }
   if (int rc = EnsureOnDevice(ctx, call, 0, err)) return rc;

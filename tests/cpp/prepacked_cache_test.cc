@@ -1,0 +1,163 @@
+// Host-only unit test of ruyamd::PrepackedCache with a malloc allocator.
+// Mirrors the reference's known answers for the cache
+// (ruy/prepacked_cache_test.cc:54-227): byte accounting 307 / 860, ejection of
+// the least recently used entry, an over-budget entry is still kept, and keys
+// that differ in pointer, shape, order or kernel layout are distinct.
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "prepacked_cache.h"
+
+using ruyamd::PackedMatrix;
+using ruyamd::PrepackedCache;
+
+static int g_failures = 0;
+static int g_live_allocations = 0;
+#define EXPECT(cond)                                                          \
+  do {                                                                        \
+    if (!(cond)) {                                                            \
+      std::fprintf(stderr, "%s:%d: EXPECT failed: %s\n", __FILE__, __LINE__, #cond); \
+      ++g_failures;                                                           \
+    }                                                                         \
+  } while (0)
+
+static void* CountingAlloc(std::size_t n) {
+  ++g_live_allocations;
+  return std::malloc(n);
+}
+static void CountingFree(void* p) {
+  if (p) --g_live_allocations;
+  std::free(p);
+}
+
+static PackedMatrix Dummy(bool is_float, int rows, int cols) {
+  PackedMatrix m;
+  m.element_size = is_float ? 4 : 1;
+  m.is_floating_point = is_float;
+  m.layout.rows = rows;
+  m.layout.cols = cols;
+  m.layout.stride = rows;
+  m.layout.order = 0;
+  m.layout.kernel_rows = 1;
+  m.layout.kernel_cols = 1;
+  return m;
+}
+
+static const auto kInserted = PrepackedCache::Action::kInsertedNewEntry;
+static const auto kExisting = PrepackedCache::Action::kGotExistingEntry;
+
+static void TestBasic() {
+  PrepackedCache cache(CountingAlloc, CountingFree, 307);
+  std::vector<std::uint8_t> data1(10 * 20), data2(5 * 3);
+  PackedMatrix mat1 = Dummy(false, 10, 20);  // 200 + 20*4 = 280 bytes
+  PackedMatrix mat2 = Dummy(false, 5, 3);    // 15 + 3*4 = 27 bytes
+  EXPECT(cache.Get(data1.data(), &mat1) == kInserted);
+  EXPECT(mat1.data != nullptr && mat1.sums != nullptr);
+  EXPECT(cache.Get(data2.data(), &mat2) == kInserted);
+  EXPECT(cache.MatrixCount() == 2);
+  EXPECT(cache.BuffersBytes() == 307);
+  PackedMatrix again = Dummy(false, 10, 20);
+  EXPECT(cache.Get(data1.data(), &again) == kExisting);
+  EXPECT(again.data == mat1.data && again.sums == mat1.sums);
+  EXPECT(cache.Get(data2.data(), &mat2) == kExisting);
+}
+
+static void TestBasicFloat() {
+  PrepackedCache cache(CountingAlloc, CountingFree, 860);
+  std::vector<float> data1(10 * 20), data2(5 * 3);
+  PackedMatrix mat1 = Dummy(true, 10, 20);  // 800 bytes, no sums
+  PackedMatrix mat2 = Dummy(true, 5, 3);    // 60 bytes
+  EXPECT(cache.Get(data1.data(), &mat1) == kInserted);
+  EXPECT(mat1.sums == nullptr);
+  EXPECT(cache.Get(data2.data(), &mat2) == kInserted);
+  EXPECT(cache.MatrixCount() == 2);
+  EXPECT(cache.BuffersBytes() == 860);
+  EXPECT(cache.Get(data1.data(), &mat1) == kExisting);
+  EXPECT(cache.Get(data2.data(), &mat2) == kExisting);
+}
+
+static void TestEjection() {
+  PrepackedCache cache(CountingAlloc, CountingFree, 306);  // one byte short of both
+  std::vector<std::uint8_t> data1(10 * 20), data2(5 * 3);
+  PackedMatrix mat1 = Dummy(false, 10, 20), mat2 = Dummy(false, 5, 3);
+  cache.Get(data1.data(), &mat1);
+  cache.Get(data2.data(), &mat2);
+  EXPECT(cache.MatrixCount() == 1);
+  EXPECT(cache.BuffersBytes() == 27);
+  EXPECT(cache.Get(data2.data(), &mat2) == kExisting);
+  EXPECT(cache.Get(data1.data(), &mat1) == kInserted);
+  EXPECT(cache.MatrixCount() == 1);
+  EXPECT(cache.BuffersBytes() == 280);
+  EXPECT(cache.Get(data1.data(), &mat1) == kExisting);
+  EXPECT(cache.Get(data2.data(), &mat2) == kInserted);
+}
+
+static void TestEjectionOrder() {
+  PrepackedCache cache(CountingAlloc, CountingFree, 1000);
+  std::vector<std::uint8_t> d1(200), d2(200), d3(200), d4(200);
+  PackedMatrix m1 = Dummy(false, 10, 20), m2 = m1, m3 = m1, m4 = m1;
+  cache.Get(d1.data(), &m1);
+  cache.Get(d2.data(), &m2);
+  cache.Get(d3.data(), &m3);
+  EXPECT(cache.Get(d1.data(), &m1) == kExisting);  // touch 1 and 3: 2 is the oldest
+  EXPECT(cache.Get(d3.data(), &m3) == kExisting);
+  cache.Get(d4.data(), &m4);
+  EXPECT(cache.MatrixCount() == 3);
+  EXPECT(cache.Get(d1.data(), &m1) == kExisting);
+  EXPECT(cache.Get(d3.data(), &m3) == kExisting);
+  EXPECT(cache.Get(d4.data(), &m4) == kExisting);
+  EXPECT(cache.Get(d2.data(), &m2) == kInserted);
+}
+
+static void TestOversizeEntryIsKept() {
+  PrepackedCache cache(CountingAlloc, CountingFree, 100);
+  std::vector<std::uint8_t> d1(200);
+  PackedMatrix m1 = Dummy(false, 10, 20);
+  EXPECT(cache.Get(d1.data(), &m1) == kInserted);  // 280 > 100: ejection stops at empty
+  EXPECT(cache.MatrixCount() == 1);
+  EXPECT(cache.Get(d1.data(), &m1) == kExisting);
+}
+
+static void TestDistinguishSubtlyDifferentMatrices() {
+  PrepackedCache cache(CountingAlloc, CountingFree);
+  EXPECT(cache.MaxBuffersBytes() == (1 << 28));
+  std::vector<std::uint8_t> data(10 * 20 + 1);
+  PackedMatrix m = Dummy(false, 10, 20);
+  EXPECT(cache.Get(data.data(), &m) == kInserted);
+  EXPECT(cache.Get(data.data() + 1, &m) == kInserted);  // other source pointer
+  m.layout.rows = 9;
+  EXPECT(cache.Get(data.data(), &m) == kInserted);
+  m.layout.cols = 19;
+  EXPECT(cache.Get(data.data(), &m) == kInserted);
+  m.layout.order = 1;
+  EXPECT(cache.Get(data.data(), &m) == kInserted);
+  m.layout.kernel_rows = 2;
+  EXPECT(cache.Get(data.data(), &m) == kInserted);
+  m.layout.kernel_cols = 2;
+  EXPECT(cache.Get(data.data(), &m) == kInserted);
+  m.layout.kernel_order = 1;
+  EXPECT(cache.Get(data.data(), &m) == kInserted);
+  m.zero_point = 3;
+  EXPECT(cache.Get(data.data(), &m) == kInserted);  // other zero point
+  EXPECT(cache.MatrixCount() == 9);
+  cache.Clear();
+  EXPECT(cache.MatrixCount() == 0 && cache.BuffersBytes() == 0);
+}
+
+int main() {
+  TestBasic();
+  TestBasicFloat();
+  TestEjection();
+  TestEjectionOrder();
+  TestOversizeEntryIsKept();
+  TestDistinguishSubtlyDifferentMatrices();
+  EXPECT(g_live_allocations == 0);  // every cache freed what it allocated
+  if (g_failures) {
+    std::fprintf(stderr, "%d failure(s)\n", g_failures);
+    return 1;
+  }
+  std::printf("prepacked_cache_test: all passed\n");
+  return 0;
+}

@@ -1,0 +1,136 @@
+"""CPU-only checks of the host side: the library loads and exports every symbol
+the C header declares, the prepacked cache follows the reference's known
+answers, the ruy:: headers accept the reference's own example programs, and
+the Python mirror has the reference's defaults. No device computation here."""
+import ctypes as C
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ruy_amd", "c_api.h")
+LIB = os.path.join(ROOT, "ruy_amd", "libruy_amd.so")
+REFERENCE = "/root/reference"
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return sorted(set(re.findall(r"RUYAMD_API\s+[^;(]*?\b(ruyamd_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(LIB), "build the library first: python -m ruy_amd.build"
+    lib = C.CDLL(LIB)
+    names = declared_symbols()
+    assert len(names) >= 25
+    for name in names:
+        assert hasattr(lib, name), "libruy_amd.so lacks %s" % name
+    lib.ruyamd_version.restype = C.c_char_p
+    assert b"gfx950" in lib.ruyamd_version()
+
+
+def test_python_binding_covers_the_header():
+    from ruy_amd import _capi
+    assert sorted(_capi.PROTOTYPES) == declared_symbols()
+
+
+def test_struct_layouts_match_the_header():
+    """ctypes mirrors vs the C compiler's view of ruyamd_mat / ruyamd_mul_params."""
+    from ruy_amd import _structs as S
+    src = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "ruy_amd/c_api.h"
+int main(void) {
+  printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(ruyamd_mat), offsetof(ruyamd_mat, rows),
+         offsetof(ruyamd_mat, zero_point), offsetof(ruyamd_mat, order), offsetof(ruyamd_mat, cache_policy),
+         sizeof(ruyamd_mul_params), offsetof(ruyamd_mul_params, clamp_min),
+         offsetof(ruyamd_mul_params, accum_dtype));
+  return 0;
+}'''
+    work = os.path.join(ROOT, "tests", "cpp", "_layout_probe")
+    with open(work + ".c", "w") as f:
+        f.write(src)
+    try:
+        subprocess.check_call(["gcc", "-I" + os.path.join(ROOT, "include"), work + ".c", "-o", work])
+        got = [int(x) for x in subprocess.check_output([work]).split()]
+    finally:
+        for ext in ("", ".c"):
+            if os.path.exists(work + ext):
+                os.remove(work + ext)
+    want = [C.sizeof(S.Mat), S.Mat.rows.offset, S.Mat.zero_point.offset, S.Mat.order.offset,
+            S.Mat.cache_policy.offset, C.sizeof(S.MulParamsStruct),
+            S.MulParamsStruct.clamp_min.offset, S.MulParamsStruct.accum_dtype.offset]
+    assert got == want
+
+
+def test_prepacked_cache_known_answers():
+    """ruy/prepacked_cache_test.cc:54-227 restated over the host-side cache class."""
+    exe = os.path.join(ROOT, "tests", "cpp", "prepacked_cache_test")
+    subprocess.check_call(["g++", "-std=c++17", "-I" + os.path.join(ROOT, "ruy_amd", "csrc"),
+                           exe + ".cc", os.path.join(ROOT, "ruy_amd", "csrc", "prepacked_cache.cc"),
+                           "-o", exe])
+    out = subprocess.check_output([exe]).decode()
+    assert "all passed" in out
+
+
+@pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "example")),
+                    reason="reference tree not present")
+@pytest.mark.parametrize("std", ["c++14", "c++17"])
+def test_reference_examples_compile_against_our_headers(std, tmp_path):
+    """The reference's two example programs must build unchanged: that is the
+    source-level drop-in claim. (Running them needs a GPU; the same cases are
+    executed by tests/cpp/api_test.cc.)"""
+    for name in ("example.cc", "parametrized_example.cc"):
+        obj = str(tmp_path / (name + ".o"))
+        subprocess.check_call(["g++", "-std=" + std, "-I" + os.path.join(ROOT, "include"), "-c",
+                               os.path.join(REFERENCE, "example", name), "-o", obj])
+        exe = str(tmp_path / name.replace(".cc", ""))
+        subprocess.check_call(["g++", obj, "-L" + os.path.join(ROOT, "ruy_amd"), "-lruy_amd", "-o", exe])
+
+
+def test_python_mirror_defaults():
+    """ruy/mul_params_test.cc:26-72 and ruy/matrix_test.cc on the Python mirror."""
+    from ruy_amd import _structs as S
+    from ruy_amd import api
+    p = api.MulParams(S.I32, S.I8)
+    assert p.bias is None
+    assert p.multiplier_fixedpoint() == 0 and p.multiplier_exponent() == 0
+    assert p.multiplier_fixedpoint_perchannel() is None
+    assert (p.clamp_min, p.clamp_max) == (-128, 127)
+    assert p.channel_dimension == api.ChannelDimension.kRow
+    assert p.perchannel_buffers_capacity_rounding() == 1
+    p.set_multiplier_fixedpoint(123)
+    p.set_multiplier_exponent(4)
+    p.set_perchannel_buffers_capacity_rounding(8)
+    assert (p.multiplier_fixedpoint(), p.multiplier_exponent()) == (123, 4)
+    assert p.perchannel_buffers_capacity_rounding() == 8
+    p.set_multiplier_fixedpoint(0)
+    p.set_multiplier_exponent(0)
+    p.set_multiplier_fixedpoint_perchannel([1])
+    p.set_multiplier_exponent_perchannel([1])
+    assert p.multiplier_fixedpoint() == 0 and p.multiplier_fixedpoint_perchannel() == [1]
+    f = api.MulParams(S.F32, S.F32)
+    assert f.clamp_min == float("-inf") and f.clamp_max == float("inf")
+    with pytest.raises(ValueError):
+        api.MulParams(S.F32, S.I8)
+    with pytest.raises(ValueError):
+        api.MulParams(S.I32, S.F32)
+    lay = api.make_simple_layout(3, 5, api.Order.kRowMajor)
+    assert lay.stride == 5 and api.offset(lay, 2, 1) == 11
+    lay = api.make_simple_layout(3, 5, api.Order.kColMajor)
+    assert lay.stride == 3 and api.offset(lay, 2, 1) == 5
+    m = api.Matrix(S.U8)
+    assert m.zero_point == 0 and m.cache_policy == api.CachePolicy.kNeverCache
+
+
+def test_context_creation_fails_loudly_without_a_gpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from ruy_amd import api
+    with pytest.raises(api.RuyAmdError):
+        api.Context()
