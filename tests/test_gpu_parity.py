@@ -187,6 +187,21 @@ def test_rejects_what_the_reference_forbids(device_ctx):
     assert device_ctx.last_used_path() == api.Path.kGfx950
 
 
+def test_golden_fixture_on_device(device_ctx):
+    """Device results against the committed outputs of the stock reference
+    library (tests/golden/stock_ruy_golden.npz)."""
+    import device_runner as D
+    import golden_cases
+    for p, want in golden_cases.load():
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        if p.dst.dtype in (S.F32, S.F64):
+            g = O.dense_of(p, got).astype(np.float64)
+            w = O.dense_of(p, want).astype(np.float64)
+            assert np.linalg.norm(g - w) <= REL_FROBENIUS_TOL * max(np.linalg.norm(w), 1e-30), p.name
+        else:
+            assert (O.dense_of(p, got) == O.dense_of(p, want)).all(), p.name
+
+
 CONFIG_CASES = [
     ("C1 int8 256^3", lambda: W.config_int8_gemm(256)),
     ("C2 fp32 1024^3", lambda: W.config_f32_gemm(1024)),
@@ -208,3 +223,166 @@ def test_benchmark_configurations(device_ctx, name, make):
     got, want = run_both(device_ctx, p)
     compare(p, got, want)
     announce(name, "kernel:", device_ctx.last_kernel_name())
+
+
+def _sample_block(problem, got_storage, rows, cols):
+    """Checker result for the (rows x cols) sub-block of `problem` (all of the
+    depth), next to the same elements of the device result."""
+    l = problem.lhs.dense()[rows, :]
+    r = problem.rhs.dense()[:, cols]
+    lhs = W.HostMatrix(problem.lhs.dtype, len(rows), problem.K, S.ORDER_ROW_MAJOR,
+                       zero_point=problem.lhs.zero_point)
+    lhs.set_values(l)
+    rhs = W.HostMatrix(problem.rhs.dtype, problem.K, len(cols), S.ORDER_COL_MAJOR,
+                       zero_point=problem.rhs.zero_point)
+    rhs.set_values(r)
+    dst = W.HostMatrix(problem.dst.dtype, len(rows), len(cols), S.ORDER_COL_MAJOR,
+                       zero_point=problem.dst.zero_point)
+    ch_row = problem.channel_dimension == S.CHANNEL_ROW
+    pick = rows if ch_row else cols
+    sub = W.Problem("sample", lhs, rhs, dst, problem.accum_dtype,
+                    bias=None if problem.bias is None else np.ascontiguousarray(problem.bias[pick]),
+                    multiplier_fixedpoint=problem.multiplier_fixedpoint,
+                    multiplier_exponent=problem.multiplier_exponent,
+                    multiplier_fixedpoint_perchannel=None if problem.multiplier_fixedpoint_perchannel is None
+                    else np.ascontiguousarray(problem.multiplier_fixedpoint_perchannel[pick]),
+                    multiplier_exponent_perchannel=None if problem.multiplier_exponent_perchannel is None
+                    else np.ascontiguousarray(problem.multiplier_exponent_perchannel[pick]),
+                    clamp_min=problem.clamp_min, clamp_max=problem.clamp_max,
+                    channel_dimension=problem.channel_dimension)
+    want = O.dense_of(sub, O.oracle_mul(sub))
+    got = O.dense_of(problem, got_storage)[np.ix_(rows, cols)]
+    return got, want
+
+
+def test_full_size_int8_gemm_8192(device_ctx):
+    """The headline shape, M=N=K=8192. The checker cannot do 5.5e11 MACs in
+    seconds, so: (1) raw int32 accumulators are verified through a checksum of
+    every element - column sums and row sums of dst against (sum of lhs rows) x
+    rhs and lhs x (sum of rhs columns), exact modulo 2^32; (2) the requantized
+    int8 result is compared bit for bit with the checker on a random 192 x 192
+    sample of rows and columns plus the four tile-corner regions."""
+    import device_runner as D
+    n = 8192
+    p = W.config_int8_gemm(n, config_id=6)
+    announce("T requantized", n)
+    got = D.device_mul(device_ctx, p, dst_fill=0)
+    assert device_ctx.last_kernel_name() == "i8_mfma"
+    rng = np.random.default_rng(77)
+    rows = np.sort(np.concatenate([rng.choice(n, 160, replace=False), np.arange(0, 16), np.arange(n - 16, n)]))
+    rows = np.unique(rows)
+    cols = np.unique(np.concatenate([rng.choice(n, 160, replace=False), np.arange(250, 262), np.arange(n - 16, n)]))
+    g, w = _sample_block(p, got, rows, cols)
+    assert (g == w).all(), "%d mismatches in the sampled block" % (g != w).sum()
+
+    announce("T raw int32 checksum", n)
+    raw = W.Problem("raw", p.lhs, p.rhs, W.HostMatrix(S.I32, n, n, S.ORDER_COL_MAJOR), S.I32, bias=p.bias)
+    got = O.dense_of(raw, D.device_mul(device_ctx, raw, dst_fill=0)).astype(np.int64)
+    L = p.lhs.dense().astype(np.int64) - p.lhs.zero_point
+    R = p.rhs.dense().astype(np.int64) - p.rhs.zero_point
+    bias = p.bias.astype(np.int64)
+    col_sums = (L.sum(axis=0) @ R + bias.sum()) % 2**32           # sum over rows of each column
+    row_sums = (L @ R.sum(axis=1) + n * bias) % 2**32              # sum over columns of each row
+    assert ((got.sum(axis=0) % 2**32) == col_sums).all()
+    assert ((got.sum(axis=1) % 2**32) == row_sums).all()
+
+
+@pytest.mark.parametrize("cols,requant", [(1, False), (4, False), (8, False), (1, True)])
+def test_full_size_int8_gemv_16384(device_ctx, cols, requant):
+    """The skinny shape M=K=16384 at full size, LHS through the prepacked cache
+    (called twice: the second call is served from the cache and must agree, the
+    reference's own caching check, ruy/test.h:733-737). Compared bit for bit
+    with the checker on every element."""
+    import device_runner as D
+    n = 16384
+    p = W.config_int8_gemv(n, cols, requant=requant)
+    announce("GEMV", n, cols, requant)
+    want = O.oracle_mul(p)
+    device_ctx.set_cache_max_bytes(n * n + 4 * n + 4096)
+    try:
+        dp = D.DeviceProblem(p, dst_fill=0)
+        dp.run(device_ctx)
+        assert device_ctx.last_kernel_name() == "i8_gemv"
+        assert device_ctx.cache_matrix_count() == 1
+        assert device_ctx.cache_buffers_bytes() == n * n + 4 * n
+        first = dp.result().copy()
+        dp.run(device_ctx)
+        assert device_ctx.cache_matrix_count() == 1
+        second = dp.result()
+        assert (first == want).all()
+        assert (second == want).all()
+    finally:
+        device_ctx.set_cache_max_bytes(1 << 28)
+
+
+def test_prepacked_cache_through_mul(device_ctx):
+    """Cache behaviour seen through Mul: policies (ruy/prepare_packed_matrices.cc
+    :38-66 with a kernel width of 8), byte accounting, distinct keys per source
+    pointer and zero point, least-recently-used ejection, clear."""
+    import device_runner as D
+    from ruy_amd import api
+    ctx = device_ctx
+    ctx.clear_prepacked_cache()
+    rng = np.random.default_rng(31)
+
+    def prob(M, K, N, policy, zp=0):
+        p = W.random_problem(rng, S.I8, S.I8, S.I32, S.I32, M, K, N, 1, 0, 0)
+        p.lhs.cache_policy = policy
+        p.lhs.zero_point = zp
+        return p
+
+    for policy, n_cols, expect in [(S.CACHE_NEVER, 1, 0), (S.CACHE_IF_LARGE_SPEEDUP, 8, 1),
+                                   (S.CACHE_IF_LARGE_SPEEDUP, 9, 0), (S.CACHE_IF_SIGNIFICANT_SPEEDUP, 32, 1),
+                                   (S.CACHE_IF_SIGNIFICANT_SPEEDUP, 33, 0), (S.CACHE_ALWAYS, 100, 1)]:
+        ctx.clear_prepacked_cache()
+        p = prob(48, 64, n_cols, policy)
+        got, want = run_both(ctx, p)
+        compare(p, got, want)
+        assert ctx.cache_matrix_count() == expect, (policy, n_cols)
+        if expect:
+            assert ctx.cache_buffers_bytes() == 48 * 64 + 48 * 4  # packed int8 + int32 sums
+    # same device buffer, different zero point -> a second entry; results stay right
+    ctx.clear_prepacked_cache()
+    p = prob(40, 80, 4, S.CACHE_ALWAYS, zp=3)
+    dp = D.DeviceProblem(p, dst_fill=0)
+    dp.run(ctx)
+    assert ctx.cache_matrix_count() == 1
+    p.lhs.zero_point = 5
+    dp2 = D.DeviceProblem(p, dst_fill=0)
+    dp2.lhs_s.data = dp.lhs_s.data  # identical source pointer
+    dp2.run(ctx)
+    assert ctx.cache_matrix_count() == 2
+    assert (dp2.result() == O.oracle_mul(p)).all()
+    # ejection: budget for two entries of 40*80+160 bytes, insert three
+    ctx.set_cache_max_bytes(2 * (40 * 80 + 160))
+    try:
+        dps = []
+        for _ in range(3):
+            q = prob(40, 80, 4, S.CACHE_ALWAYS)
+            d = D.DeviceProblem(q, dst_fill=0)
+            d.run(ctx)
+            assert (d.result() == O.oracle_mul(q)).all()
+            dps.append(d)
+        assert ctx.cache_matrix_count() == 2
+        dps[2].run(ctx)
+        dps[1].run(ctx)
+        assert ctx.cache_matrix_count() == 2  # both hits
+        dps[0].run(ctx)                        # re-inserted, ejecting the oldest (2)
+        assert ctx.cache_matrix_count() == 2
+        assert (dps[0].result() == O.oracle_mul(dps[0].problem)).all()
+    finally:
+        ctx.set_cache_max_bytes(1 << 28)
+    assert ctx.cache_matrix_count() == 0
+
+
+def test_tuned_kernels_are_the_ones_that_run(device_ctx):
+    """Each benchmark configuration must be served by its tuned kernel, not by
+    the generic one."""
+    import device_runner as D
+    expect = [(W.config_int8_gemm(256), "i8_mfma"), (W.config_f32_gemm(256), "f32_mfma"),
+              (W.config_int8_perchannel_conv(256, 256, 196), "i8_mfma"),
+              (W.config_int8_int16(256, 256, 64), "i8i16_mfma"), (W.config_int8_gemv(512, 4), "i8_gemv")]
+    for p, kernel in expect:
+        D.device_mul(device_ctx, p)
+        assert device_ctx.last_kernel_name() == kernel, p.name
+    device_ctx.clear_prepacked_cache()

@@ -365,6 +365,21 @@ def test_overflow_flag():
     assert O.oracle_mul(p, want_overflow=True)[1] is True
 
 
+def test_golden_fixture_from_stock_reference():
+    """tests/golden/stock_ruy_golden.npz holds ruy::ReferenceMul outputs written
+    by tests/golden/make_stock_ruy_golden.py; they travel where the reference
+    library cannot."""
+    import golden_cases
+    loaded = golden_cases.load()
+    assert len(loaded) >= 100
+    for p, want in loaded:
+        got = O.oracle_mul(p)
+        if p.dst.dtype in (S.F32, S.F64):
+            assert (got == want).all(), p.name  # same ascending-k scalar loop
+        else:
+            assert (got == want).all(), p.name
+
+
 # ---------------------------------------------------------------------------
 # Against the stock reference library, when built.
 
