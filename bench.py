@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the int8 GEMM")
     ap.add_argument("--gemv-size", type=int, default=16384, help="M=K of the int8 GEMV")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 256 MiB device copies, so that a counter run "
+                         "(FETCH_SIZE / WRITE_SIZE) has a dispatch of known traffic to scale by")
     return ap.parse_args()
 
 
@@ -59,13 +62,18 @@ def time_steps(run, steps, warmup, ctx):
     torch.cuda.synchronize()
     ctx.kernel_timing()  # drop the warm-up launches
     torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()
     for _ in range(steps):
         run()
+    e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    region_ms = e0.elapsed_time(e1) / steps  # events on the launch stream around all K steps
     kernel_ms, launches = ctx.kernel_timing()
-    return wall / steps, (kernel_ms / launches if launches else None)
+    return wall / steps, (kernel_ms / launches if launches else None), region_ms
 
 
 def load_traffic(name):
@@ -141,7 +149,7 @@ def bench_gemm(ctx, args):
     dp = device_problem(problem)
     dp.run(ctx)
     kernel = ctx.last_kernel_name()
-    step_s, kernel_ms = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx)
+    step_s, kernel_ms, _ = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx)
     ops = float(problem.ops())
     out = {
         "value": ops / step_s / 1e12,
@@ -182,7 +190,13 @@ def bench_gemv(ctx, args):
         dps[state["i"] % rotate].run(ctx)
         state["i"] += 1
 
-    step_s, kernel_ms = time_steps(run, args.steps * 4, args.warmup * 4, ctx)
+    # A step is exactly one kernel here (operand and sums come from the cache),
+    # and that kernel is short enough for a per-launch event pair to add ~10 %
+    # to it; so per-launch events are switched off and its duration is taken
+    # from one event pair around all launches of the timed region.
+    ctx.set_kernel_timing(False)
+    step_s, _, kernel_ms = time_steps(run, args.steps * 4, args.warmup * 4, ctx)
+    ctx.set_kernel_timing(True)
     nbytes = float(problems[0].algorithmic_bytes())
     out = {
         "metric": "int8 GEMV M=K=%d N=1 algorithmic HBM GB/s" % n,
@@ -261,6 +275,13 @@ def main():
                 line["cpu_baseline"] = gv["cpu_baseline"]
         else:
             line["gemv"] = gv
+    if args.copy_calibration:
+        a = torch.full((256 << 20,), 3, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        line["copy_calibration"] = {"bytes_read": 256 << 20, "bytes_written": 256 << 20, "copies": 3}
     ctx.close()
     print(json.dumps(line))
 
