@@ -386,3 +386,21 @@ def test_tuned_kernels_are_the_ones_that_run(device_ctx):
         D.device_mul(device_ctx, p)
         assert device_ctx.last_kernel_name() == kernel, p.name
     device_ctx.clear_prepacked_cache()
+
+
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I16),
+                                 (S.I8, S.U8, S.I32, S.I32)], ids=cases.tuple_name)
+def test_skinny_shapes_both_orientations(device_ctx, tup):
+    """Narrow side on the right (matrix x few vectors) and on the left (few
+    vectors x matrix), depths that are not multiples of the 1024-byte step,
+    row counts that do not fill the last workgroup: both skinny kernels."""
+    rng = np.random.default_rng(123)
+    for shape in [(300, 1500, 5), (5, 1500, 300), (1031, 2048, 8), (8, 4100, 513), (257, 1024, 2),
+                  (2, 1100, 260), (1000, 3000, 3), (64, 9000, 7), (4, 64, 4), (3, 20000, 1)]:
+        for orders in (cases.RCC, cases.ALL_ORDERS[int(rng.integers(8))]):
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=bool(rng.integers(2)),
+                                 name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
+            assert device_ctx.last_kernel_name() == "i8_gemv"
