@@ -161,7 +161,6 @@ int ruyamd_ctx_synchronize(ruyamd_ctx* ctx) {
     ctx->last_error = "hipStreamSynchronize failed";
     return RUYAMD_E_HIP;
   }
-  ctx->pending_async = false;
   return RUYAMD_OK;
 }
 

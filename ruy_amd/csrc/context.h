@@ -48,7 +48,6 @@ struct ruyamd_ctx {
   hipStream_t own_stream = nullptr;
   hipStream_t stream = nullptr;
   bool synchronous = true;
-  bool pending_async = false;  // work enqueued by an asynchronous call
   int last_used_path = RUYAMD_PATH_NONE;
   int runtime_enabled_paths = RUYAMD_PATH_NONE;  // kNone = not decided yet
   int max_num_threads = 1;

@@ -65,6 +65,9 @@ struct GemvI8Args {
 };
 
 hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args);
+// fp32 version: the same argument block with K, ld_wide and ld_narrow counted
+// in bytes of fp32 data, an fp32 destination and the float write-back.
+hipError_t LaunchGemvF32(hipStream_t stream, const GemvI8Args& args);
 
 // A matrix seen as `count` depth-vectors of length K: vector c, depth k is
 // data[c * stride_c + k * stride_k] (elements of `dtype`, uint8 or int8).

@@ -163,11 +163,10 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
   if (hipSetDevice(ctx->device) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "hipSetDevice failed");
   if (dst->rows == 0 || dst->cols == 0) return RUYAMD_OK;
 
-  // The previous call's scratch may still be in use by an asynchronous launch.
-  if (ctx->pending_async && ctx->workspace.capacity() > 0) {
-    // Stream order protects reuse: every user of the scratch was enqueued on
-    // ctx->stream before anything this call enqueues.
-  }
+  // Scratch of the previous call is reused. If that call was asynchronous its
+  // kernels may not have run yet, but everything that touches the scratch -
+  // theirs and ours - is enqueued on ctx->stream, so stream order keeps the
+  // uses apart.
   ctx->workspace.Reset();
 
   bool staged = false, ok = true;
@@ -244,9 +243,6 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
   if (ctx->synchronous || staged) {
     if (hipStreamSynchronize(ctx->stream) != hipSuccess)
       return Fail(ctx, RUYAMD_E_HIP, std::string("kernel execution failed: ") + hipGetErrorString(hipGetLastError()));
-    ctx->pending_async = false;
-  } else {
-    ctx->pending_async = true;
   }
   return RUYAMD_OK;
 }

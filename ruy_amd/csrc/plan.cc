@@ -324,6 +324,33 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   OperandF32 a, b;
   if (int rc = PrepareOperandF32(ctx, call, 0, call->lhs_cache_policy, call->lhs_src_key, N, &a, err)) return rc;
   if (int rc = PrepareOperandF32(ctx, call, 1, call->rhs_cache_policy, call->rhs_src_key, M, &b, err)) return rc;
+  if (N <= kSkinnyWidth || M <= kSkinnyWidth) {
+    // Bandwidth-bound shapes: stream the wide side once, no matrix instructions.
+    GemvI8Args g;
+    g.swapped = !(N <= kSkinnyWidth && (M > kSkinnyWidth || M >= N));
+    const OperandF32& wide = g.swapped ? b : a;
+    const OperandF32& narrow = g.swapped ? a : b;
+    g.wide = reinterpret_cast<const int8_t*>(wide.data);
+    g.narrow = reinterpret_cast<const int8_t*>(narrow.data);
+    g.wide_bytes = wide.bytes;
+    g.narrow_bytes = narrow.bytes;
+    g.ld_wide = wide.ld * 4;
+    g.ld_narrow = narrow.ld * 4;
+    g.rows = g.swapped ? N : M;
+    g.narrow_count = g.swapped ? M : N;
+    g.K = RoundUp(K, 4) * 4;
+    g.ep = call->ep;
+    g.dst = call->dst;
+    const bool timed = ctx->TimingBegin();
+    const hipError_t launched = LaunchGemvF32(ctx->stream, g);
+    if (timed) ctx->TimingEnd();
+    if (launched != hipSuccess) {
+      *err = "fp32 skinny kernel launch failed";
+      return RUYAMD_E_HIP;
+    }
+    ctx->last_kernel = RUYAMD_KERNEL_F32_GEMV;
+    return RUYAMD_OK;
+  }
   GemmArgs args;
   args.k_bytes = RoundUp(K, 4) * 4;
   const bool swap = SetupDestination(*call, &args);
@@ -429,7 +456,18 @@ int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
 int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const DevMat& lhs = call->lhs;
   const DevMat& rhs = call->rhs;
-  if (!ctx->force_generic) {
+  // The tuned kernels address operands through 32-bit buffer offsets; anything
+  // of 2 GiB or more goes to the generic kernel, which uses 64-bit offsets.
+  auto extent_bytes = [](const DevMat& m) {
+    if (m.rows == 0 || m.cols == 0) return uint64_t(0);
+    return (uint64_t(m.rows - 1) * uint64_t(m.rs) + uint64_t(m.cols - 1) * uint64_t(m.cs) + 1) *
+           uint64_t(DtypeSize(m.dtype));
+  };
+  const uint64_t kLimit = (uint64_t(1) << 31) - (uint64_t(1) << 20);
+  const bool huge = extent_bytes(lhs) >= kLimit || extent_bytes(rhs) >= kLimit ||
+                    uint64_t(lhs.rows) * (uint64_t(lhs.cols) + 16) * DtypeSize(lhs.dtype) >= kLimit ||
+                    uint64_t(rhs.cols) * (uint64_t(rhs.rows) + 16) * DtypeSize(rhs.dtype) >= kLimit / 2;
+  if (!ctx->force_generic && !huge) {
     if (Is8Bit(lhs.dtype) && Is8Bit(rhs.dtype)) return RunInt8(ctx, call, err);
     {
       // The int8 side must run along the destination's contiguous dimension.

@@ -389,7 +389,8 @@ def test_tuned_kernels_are_the_ones_that_run(device_ctx):
 
 
 @pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I16),
-                                 (S.I8, S.U8, S.I32, S.I32)], ids=cases.tuple_name)
+                                 (S.I8, S.U8, S.I32, S.I32), (S.F32, S.F32, S.F32, S.F32)],
+                         ids=cases.tuple_name)
 def test_skinny_shapes_both_orientations(device_ctx, tup):
     """Narrow side on the right (matrix x few vectors) and on the left (few
     vectors x matrix), depths that are not multiples of the 1024-byte step,
@@ -403,4 +404,4 @@ def test_skinny_shapes_both_orientations(device_ctx, tup):
             announce(p.name)
             got, want = run_both(device_ctx, p)
             compare(p, got, want)
-            assert device_ctx.last_kernel_name() == "i8_gemv"
+            assert device_ctx.last_kernel_name() == ("f32_gemv" if tup[0] == S.F32 else "i8_gemv")
