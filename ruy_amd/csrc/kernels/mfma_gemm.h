@@ -38,6 +38,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "../epilogue.h"
 #include "../internal.h"
 #include "gemm_i8.h"
@@ -77,6 +79,18 @@ __device__ __forceinline__ void LoadToLds16(uint32_t lds_base, uint32_t voffset,
       "buffer_load_dwordx4 %1, %2, 0 offen lds"
       :
       : "s"(lds_base), "v"(voffset), "s"(rsrc)
+      : "memory");
+}
+
+// Same, with a wave-uniform byte offset added to every lane's address (it
+// takes no part in the bounds check, which looks at `voffset` only).
+__device__ __forceinline__ void LoadToLds16(uint32_t lds_base, uint32_t voffset, uint32_t soffset, v4i rsrc) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
       : "memory");
 }
 
@@ -207,6 +221,19 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
       LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, off, b_rsrc);
     }
   };
+  // The same for a ring step that lies entirely inside the depth: no
+  // per-granule test, and the step's depth offset travels as the instruction's
+  // scalar offset, so nothing but the load itself is issued.
+  auto issue_one_full = [&](int kt, int n) {
+    const uint32_t kbase = kt * kBK;
+    const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
+    if (n < C::kALoads) {
+      LoadToLds16(stage + (wave * C::kALoads + n) * 1024, a_goff[n], kbase, a_rsrc);
+    } else {
+      const int i = n - C::kALoads;
+      LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, b_goff[i], kbase, b_rsrc);
+    }
+  };
   auto issue = [&](int kt) {
 #pragma unroll
     for (int n = 0; n < C::kLoadsPerStage; ++n) issue_one(kt, n);
@@ -237,6 +264,14 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
     for (int j = 0; j < WN; ++j)
       f.b[j] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * 32 * kBK);
   };
+  // Fragment number r (0 .. WM+WN-1: the A fragments, then the B fragments).
+  auto read_one = [&](int kt, int ks, int r, Frags& f) {
+    const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
+    if (r < WM)
+      f.a[r] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + r * 32 * kBK);
+    else
+      f.b[r - WM] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + (r - WM) * 32 * kBK);
+  };
 
   typename Traits::Acc acc[WM][WN];
 #pragma unroll
@@ -245,12 +280,41 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
     for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-  auto mma = [&](const Frags& f) {
+
+  // One depth sub-step: the WM*WN matrix instructions on `cur`, with the LDS
+  // reads of the next fragments (depth sub-step ks_next of ring step kt_next)
+  // and, if kt_dma >= 0, the direct-to-LDS loads of ring step kt_dma dealt out
+  // one at a time between them. A matrix instruction occupies its pipe for 32
+  // cycles but issues in a few, so whatever is issued right behind it is free;
+  // a block of loads issued back to back instead would stall the pipe.
+  constexpr int kMmas = WM * WN;
+  constexpr int kFrags = WM + WN;
+  // The fragment reads go behind the first matrix instructions of the
+  // sub-step, so that they have landed well before the next sub-step starts.
+  constexpr int kReadSlots = kMmas < kFrags ? kMmas : kFrags;
+  auto sub_step = [&](const Frags& cur, Frags& next, int kt_next, int ks_next, int kt_dma,
+                      auto dma_is_full_step) {
 #pragma unroll
-    for (int i = 0; i < WM; ++i)
+    for (int n = 0; n < kMmas; ++n) {
+      __builtin_amdgcn_sched_barrier(0);
+      Traits::Mma(cur.a[n / WN], cur.b[n % WN], acc[n / WN][n % WN]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (n < kReadSlots) {
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
-        Traits::Mma(f.a[i], f.b[j], acc[i][j]);
+        for (int r = n * kFrags / kReadSlots; r < (n + 1) * kFrags / kReadSlots; ++r)
+          read_one(kt_next, ks_next, r, next);
+      }
+      if (kt_dma >= 0) {
+#pragma unroll
+        for (int l = n * C::kLoadsPerStage / kMmas; l < (n + 1) * C::kLoadsPerStage / kMmas; ++l) {
+          if (decltype(dma_is_full_step)::value)
+            issue_one_full(kt_dma, l);
+          else
+            issue_one(kt_dma, l);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   const int k_tiles = (K + kBK - 1) / kBK;
@@ -268,36 +332,26 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   __syncthreads();
   Frags f[2];
   read_frags(0, 0, f[0]);
-  for (int kt = 0; kt < k_tiles; ++kt) {
+  auto ring_step = [&](int kt, auto dma_is_full_step) {
 #pragma unroll
     for (int ks = 0; ks < C::kKSteps; ++ks) {
       if (ks + 1 < C::kKSteps) {
-        read_frags(kt, ks + 1, f[(ks + 1) & 1]);
-        __builtin_amdgcn_sched_barrier(0);
-        mma(f[ks & 1]);
-        __builtin_amdgcn_sched_barrier(0);
+        sub_step(f[ks & 1], f[(ks + 1) & 1], kt, ks + 1, -1, dma_is_full_step);
       } else {
         WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
         __syncthreads();
-        read_frags(kt + 1, 0, f[0]);
-        // The loads of step kt+kStages are issued one at a time between the
-        // matrix instructions of this sub-step, so the matrix pipe keeps
-        // running while the addresses are generated.
-        const Frags& g = f[ks & 1];
-        constexpr int kMmas = WM * WN;
-#pragma unroll
-        for (int n = 0; n < kMmas; ++n) {
-          __builtin_amdgcn_sched_barrier(0);
-          Traits::Mma(g.a[n / WN], g.b[n % WN], acc[n / WN][n % WN]);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int l = n * C::kLoadsPerStage / kMmas; l < (n + 1) * C::kLoadsPerStage / kMmas; ++l)
-            issue_one(kt + C::kStages, l);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        sub_step(f[ks & 1], f[0], kt + 1, 0, kt + C::kStages, dma_is_full_step);
       }
     }
-  }
+  };
+  // While the step whose loads are being issued (kt + kStages) lies entirely
+  // inside the depth, the cheap form of the loads is used; the last few steps
+  // (a partial step and the ones past the end, which fetch zeros) take the
+  // bounds-tested form.
+  int kt = 0;
+  const int full_end = K / kBK - C::kStages;
+  for (; kt < full_end; ++kt) ring_step(kt, std::true_type());
+  for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type());
   WaitVmcnt<0>();
   __syncthreads();  // every wave is done with the operand ring
 
