@@ -223,6 +223,27 @@ def bench_gemv(ctx, args):
     return out
 
 
+def bench_other_configs(ctx, steps, warmup):
+    """Time (not roofline) of the remaining configurations: small or
+    latency-bound shapes whose gate is parity; reported for completeness."""
+    from ruy_amd import workloads as W
+    out = []
+    ctx.set_kernel_timing(False)  # a per-launch event pair would dominate these short steps
+    for name, problem in [("C1 int8 256^3", W.config_int8_gemm(256)),
+                          ("C2 fp32 1024^3", W.config_f32_gemm(1024)),
+                          ("C2 fp32 1024^3 relu6", W.config_f32_gemm(1024, relu6=True)),
+                          ("C3 int8 per-channel 1024x1024x196", W.config_int8_perchannel_conv()),
+                          ("C4 int8xint16 2048x2048x512", W.config_int8_int16())]:
+        dp = device_problem(problem)
+        dp.run(ctx)
+        kernel = ctx.last_kernel_name()
+        step_s, _, _ = time_steps(lambda: dp.run(ctx), steps, warmup, ctx)
+        out.append({"config": name, "kernel": kernel, "us_per_step": step_s * 1e6,
+                    "Top/s": problem.ops() / step_s / 1e12})
+    ctx.set_kernel_timing(True)
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -275,6 +296,8 @@ def main():
                 line["cpu_baseline"] = gv["cpu_baseline"]
         else:
             line["gemv"] = gv
+    if args.workload == "all":
+        line["other_configs"] = bench_other_configs(ctx, args.steps, args.warmup)
     if args.copy_calibration:
         a = torch.full((256 << 20,), 3, dtype=torch.uint8, device="cuda")
         b = torch.empty_like(a)

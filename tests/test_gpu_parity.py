@@ -405,3 +405,36 @@ def test_skinny_shapes_both_orientations(device_ctx, tup):
             got, want = run_both(device_ctx, p)
             compare(p, got, want)
             assert device_ctx.last_kernel_name() == ("f32_gemv" if tup[0] == S.F32 else "i8_gemv")
+
+
+def test_caller_stream_asynchronous_calls_and_kernel_timing(device_ctx):
+    """Device-side controls without a counterpart in the reference: launching on
+    a caller-owned stream, returning before completion, per-kernel timing."""
+    import torch
+    import device_runner as D
+    from ruy_amd import api
+    ctx = api.Context()
+    try:
+        stream = torch.cuda.Stream()
+        ctx.set_stream(stream.cuda_stream)
+        ctx.set_synchronous(False)
+        ctx.set_kernel_timing(True)
+        p = W.config_int8_gemm(512)
+        want = O.oracle_mul(p)
+        dp = D.DeviceProblem(p, dst_fill=0)
+        with torch.cuda.stream(stream):
+            for _ in range(5):
+                dp.run(ctx)
+            done = torch.cuda.Event()
+            done.record()
+        done.synchronize()
+        assert (dp.dst_t.cpu().numpy() == want).all()
+        ms, launches = ctx.kernel_timing()
+        assert launches == 5 and 0 < ms < 50
+        assert ctx.kernel_timing() == (0.0, 0)
+        # an asynchronous context still completes host-pointer calls before returning
+        got = D.host_pointer_mul(ctx, p, dst_fill=0)
+        assert (got == want).all()
+        ctx.synchronize()
+    finally:
+        ctx.close()
