@@ -11,6 +11,9 @@ _TORCH = {S.U8: torch.uint8, S.I8: torch.int8, S.I16: torch.int16, S.I32: torch.
           S.F32: torch.float32, S.F64: torch.float64}
 
 
+GUARD_ELEMENTS = 256
+
+
 def to_dev(arr):
     return torch.from_numpy(np.ascontiguousarray(arr)).cuda()
 
@@ -24,9 +27,16 @@ class DeviceProblem:
         self.lhs_t = to_dev(p.lhs.storage)
         self.rhs_t = to_dev(p.rhs.storage)
         d = p.dst
-        fill = np.full(max(d.n_storage, 1), 0, dtype=d.storage.dtype)
+        # The destination sits between two guard zones that must come back
+        # untouched (the idea of the reference's guard-page allocator,
+        # ruy/test.h:395-445, for a device buffer).
+        self.guard = GUARD_ELEMENTS
+        self.n_dst = max(d.n_storage, 1)
+        fill = np.full(self.n_dst + 2 * self.guard, 0, dtype=d.storage.dtype)
         fill.view(np.uint8)[:] = dst_fill
-        self.dst_t = to_dev(fill)
+        self.dst_fill = dst_fill
+        self.dst_all = to_dev(fill)
+        self.dst_t = self.dst_all[self.guard:self.guard + self.n_dst]
         self.bias_t = to_dev(p.bias) if p.bias is not None else None
         self.mf_t = self.me_t = None
         if p.multiplier_fixedpoint_perchannel is not None:
@@ -48,7 +58,10 @@ class DeviceProblem:
 
     def result(self):
         torch.cuda.synchronize()
-        return self.dst_t.cpu().numpy()
+        everything = self.dst_all.cpu().numpy()
+        guards = np.concatenate([everything[:self.guard], everything[self.guard + self.n_dst:]])
+        assert (guards.view(np.uint8) == self.dst_fill).all(), "write outside the destination buffer"
+        return everything[self.guard:self.guard + self.n_dst].copy()
 
 
 def device_mul(ctx, problem, dst_fill=0x5A):

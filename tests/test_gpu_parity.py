@@ -438,3 +438,21 @@ def test_caller_stream_asynchronous_calls_and_kernel_timing(device_ctx):
         ctx.synchronize()
     finally:
         ctx.close()
+
+
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.U8),
+                                 (S.F32, S.F32, S.F32, S.F32), (S.I8, S.I16, S.I32, S.I16),
+                                 (S.I8, S.I8, S.I32, S.I32), (S.U8, S.U8, S.I32, S.I16)],
+                         ids=cases.tuple_name)
+def test_reference_slow_shape_list(device_ctx, tup):
+    """The reference's test_slow shapes (ruy/test_slow.cc:29-68): big narrow
+    products incl. 7x45984x5 (sums that leave the int16 range), big shallow
+    ones, power-of-two depths 1024/2048/4096 and GEMV sizes 1025/1409."""
+    rng = np.random.default_rng(777 + cases.TYPE_TUPLES.index(tup))
+    for shape in cases.SLOW_SHAPES:
+        for orders, strided in ((cases.RCC, False), (cases.ALL_ORDERS[int(rng.integers(8))], True)):
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=strided,
+                                 name="%s %s %s strided=%s" % (cases.tuple_name(tup), shape, orders, strided))
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
