@@ -19,26 +19,26 @@ enum class Path : std::uint8_t {
   kGfx950 = 0x10,
 };
 
-inline constexpr Path operator|(Path p, Path q) {
-  return static_cast<Path>(static_cast<std::uint32_t>(p) | static_cast<std::uint32_t>(q));
-}
-inline constexpr Path operator&(Path p, Path q) {
-  return static_cast<Path>(static_cast<std::uint32_t>(p) & static_cast<std::uint32_t>(q));
-}
-inline constexpr Path operator^(Path p, Path q) {
-  return static_cast<Path>(static_cast<std::uint32_t>(p) ^ static_cast<std::uint32_t>(q));
-}
-inline constexpr Path operator~(Path p) { return static_cast<Path>(~static_cast<std::uint32_t>(p)); }
-inline constexpr bool Disjoint(Path p, Path q) { return (p & q) == Path::kNone; }
+namespace detail {
+constexpr std::uint32_t PathBits(Path p) { return static_cast<std::uint32_t>(p); }
+constexpr Path PathFromBits(std::uint32_t bits) { return static_cast<Path>(bits); }
+}  // namespace detail
 
+// Path values are bit masks; the usual set operations apply.
+constexpr Path operator|(Path a, Path b) { return detail::PathFromBits(detail::PathBits(a) | detail::PathBits(b)); }
+constexpr Path operator&(Path a, Path b) { return detail::PathFromBits(detail::PathBits(a) & detail::PathBits(b)); }
+constexpr Path operator^(Path a, Path b) { return detail::PathFromBits(detail::PathBits(a) ^ detail::PathBits(b)); }
+constexpr Path operator~(Path a) { return detail::PathFromBits(~detail::PathBits(a)); }
+constexpr bool Disjoint(Path a, Path b) { return (detail::PathBits(a) & detail::PathBits(b)) == 0; }
+
+// The highest bit set in `mask` (Path::kNone for an empty mask).
 inline Path GetMostSignificantPath(Path mask) {
-  std::uint32_t m = static_cast<std::uint32_t>(mask), top = 0;
-  for (std::uint32_t bit = 0x80; bit; bit >>= 1)
-    if (m & bit) {
-      top = bit;
-      break;
-    }
-  return static_cast<Path>(top);
+  std::uint32_t bits = detail::PathBits(mask) & 0xffu, top = 0;
+  while (bits) {
+    top = bits & (~bits + 1u);  // lowest set bit; the last one standing is the highest
+    bits &= bits - 1u;
+  }
+  return detail::PathFromBits(top);
 }
 
 constexpr Path kNonArchPaths = Path::kStandardCpp;

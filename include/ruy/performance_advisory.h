@@ -8,11 +8,12 @@ namespace ruy {
 
 enum class PerformanceAdvisory { kNone = 0, kReallocatedPerChannelBuffer = 0x1 };
 
-inline constexpr PerformanceAdvisory operator|(PerformanceAdvisory p, PerformanceAdvisory q) {
-  return static_cast<PerformanceAdvisory>(static_cast<int>(p) | static_cast<int>(q));
+// Advisories are bit flags.
+constexpr PerformanceAdvisory operator|(PerformanceAdvisory a, PerformanceAdvisory b) {
+  return PerformanceAdvisory(int(a) | int(b));
 }
-inline constexpr PerformanceAdvisory operator&(PerformanceAdvisory p, PerformanceAdvisory q) {
-  return static_cast<PerformanceAdvisory>(static_cast<int>(p) & static_cast<int>(q));
+constexpr PerformanceAdvisory operator&(PerformanceAdvisory a, PerformanceAdvisory b) {
+  return PerformanceAdvisory(int(a) & int(b));
 }
 
 }  // namespace ruy
