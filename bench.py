@@ -278,10 +278,42 @@ def bench_other_configs(ctx, steps, warmup):
         dp.run(ctx)
         kernel = ctx.last_kernel_name()
         step_s, _, _ = time_steps(lambda: dp.run(ctx), steps, warmup, ctx)
-        out.append({"config": name, "kernel": kernel, "us_per_step": step_s * 1e6,
-                    "Top/s": problem.ops() / step_s / 1e12})
+        entry = {"config": name, "kernel": kernel, "us_per_step": step_s * 1e6,
+                 "Top/s": problem.ops() / step_s / 1e12}
+        if problem.ops() < 1e9:
+            entry["us_per_step_graph"] = graph_replay_us(ctx, dp)
+        out.append(entry)
     ctx.set_kernel_timing(True)
     return out
+
+
+def graph_replay_us(ctx, dp, calls=32, replays=20):
+    """Per-call time when `calls` back-to-back calls are recorded into one HIP
+    graph and the graph is replayed: what a caller with a fixed sequence of
+    small products pays once the per-call host work is out of the way."""
+    import torch
+    side = torch.cuda.Stream()
+    previous = torch.cuda.current_stream().cuda_stream
+    ctx.synchronize()
+    ctx.set_stream(side.cuda_stream)
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(calls):
+                dp.run(ctx)
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                graph.replay()
+            side.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(replays):
+                graph.replay()
+            side.synchronize()
+            dt = time.perf_counter() - t0
+        del graph
+    finally:
+        ctx.set_stream(previous)
+    return dt / (replays * calls) * 1e6
 
 
 def main():

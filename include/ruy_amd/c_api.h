@@ -153,7 +153,21 @@ RUYAMD_API int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs,
  * (ruy/thread_pool.cc:239 waits for all workers). `ruyamd_ctx_set_stream`
  * makes the context launch on a caller-owned hipStream_t (NULL = the legacy
  * default stream); `ruyamd_ctx_set_synchronous(ctx, 0)` makes calls whose
- * operands are all device-resident return after enqueueing. */
+ * operands are all device-resident return after enqueueing.
+ *
+ * Graph capture. ruyamd_mul may be called while the context's stream is
+ * capturing (hipStreamBeginCapture): the call then only records its kernels
+ * and never waits, whatever the synchronous setting. While capturing, every
+ * buffer must be device memory, an operand with a cache policy must already be
+ * in the prepacked cache, and the scratch memory the call needs must already
+ * exist - all three hold once the same call has run once outside the capture;
+ * otherwise the call fails with RUYAMD_E_UNSUPPORTED or RUYAMD_E_HIP and
+ * records nothing. Scratch memory a captured call used is kept until the
+ * context is destroyed and cache entries it used are exempt from ejection, so
+ * a graph stays replayable until ruyamd_ctx_clear_prepacked_cache,
+ * ruyamd_ctx_set_cache_max_bytes or ruyamd_ctx_destroy. Replays share that
+ * scratch with the context's later calls: order them on one stream. Kernel
+ * timing skips captured calls. */
 RUYAMD_API int ruyamd_ctx_set_stream(ruyamd_ctx* ctx, void* hip_stream);
 RUYAMD_API int ruyamd_ctx_set_synchronous(ruyamd_ctx* ctx, int synchronous);
 RUYAMD_API int ruyamd_ctx_synchronize(ruyamd_ctx* ctx);

@@ -25,6 +25,7 @@ void* Workspace::Alloc(std::size_t bytes) {
       return p;
     }
   }
+  if (!growth_allowed_) return nullptr;
   std::size_t size = need < (std::size_t(1) << 20) ? (std::size_t(1) << 20) : need;
   void* p = nullptr;
   if (hipMalloc(&p, size) != hipSuccess) {
@@ -36,7 +37,7 @@ void* Workspace::Alloc(std::size_t bytes) {
 }
 
 void Workspace::Reset() {
-  if (blocks_.size() > 1) {
+  if (blocks_.size() > 1 && !pinned_ && growth_allowed_) {
     // Coalesce: one block as large as everything the last call needed.
     std::size_t total = 0;
     for (auto& b : blocks_) {
@@ -60,7 +61,7 @@ void Workspace::Reset() {
 using ruyamd::PrepackedCache;
 
 bool ruyamd_ctx::TimingBegin() {
-  if (!kernel_timing) return false;
+  if (!kernel_timing || capturing) return false;
   std::pair<hipEvent_t, hipEvent_t> ev;
   if (!timing_pool.empty()) {
     ev = timing_pool.back();

@@ -21,7 +21,10 @@ namespace ruyamd {
 // released together at the start of the next call (ruy's
 // Allocator::FreeAll, ruy/frontend.cc:34). If a call outgrows the current
 // block an extra block is taken, and the next Reset replaces all blocks with
-// one that is large enough.
+// one that is large enough. Once Pin() has been called (work that refers to
+// the scratch was recorded for later replay) blocks are never released or
+// replaced before the workspace is destroyed, and while growth is disabled
+// Alloc fails instead of taking a new block.
 class Workspace {
  public:
   ~Workspace();
@@ -31,6 +34,8 @@ class Workspace {
   // Call only when no kernel still uses the previous call's scratch.
   void Reset();
   std::size_t capacity() const;
+  void Pin() { pinned_ = true; }
+  void set_growth_allowed(bool allowed) { growth_allowed_ = allowed; }
 
  private:
   struct Block {
@@ -39,6 +44,8 @@ class Workspace {
     std::size_t used;
   };
   std::vector<Block> blocks_;
+  bool pinned_ = false;
+  bool growth_allowed_ = true;
 };
 
 }  // namespace ruyamd
@@ -48,6 +55,7 @@ struct ruyamd_ctx {
   hipStream_t own_stream = nullptr;
   hipStream_t stream = nullptr;
   bool synchronous = true;
+  bool capturing = false;  // this call's stream is recording a graph
   int last_used_path = RUYAMD_PATH_NONE;
   int runtime_enabled_paths = RUYAMD_PATH_NONE;  // kNone = not decided yet
   int max_num_threads = 1;

@@ -1,18 +1,22 @@
-// int8 skinny multiplication (at most 8 vectors on the narrow side) without
-// matrix instructions: a pure HBM-streaming kernel. Replaces the reference's
-// single-column 8-bit kernels (ruy/kernel_avx512.cc:628-870) and their
-// dispatch (ruy/kernel_x86.h:54-59), extended from 1 to 8 columns.
+// int8 skinny multiplication (at most 8 vectors on the narrow side): pure
+// HBM-streaming kernels. They replace the reference's single-column 8-bit
+// kernels (ruy/kernel_avx512.cc:628-870) and their dispatch
+// (ruy/kernel_x86.h:54-59), extended from 1 to 8 columns.
 //
 // "Wide" operand: `rows` depth-contiguous int8 vectors of length K (the weight
-// matrix's rows, or its cached packed copy). "Narrow" operand: NB <= 8
-// depth-contiguous int8 vectors. Each wave owns kRowsPerWave wide vectors and
-// walks the depth 1024 bytes at a time: every lane holds 16 depth bytes of each
-// narrow vector in registers and applies them with v_dot4_i32_i8 to the 16
-// bytes it loads from each of its wide vectors, so the narrow operand is read
-// (from L2) once per kRowsPerWave wide vectors and the wide operand (from HBM)
-// exactly once. The
-// per-lane partial sums are reduced across the wave at the end and the fused
-// write-back (zero points, bias, requantization, clamp) runs on the totals.
+// matrix's rows, or its cached packed copy), read from HBM exactly once.
+// "Narrow" operand: at most 8 depth-contiguous int8 vectors.
+//
+// One narrow vector: GemvI8Kernel. Each wave owns two wide vectors and walks
+// the depth 1024 bytes at a time; every lane holds 16 depth bytes of the narrow
+// vector in registers and applies them with v_dot4_i32_i8 to the 16 bytes it
+// loads from each of its wide vectors. The per-lane partial sums are reduced
+// across the wave at the end and the fused write-back (zero points, bias,
+// requantization, clamp) runs on the totals.
+//
+// Two to eight narrow vectors: GemvI8MmaKernel, further down, which leaves
+// the multiply-accumulate and the summation over the depth to the matrix
+// cores.
 #include <hip/hip_runtime.h>
 
 #include "../epilogue.h"
@@ -137,17 +141,6 @@ void Launch(hipStream_t stream, const GemvI8Args& args) {
   hipLaunchKernelGGL((GemvI8Kernel<NB, R>), grid, dim3(64 * kWaves), 0, stream, args);
 }
 
-// ---------------------------------------------------------------------------
-// Variant for 2..8 narrow vectors whose whole depth fits in LDS: the workgroup
-// (8 waves) first copies the narrow operand into LDS with direct-to-LDS loads,
-// then every wave streams groups of 4 wide vectors through a 4-deep register
-// ring while the narrow slices come from LDS. Compared with the kernel above,
-// the narrow operand costs no registers for double buffering and no repeated
-// L2 reads, which leaves room for twice the loads in flight.
-// ---------------------------------------------------------------------------
-
-constexpr int kLdsRows = 4;        // wide vectors per group
-
 // 16 bytes per lane from the buffer straight to LDS at lds_base + 16*lane.
 // Issued as assembly so that the compiler does not serialise later LDS reads
 // against it; the caller waits on vmcnt and a barrier before reading.
@@ -171,128 +164,185 @@ __device__ __forceinline__ v4i RsrcWords(const void* p, uint32_t bytes) {
   return r;
 }
 
-// Sum over the 64 lanes as a wave-uniform value: four DPP steps leave each row
-// of 16 lanes holding its row sum, then the four row sums are read with
-// v_readlane.
-__device__ __forceinline__ int WaveSumDpp(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
-  v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
-  v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false);  // row_half_mirror
-  v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, false);  // row_mirror
-  return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) +
-         __builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48);
+// ---------------------------------------------------------------------------
+// Matrix-core variant for 2..8 narrow vectors. One wave per workgroup owns 16
+// wide vectors and walks the whole depth 512 bytes at a time through a ring
+// of LDS stages that only it uses (no barriers): a stage holds the 16 x 512
+// wide bytes and the 8 x 512 narrow bytes of one depth step, both brought in
+// by direct-to-LDS loads in which every instruction fetches whole 512-byte
+// runs. The products are formed by v_mfma_i32_16x16x64_i8 with the wide
+// vectors as matrix rows and the narrow vectors as columns 0..7 (columns
+// 8..15 read a 16-byte slot of zeros), which also does the summation over the
+// depth that the dot-product kernels above spend most of their vector
+// instructions on: per depth step the wave issues 12 loads, 16 LDS reads and
+// 8 matrix instructions and otherwise waits for HBM.
+//
+// LDS layout of a stage: vector v (0..15 wide, 16..23 narrow) at v*512; the
+// 16-byte chunk c of the vector's 512-byte run sits in slot c ^ (v & 7), so
+// that the 16 lanes of a matrix-operand read (16 vectors, one chunk index)
+// fall into different bank groups.
+// ---------------------------------------------------------------------------
+
+constexpr int kMmaRows = 16;
+constexpr int kMmaVectors = kMmaRows + 8;  // per stage: 16 wide, 8 narrow
+constexpr int kRotate = 11;
+
+template <int N>
+__device__ __forceinline__ void WaitVmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <int NB, int kLdsWaves, int kLdsRing>
-__global__ __launch_bounds__(64 * kLdsWaves) void GemvI8LdsKernel(GemvI8Args args) {
-  constexpr int kLdsGroupsPerWave = 16 / kLdsWaves;
-  extern __shared__ __attribute__((aligned(16))) char lds[];
+// kStep: depth bytes per ring stage (256, 512 or 1024). kSplit: waves per
+// workgroup; wave w walks the w-th part of the depth and the partial result
+// blocks are added through LDS at the end.
+template <int kRing, int kStep, int kSplit>
+__global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) {
+  constexpr int kStage = kMmaVectors * kStep;
+  constexpr int kRunsPerLoad = 1024 / kStep;       // runs of kStep bytes moved by one load
+  constexpr int kLanesPerRun = kStep / 16;
+  constexpr int kLoadsPerStage = kMmaVectors / kRunsPerLoad;
+  constexpr int kWideLoads = kMmaRows / kRunsPerLoad;
+  constexpr int kWaveLds = kRing * kStage + 16;    // ring + a 16-byte slot of zeros
+  static_assert((kRing - 1) * kLoadsPerStage <= 63, "vmcnt is a 6-bit counter");
+  extern __shared__ __attribute__((aligned(16))) char lds_all[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const __amdgpu_buffer_rsrc_t w_rsrc = MakeRsrc(args.wide, args.wide_bytes);
+  char* lds = lds_all + wave * kWaveLds;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const v4i w_rsrc = RsrcWords(args.wide, args.wide_bytes);
   const v4i n_rsrc = RsrcWords(args.narrow, args.narrow_bytes);
   const int K = args.K;  // multiple of 16
-  const int chunks_per_vec = K / 16;
+  const int row0 = blockIdx.x * kMmaRows;
+  constexpr int kZeroSlot = kRing * kStage;
+  if (lane < 4) reinterpret_cast<int*>(lds + kZeroSlot)[lane] = 0;
 
-  // ---- narrow operand -> LDS as [j][K] ----
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
-  const int total_chunks = NB * chunks_per_vec;
-  for (int c0 = wave * 64; c0 < total_chunks; c0 += kLdsWaves * 64) {
-    const int c = c0 + lane;
-    const int j = c / chunks_per_vec;
-    const int kc = c - j * chunks_per_vec;
-    const uint32_t off = (c < total_chunks && j < args.narrow_count)
-                             ? uint32_t(j) * uint32_t(args.ld_narrow) + kc * 16
-                             : kOutOfRange;
-    LoadToLds16(lds_base + c0 * 16, off, n_rsrc);
+  // Load side: instruction i of a stage moves vectors i*kRunsPerLoad ..; lane
+  // l takes run l / kLanesPerRun of them and fills LDS slot l % kLanesPerRun.
+  const int run = lane / kLanesPerRun;
+  const int slot = lane % kLanesPerRun;
+  uint32_t v_off[kLoadsPerStage];  // byte offset of this lane's chunk at depth 0
+  int v_chunk[kLoadsPerStage];
+#pragma unroll
+  for (int i = 0; i < kLoadsPerStage; ++i) {
+    const int v = i * kRunsPerLoad + run;
+    const int c = slot ^ (v & 7);
+    v_chunk[i] = c;
+    if (v < kMmaRows) {
+      const int row = row0 + v;
+      v_off[i] = row < args.rows ? uint32_t(row) * uint32_t(args.ld_wide) + c * 16 : kOutOfRange;
+    } else {
+      const int j = v - kMmaRows;
+      v_off[i] = j < args.narrow_count ? uint32_t(j) * uint32_t(args.ld_narrow) + c * 16 : kOutOfRange;
+    }
+  }
+  auto issue = [&](int s, int ring_slot) {
+    const int k0 = s * kStep;
+    const uint32_t base = lds_base + ring_slot * kStage;
+    if (k0 + kStep <= K) {
+#pragma unroll
+      for (int i = 0; i < kLoadsPerStage; ++i)
+        LoadToLds16(base + i * 1024, v_off[i] + k0, i < kWideLoads ? w_rsrc : n_rsrc);
+    } else {
+      // The last, partial step: chunks past the depth read as zeros.
+#pragma unroll
+      for (int i = 0; i < kLoadsPerStage; ++i)
+        LoadToLds16(base + i * 1024, k0 + v_chunk[i] * 16 < K ? v_off[i] + k0 : kOutOfRange,
+                    i < kWideLoads ? w_rsrc : n_rsrc);
+    }
+  };
+
+  // Matrix side: lane l supplies row (column) l%16, depth bytes 16*(l/16)..+15
+  // of each 64-byte block.
+  const int mv = lane & 15;
+  const int q = lane >> 4;
+  const bool narrow_lane = mv < 8;
+  v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+  auto consume = [&](int ring_slot) {
+    const char* stage = lds + ring_slot * kStage;
+    const char* a_row = stage + mv * kStep;
+    const char* b_row = stage + (kMmaRows + mv) * kStep;
+#pragma unroll
+    for (int kb = 0; kb < kStep / 64; ++kb) {
+      const int sl = ((kb * 4 + q) ^ (mv & 7)) * 16;
+      const v4i a = *reinterpret_cast<const v4i*>(a_row + sl);
+      const v4i b = *reinterpret_cast<const v4i*>(narrow_lane ? b_row + sl : lds + kZeroSlot);
+      if (kb & 1)
+        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc1, 0, 0, 0);
+      else
+        acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc0, 0, 0, 0);
+    }
+  };
+
+  const int steps_total = (K + kStep - 1) / kStep;
+  const int steps_per_wave = (steps_total + kSplit - 1) / kSplit;
+  const int s_begin = wave * steps_per_wave;
+  const int s_end = min(steps_total, s_begin + steps_per_wave);
+  // The order of the depth steps does not matter for the sums. Each workgroup
+  // starts at a different step and wraps around, so that workgroups running
+  // side by side do not all ask the same memory channels at the same time.
+  const int n_steps = s_end - s_begin;
+  int next = 0;  // next step to issue, as an index into the rotated order
+  int phys = n_steps > 0 ? s_begin + (blockIdx.x * kRotate) % n_steps : 0;
+  auto issue_next = [&](int ring_slot) {
+    issue(phys, ring_slot);
+    ++next;
+    phys = phys + 1 == s_end ? s_begin : phys + 1;
+  };
+#pragma unroll
+  for (int p = 0; p < kRing; ++p)
+    if (p < n_steps) issue_next(p);
+  int ring_slot = 0;
+  for (int s = 0; s < n_steps; ++s) {
+    // In-order completion: with kRing stages outstanding the oldest has landed
+    // once at most kRing-1 stages' loads remain. Near the end fewer stages are
+    // outstanding and everything is awaited.
+    if (s + kRing <= n_steps)
+      WaitVmcnt<(kRing - 1) * kLoadsPerStage>();
+    else
+      WaitVmcnt<0>();
+    consume(ring_slot);
+    if (next < n_steps) issue_next(ring_slot);
+    ring_slot = ring_slot + 1 == kRing ? 0 : ring_slot + 1;
+  }
+  v4i acc = acc0 + acc1;
+  if (kSplit > 1) {
+    // Every load of this wave has landed; its ring now carries its partial block.
+    if (wave > 0) reinterpret_cast<v4i*>(lds)[lane] = acc;
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 1; w < kSplit; ++w) acc += reinterpret_cast<const v4i*>(lds_all + w * kWaveLds)[lane];
   }
 
-  const int steps = (K + 1023) / 1024;
-  const int ring_rounds = (steps + kLdsRing - 1) / kLdsRing;
-  for (int g = 0; g < kLdsGroupsPerWave; ++g) {
-    const int row0 = ((blockIdx.x * kLdsGroupsPerWave + g) * kLdsWaves + wave) * kLdsRows;
-    uint32_t w_off[kLdsRows];
+  // Result block: lane l holds column l%16, rows 4*(l/16)..+3.
+  const int j = mv;
+  if (j < args.narrow_count) {
 #pragma unroll
-    for (int r = 0; r < kLdsRows; ++r) {
-      const int row = row0 + r;
-      w_off[r] = row < args.rows ? uint32_t(row) * uint32_t(args.ld_wide) + lane * 16 : kOutOfRange;
-    }
-    int acc[kLdsRows][NB];
-#pragma unroll
-    for (int r = 0; r < kLdsRows; ++r)
-#pragma unroll
-      for (int j = 0; j < NB; ++j) acc[r][j] = 0;
-
-    v4i ring[kLdsRing][kLdsRows];
-    auto load_step = [&](int s, v4i (&w)[kLdsRows]) {
-      const int k0 = s * 1024;
-      const bool in = k0 + lane * 16 < K;
-#pragma unroll
-      for (int r = 0; r < kLdsRows; ++r)
-        w[r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, in ? w_off[r] + k0 : kOutOfRange, 0, 0);
-    };
-#pragma unroll
-    for (int p = 0; p < kLdsRing; ++p) load_step(p, ring[p]);
-    if (g == 0) {
-      // The first wide loads are already in flight while the narrow operand
-      // lands in LDS.
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-    }
-    if (row0 >= args.rows) continue;
-    for (int round = 0; round < ring_rounds; ++round) {
-#pragma unroll
-      for (int p = 0; p < kLdsRing; ++p) {
-        const int s = round * kLdsRing + p;
-        const int k = s * 1024 + lane * 16;
-        // Past the depth the wide values are zero; only keep the LDS address in range.
-        const int kk = k < K ? k : 0;
-        v4i n[NB];
-#pragma unroll
-        for (int j = 0; j < NB; ++j) n[j] = *reinterpret_cast<const v4i*>(lds + j * K + kk);
-#pragma unroll
-        for (int r = 0; r < kLdsRows; ++r)
-#pragma unroll
-          for (int j = 0; j < NB; ++j) acc[r][j] = Dot16(ring[p][r], n[j], acc[r][j]);
-        load_step(s + kLdsRing, ring[p]);
+    for (int v = 0; v < 4; ++v) {
+      const int row = row0 + 4 * q + v;
+      if (row < args.rows) {
+        const int di = args.swapped ? j : row;
+        const int dj = args.swapped ? row : j;
+        const int32_t out = FinishInt<true>(acc[v], di, dj, args.ep);
+        StoreInt(args.dst.data, args.dst.dtype, int64_t(di) * args.dst.rs + int64_t(dj) * args.dst.cs, out);
       }
-    }
-
-    // Reduce; lane r*NB + j finishes and stores element (row0 + r, j).
-    int mine = 0;
-#pragma unroll
-    for (int r = 0; r < kLdsRows; ++r)
-#pragma unroll
-      for (int j = 0; j < NB; ++j) {
-        const int total = WaveSumDpp(acc[r][j]);
-        if (lane == r * NB + j) mine = total;
-      }
-    const int r = lane / NB;
-    const int j = lane % NB;
-    const int row = row0 + r;
-    if (lane < kLdsRows * NB && row < args.rows && j < args.narrow_count) {
-      const int di = args.swapped ? j : row;
-      const int dj = args.swapped ? row : j;
-      const int32_t v = FinishInt<true>(mine, di, dj, args.ep);
-      StoreInt(args.dst.data, args.dst.dtype, int64_t(di) * args.dst.rs + int64_t(dj) * args.dst.cs, v);
     }
   }
 }
 
-template <int NB, int kLdsWaves, int kLdsRing>
-hipError_t LaunchLds(hipStream_t stream, const GemvI8Args& args) {
-  const size_t lds_bytes = size_t(NB) * args.K;
-  auto kernel = GemvI8LdsKernel<NB, kLdsWaves, kLdsRing>;
-  static size_t attr_bytes = 0;
-  if (lds_bytes > 48 * 1024 && lds_bytes > attr_bytes) {
+template <int kRing, int kStep, int kSplit>
+hipError_t LaunchMma(hipStream_t stream, const GemvI8Args& args) {
+  constexpr size_t lds_bytes = size_t(kSplit) * (size_t(kRing) * kMmaVectors * kStep + 16);
+  auto kernel = GemvI8MmaKernel<kRing, kStep, kSplit>;
+  static bool attr_set = false;
+  if (lds_bytes > 48 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (e != hipSuccess) return e;
-    attr_bytes = lds_bytes;
+    attr_set = true;
   }
-  const int rows_per_block = 16 * kLdsRows;
-  const dim3 grid((args.rows + rows_per_block - 1) / rows_per_block);
-  hipLaunchKernelGGL(kernel, grid, dim3(64 * kLdsWaves), lds_bytes, stream, args);
+  const dim3 grid((args.rows + kMmaRows - 1) / kMmaRows);
+  hipLaunchKernelGGL(kernel, grid, dim3(64 * kSplit), lds_bytes, stream, args);
   return hipGetLastError();
 }
 
@@ -300,29 +350,26 @@ hipError_t LaunchLds(hipStream_t stream, const GemvI8Args& args) {
 
 hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
   if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
-  // Two or more narrow vectors that fit in LDS (and enough wide vectors to be
-  // worth a 512-thread workgroup): the LDS-resident variant.
-  if (args.narrow_count >= 2 && args.rows >= 256 && args.K >= 1024) {
-    const int nb = args.narrow_count <= 2 ? 2 : args.narrow_count <= 4 ? 4 : 8;
-    if (size_t(nb) * args.K <= 144 * 1024) {
-      // 8 waves with a 4-deep ring measured best on the 16384^2 weight.
-      if (nb == 2) return LaunchLds<2, 8, 4>(stream, args);
-      if (nb == 4) return LaunchLds<4, 8, 4>(stream, args);
-      return LaunchLds<8, 8, 4>(stream, args);
-    }
-  }
-  // Wide vectors per wave: fewer for narrower problems, where more and
-  // smaller waves keep more of the stream in flight (measured on the 16384^2
-  // weight: 2 for one column, 4 beyond).
-  if (args.narrow_count <= 1)
+  // What the kernels assume: at most 8 narrow vectors, 16-byte granularity of
+  // the depth, of both pitches and of both base addresses.
+  if (args.narrow_count > 8 || args.K % 16 != 0 || args.ld_wide % 16 != 0 ||
+      (args.narrow_count > 1 && args.ld_narrow % 16 != 0) ||
+      (reinterpret_cast<uintptr_t>(args.wide) | reinterpret_cast<uintptr_t>(args.narrow)) % 16 != 0)
+    return hipErrorInvalidValue;
+  if (args.narrow_count == 1) {
+    // One column: the dot-product kernel. Its many small waves are scheduled
+    // dynamically and it streams a little faster than the matrix-core kernel
+    // at every size measured.
     Launch<1, 2>(stream, args);
-  else if (args.narrow_count <= 2)
-    Launch<2, 4>(stream, args);
-  else if (args.narrow_count <= 4)
-    Launch<4, 4>(stream, args);
-  else
-    Launch<8, 4>(stream, args);
-  return hipGetLastError();
+    return hipGetLastError();
+  }
+  // Matrix-core kernel. With few groups of 16 wide vectors the depth is split
+  // over the waves of a workgroup to get enough loads in flight.
+  const int groups = (args.rows + kMmaRows - 1) / kMmaRows;
+  const int steps = (args.K + 511) / 512;
+  if (groups >= 512 || steps < 4) return LaunchMma<2, 512, 1>(stream, args);
+  if (steps < 8) return LaunchMma<2, 512, 2>(stream, args);
+  return LaunchMma<2, 512, 4>(stream, args);
 }
 
 }  // namespace ruyamd

@@ -120,6 +120,33 @@ const void* StageIn(ruyamd_ctx* ctx, const void* p, std::size_t bytes, bool* sta
   return d;
 }
 
+// Finds out whether the context's stream is recording a graph and holds the
+// context in that mode for the duration of one call.
+class CaptureScope {
+ public:
+  explicit CaptureScope(ruyamd_ctx* ctx) : ctx_(ctx) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &status) != hipSuccess) {
+      (void)hipGetLastError();
+      status = hipStreamCaptureStatusNone;
+    }
+    ctx->capturing = status == hipStreamCaptureStatusActive;
+    if (ctx->capturing) {
+      ctx->workspace.Pin();
+      ctx->workspace.set_growth_allowed(false);
+    }
+  }
+  ~CaptureScope() {
+    ctx_->capturing = false;
+    ctx_->workspace.set_growth_allowed(true);
+  }
+  CaptureScope(const CaptureScope&) = delete;
+  CaptureScope& operator=(const CaptureScope&) = delete;
+
+ private:
+  ruyamd_ctx* ctx_;
+};
+
 DevMat ToDevMat(const ruyamd_mat& m, const void* device_data) {
   DevMat d;
   d.data = const_cast<void*>(device_data);
@@ -162,6 +189,20 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
 
   if (hipSetDevice(ctx->device) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "hipSetDevice failed");
   if (dst->rows == 0 || dst->cols == 0) return RUYAMD_OK;
+
+  // A stream that is recording a graph takes kernel launches only: nothing
+  // below may allocate, free, copy from or to the host, or wait. Scratch
+  // memory and cache entries that recorded kernels refer to stay where they
+  // are until the context is destroyed (cache entries: or cleared).
+  CaptureScope capture_scope(ctx);
+  if (ctx->capturing) {
+    const void* pointers[] = {lhs->data, rhs->data, dst->data, p->bias, p->multiplier_fixedpoint_perchannel,
+                              p->multiplier_exponent_perchannel};
+    for (const void* ptr : pointers) {
+      if (ptr && !IsDevicePointer(ptr))
+        return Fail(ctx, RUYAMD_E_UNSUPPORTED, "the stream is capturing: every buffer must be device memory");
+    }
+  }
 
   // Scratch of the previous call is reused. If that call was asynchronous its
   // kernels may not have run yet, but everything that touches the scratch -
@@ -228,7 +269,11 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
 
   std::string err;
   const int rc = RunMul(ctx, &call, &err);
-  if (rc != RUYAMD_OK) return Fail(ctx, rc, err);
+  if (rc != RUYAMD_OK) {
+    if (ctx->capturing && rc == RUYAMD_E_HIP)
+      err += " (the stream is capturing, so no memory can be allocated: run the same call once before the capture)";
+    return Fail(ctx, rc, err);
+  }
   staged = staged || call.staged_any;
 
   if (!dst_on_device) {
@@ -240,7 +285,7 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
       return Fail(ctx, RUYAMD_E_HIP, "copying the destination back to the host failed");
     staged = true;
   }
-  if (ctx->synchronous || staged) {
+  if ((ctx->synchronous || staged) && !ctx->capturing) {
     if (hipStreamSynchronize(ctx->stream) != hipSuccess)
       return Fail(ctx, RUYAMD_E_HIP, std::string("kernel execution failed: ") + hipGetErrorString(hipGetLastError()));
   }

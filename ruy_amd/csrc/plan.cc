@@ -42,6 +42,16 @@ struct Operand8 {
   uint32_t bytes = 0;
 };
 
+// While the stream records a graph the cache may neither allocate nor eject:
+// a hit is pinned (the recorded kernels keep reading its buffers on every
+// replay), a miss is an error.
+PrepackedCache::Mode CacheMode(const ruyamd_ctx* ctx) {
+  return ctx->capturing ? PrepackedCache::Mode::kPinExisting : PrepackedCache::Mode::kInsertOnMiss;
+}
+const char kCaptureCacheMiss[] =
+    "the stream is capturing and an operand with a cache policy is not in the prepacked cache yet: "
+    "run the same call once before the capture";
+
 // Prepares one side: from the cache, in place, or packed into the workspace.
 // `src` views the side as `count` depth vectors (LHS rows / RHS columns).
 int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point, bool need_sums,
@@ -77,7 +87,11 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
     pm.layout.kernel_rows = 16;
     pm.layout.kernel_cols = 1;
     pm.zero_point = out->zero_point;
-    const auto action = ctx->cache->Get(src_key, &pm);
+    const auto action = ctx->cache->Get(src_key, &pm, CacheMode(ctx));
+    if (action == PrepackedCache::Action::kMissing) {
+      *err = kCaptureCacheMiss;
+      return RUYAMD_E_UNSUPPORTED;
+    }
     if (!pm.data) {
       *err = "device allocation for a cached packed matrix failed";
       return RUYAMD_E_HIP;
@@ -251,7 +265,11 @@ int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy
     pm.layout.stride = ld;
     pm.layout.kernel_rows = 4;
     pm.layout.kernel_cols = 1;
-    const auto action = ctx->cache->Get(src_key, &pm);
+    const auto action = ctx->cache->Get(src_key, &pm, CacheMode(ctx));
+    if (action == PrepackedCache::Action::kMissing) {
+      *err = kCaptureCacheMiss;
+      return RUYAMD_E_UNSUPPORTED;
+    }
     if (!pm.data) {
       *err = "device allocation for a cached packed matrix failed";
       return RUYAMD_E_HIP;

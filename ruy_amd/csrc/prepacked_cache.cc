@@ -14,13 +14,19 @@ std::size_t PrepackedCache::KeyHash::operator()(const Key& k) const {
   return h;
 }
 
-PrepackedCache::Action PrepackedCache::Get(const void* src_data, PackedMatrix* packed_matrix) {
+PrepackedCache::Action PrepackedCache::Get(const void* src_data, PackedMatrix* packed_matrix, Mode mode) {
   Key key{src_data, packed_matrix->layout, packed_matrix->zero_point};
   auto it = cache_.find(key);
   if (it != cache_.end()) {
     it->second.timestamp = timestamp_++;
+    if (mode == Mode::kPinExisting) it->second.pinned = true;
     *packed_matrix = it->second.packed;
     return Action::kGotExistingEntry;
+  }
+  if (mode == Mode::kPinExisting) {
+    packed_matrix->data = nullptr;
+    packed_matrix->sums = nullptr;
+    return Action::kMissing;
   }
   const std::ptrdiff_t data_bytes = packed_matrix->DataBytes();
   const std::ptrdiff_t sums_bytes = packed_matrix->SumsBytes();
@@ -43,19 +49,24 @@ PrepackedCache::Action PrepackedCache::Get(const void* src_data, PackedMatrix* p
 }
 
 void PrepackedCache::EjectUntilRoomFor(std::ptrdiff_t new_bytes) {
-  while (!cache_.empty() && buffers_bytes_ + new_bytes > max_buffers_bytes_) EjectOne();
+  while (!cache_.empty() && buffers_bytes_ + new_bytes > max_buffers_bytes_) {
+    if (!EjectOne()) break;
+  }
 }
 
-void PrepackedCache::EjectOne() {
-  auto oldest = cache_.begin();
+bool PrepackedCache::EjectOne() {
+  auto oldest = cache_.end();
   for (auto it = cache_.begin(); it != cache_.end(); ++it) {
-    if (it->second.timestamp < oldest->second.timestamp) oldest = it;
+    if (it->second.pinned) continue;
+    if (oldest == cache_.end() || it->second.timestamp < oldest->second.timestamp) oldest = it;
   }
+  if (oldest == cache_.end()) return false;
   const PackedMatrix& pm = oldest->second.packed;
   buffers_bytes_ -= pm.DataBytes() + pm.SumsBytes();
   free_(pm.data);
   if (pm.sums) free_(pm.sums);
   cache_.erase(oldest);
+  return true;
 }
 
 void PrepackedCache::Clear() {

@@ -52,7 +52,11 @@ struct PackedMatrix {
 
 class PrepackedCache final {
  public:
-  enum class Action { kGotExistingEntry, kInsertedNewEntry };
+  enum class Action { kGotExistingEntry, kInsertedNewEntry, kMissing };
+  // kPinExisting never allocates or frees: a hit is marked so that ejection
+  // passes it over from then on (its buffers may be referenced by work that
+  // was recorded for later replay), a miss returns kMissing.
+  enum class Mode { kInsertOnMiss, kPinExisting };
   using AllocFn = std::function<void*(std::size_t)>;
   using FreeFn = std::function<void(void*)>;
 
@@ -72,7 +76,7 @@ class PrepackedCache final {
   // new one fits or the cache is empty (an entry larger than the whole budget
   // is still kept), and inserts it; the caller must then pack into the buffers.
   // Returns kInsertedNewEntry with null data if allocation failed.
-  Action Get(const void* src_data, PackedMatrix* packed_matrix);
+  Action Get(const void* src_data, PackedMatrix* packed_matrix, Mode mode = Mode::kInsertOnMiss);
 
   std::ptrdiff_t BuffersBytes() const { return buffers_bytes_; }
   int MatrixCount() const { return static_cast<int>(cache_.size()); }
@@ -98,9 +102,10 @@ class PrepackedCache final {
   struct Entry {
     PackedMatrix packed;
     uint64_t timestamp;
+    bool pinned = false;  // only Clear() releases a pinned entry
   };
   void EjectUntilRoomFor(std::ptrdiff_t new_bytes);
-  void EjectOne();
+  bool EjectOne();  // false when only pinned entries are left
 
   AllocFn alloc_;
   FreeFn free_;

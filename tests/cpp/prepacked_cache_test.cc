@@ -111,6 +111,42 @@ static void TestEjectionOrder() {
   EXPECT(cache.Get(d2.data(), &m2) == kInserted);
 }
 
+// Not in the reference: entries looked up in kPinExisting mode (their buffers
+// are referenced by recorded work) survive ejection; a miss in that mode
+// neither allocates nor inserts.
+static void TestPinnedEntriesSurviveEjection() {
+  PrepackedCache cache(CountingAlloc, CountingFree, 1000);
+  std::vector<std::uint8_t> d1(200), d2(200), d3(200), d4(200), d5(200);
+  PackedMatrix m1 = Dummy(false, 10, 20), m2 = m1, m3 = m1, m4 = m1, m5 = m1;
+  const auto kPin = PrepackedCache::Mode::kPinExisting;
+  const long allocs_before = g_live_allocations;
+  EXPECT(cache.Get(d1.data(), &m1, kPin) == PrepackedCache::Action::kMissing);
+  EXPECT(m1.data == nullptr && cache.MatrixCount() == 0 && g_live_allocations == allocs_before);
+  m1 = Dummy(false, 10, 20);
+  cache.Get(d1.data(), &m1);
+  cache.Get(d2.data(), &m2);
+  cache.Get(d3.data(), &m3);
+  void* const pinned_data = m1.data;
+  EXPECT(cache.Get(d1.data(), &m1, kPin) == kExisting);  // pin the oldest entry
+  EXPECT(m1.data == pinned_data);
+  cache.Get(d2.data(), &m2);
+  cache.Get(d3.data(), &m3);                             // 1 is least recently used again
+  cache.Get(d4.data(), &m4);                             // ejects 2, not the pinned 1
+  EXPECT(cache.Get(d1.data(), &m1) == kExisting);
+  EXPECT(cache.Get(d3.data(), &m3) == kExisting);
+  EXPECT(cache.Get(d2.data(), &m2) == kInserted);        // ejects 4 (oldest unpinned)
+  EXPECT(cache.Get(d1.data(), &m1) == kExisting && m1.data == pinned_data);
+  // With only pinned entries left ejection stops, as it does on an empty cache.
+  PrepackedCache small(CountingAlloc, CountingFree, 300);
+  PackedMatrix a = Dummy(false, 10, 20), b = a;
+  small.Get(d1.data(), &a);
+  EXPECT(small.Get(d1.data(), &a, kPin) == kExisting);
+  EXPECT(small.Get(d5.data(), &b) == kInserted);
+  EXPECT(small.MatrixCount() == 2);
+  small.Clear();  // Clear releases pinned entries too
+  EXPECT(small.MatrixCount() == 0 && small.BuffersBytes() == 0);
+}
+
 static void TestOversizeEntryIsKept() {
   PrepackedCache cache(CountingAlloc, CountingFree, 100);
   std::vector<std::uint8_t> d1(200);
@@ -152,6 +188,7 @@ int main() {
   TestEjection();
   TestEjectionOrder();
   TestOversizeEntryIsKept();
+  TestPinnedEntriesSurviveEjection();
   TestDistinguishSubtlyDifferentMatrices();
   EXPECT(g_live_allocations == 0);  // every cache freed what it allocated
   if (g_failures) {

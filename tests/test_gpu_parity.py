@@ -393,11 +393,14 @@ def test_tuned_kernels_are_the_ones_that_run(device_ctx):
                          ids=cases.tuple_name)
 def test_skinny_shapes_both_orientations(device_ctx, tup):
     """Narrow side on the right (matrix x few vectors) and on the left (few
-    vectors x matrix), depths that are not multiples of the 1024-byte step,
-    row counts that do not fill the last workgroup: both skinny kernels."""
+    vectors x matrix), depths that are not multiples of a kernel's depth step,
+    row counts that do not fill the last workgroup. The shapes reach the
+    one-column kernel and every depth-split variant of the 2..8-column kernel
+    (few or many groups of 16 rows; fewer than 4, 4..7, 8 or more depth steps)."""
     rng = np.random.default_rng(123)
     for shape in [(300, 1500, 5), (5, 1500, 300), (1031, 2048, 8), (8, 4100, 513), (257, 1024, 2),
-                  (2, 1100, 260), (1000, 3000, 3), (64, 9000, 7), (4, 64, 4), (3, 20000, 1)]:
+                  (2, 1100, 260), (1000, 3000, 3), (64, 9000, 7), (4, 64, 4), (3, 20000, 1),
+                  (8200, 2099, 6), (7, 5000, 8195), (8193, 300, 8), (17, 8192, 2)]:
         for orders in (cases.RCC, cases.ALL_ORDERS[int(rng.integers(8))]):
             p = W.random_problem(rng, *tup, *shape, *orders, strided=bool(rng.integers(2)),
                                  name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
