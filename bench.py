@@ -255,6 +255,35 @@ def bench_gemv(ctx, args):
             "kernel_ms": kernel_ms,
         },
     }
+    # The same weights against 4 and 8 activation vectors (the skinny kernel on
+    # the matrix cores), reusing the cache entries made above.
+    out["more_columns"] = []
+    for cols in (4, 8):
+        wider = []
+        for base_problem, base_dp in zip(problems, dps):
+            p = W.config_int8_gemv(n, cols, lhs=base_problem.lhs)
+            dp = device_problem(p)
+            dp.lhs_t = base_dp.lhs_t  # same device weights, hence the same cache entry
+            dp.lhs_s = p.lhs.struct(base_dp.lhs_t.data_ptr())
+            wider.append(dp)
+        state["i"] = 0
+
+        def run_wider():
+            wider[state["i"] % rotate].run(ctx)
+            state["i"] += 1
+
+        run_wider()
+        kernel_wider = ctx.last_kernel_name()
+        ctx.set_kernel_timing(False)
+        step_w, _, kernel_ms_w = time_steps(run_wider, args.steps * 4, args.warmup * 4, ctx)
+        ctx.set_kernel_timing(True)
+        nbytes_w = float(wider[0].problem.algorithmic_bytes())
+        out["more_columns"].append({
+            "N": cols, "kernel": kernel_wider, "ms_per_step": step_w * 1e3, "kernel_ms": kernel_ms_w,
+            "algorithmic_bytes": nbytes_w, "GB/s": nbytes_w / (kernel_ms_w * 1e-3) / 1e9,
+            "frac": nbytes_w / (kernel_ms_w * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "traffic": load_traffic("int8_gemv_%d_n%d" % (n, cols))})
+        del wider
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_gemv(problems[0])
     del dps
