@@ -1,11 +1,11 @@
-// int8 skinny multiplication (at most 8 vectors on the narrow side): pure
+// int8 skinny multiplication (at most 16 vectors on the narrow side): pure
 // HBM-streaming kernels. They replace the reference's single-column 8-bit
 // kernels (ruy/kernel_avx512.cc:628-870) and their dispatch
-// (ruy/kernel_x86.h:54-59), extended from 1 to 8 columns.
+// (ruy/kernel_x86.h:54-59), extended from 1 to 16 columns.
 //
 // "Wide" operand: `rows` depth-contiguous int8 vectors of length K (the weight
 // matrix's rows, or its cached packed copy), read from HBM exactly once.
-// "Narrow" operand: at most 8 depth-contiguous int8 vectors.
+// "Narrow" operand: at most 16 depth-contiguous int8 vectors.
 //
 // One narrow vector: GemvI8Kernel. Each wave owns two wide vectors and walks
 // the depth 1024 bytes at a time; every lane holds 16 depth bytes of the narrow
@@ -14,7 +14,7 @@
 // across the wave at the end and the fused write-back (zero points, bias,
 // requantization, clamp) runs on the totals.
 //
-// Two to eight narrow vectors: GemvI8MmaKernel, further down, which leaves
+// Two to sixteen narrow vectors: GemvI8MmaKernel, further down, which leaves
 // the multiply-accumulate and the summation over the depth to the matrix
 // cores.
 #include <hip/hip_runtime.h>
@@ -165,26 +165,25 @@ __device__ __forceinline__ v4i RsrcWords(const void* p, uint32_t bytes) {
 }
 
 // ---------------------------------------------------------------------------
-// Matrix-core variant for 2..8 narrow vectors. One wave per workgroup owns 16
+// Matrix-core variant for 2..16 narrow vectors. One wave per workgroup owns 16
 // wide vectors and walks the whole depth 512 bytes at a time through a ring
 // of LDS stages that only it uses (no barriers): a stage holds the 16 x 512
-// wide bytes and the 8 x 512 narrow bytes of one depth step, both brought in
-// by direct-to-LDS loads in which every instruction fetches whole 512-byte
-// runs. The products are formed by v_mfma_i32_16x16x64_i8 with the wide
-// vectors as matrix rows and the narrow vectors as columns 0..7 (columns
-// 8..15 read a 16-byte slot of zeros), which also does the summation over the
-// depth that the dot-product kernels above spend most of their vector
-// instructions on: per depth step the wave issues 12 loads, 16 LDS reads and
-// 8 matrix instructions and otherwise waits for HBM.
+// wide bytes and the 8 x 512 (or 16 x 512) narrow bytes of one depth step,
+// both brought in by direct-to-LDS loads in which every instruction fetches
+// whole 512-byte runs. The products are formed by v_mfma_i32_16x16x64_i8 with
+// the wide vectors as matrix rows and the narrow vectors as columns (when
+// only 8 are staged, columns 8..15 read a 16-byte slot of zeros), which also
+// does the summation over the depth that the dot-product kernel above spends
+// most of its vector instructions on: per depth step the wave issues 12 (16)
+// loads, 16 LDS reads and 8 matrix instructions and otherwise waits for HBM.
 //
-// LDS layout of a stage: vector v (0..15 wide, 16..23 narrow) at v*512; the
+// LDS layout of a stage: vector v (0..15 wide, 16.. narrow) at v*512; the
 // 16-byte chunk c of the vector's 512-byte run sits in slot c ^ (v & 7), so
 // that the 16 lanes of a matrix-operand read (16 vectors, one chunk index)
 // fall into different bank groups.
 // ---------------------------------------------------------------------------
 
 constexpr int kMmaRows = 16;
-constexpr int kMmaVectors = kMmaRows + 8;  // per stage: 16 wide, 8 narrow
 constexpr int kRotate = 11;
 
 template <int N>
@@ -194,9 +193,12 @@ __device__ __forceinline__ void WaitVmcnt() {
 
 // kStep: depth bytes per ring stage (256, 512 or 1024). kSplit: waves per
 // workgroup; wave w walks the w-th part of the depth and the partial result
-// blocks are added through LDS at the end.
-template <int kRing, int kStep, int kSplit>
+// blocks are added through LDS at the end. kNarrow: narrow vectors staged, 8
+// or 16 (with 16 every column of the matrix instruction is a real one).
+template <int kRing, int kStep, int kSplit, int kNarrow>
 __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) {
+  static_assert(kNarrow == 8 || kNarrow == 16, "");
+  constexpr int kMmaVectors = kMmaRows + kNarrow;  // vectors per stage
   constexpr int kStage = kMmaVectors * kStep;
   constexpr int kRunsPerLoad = 1024 / kStep;       // runs of kStep bytes moved by one load
   constexpr int kLanesPerRun = kStep / 16;
@@ -255,7 +257,7 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
   // of each 64-byte block.
   const int mv = lane & 15;
   const int q = lane >> 4;
-  const bool narrow_lane = mv < 8;
+  const bool narrow_lane = mv < kNarrow;
   v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
   auto consume = [&](int ring_slot) {
     const char* stage = lds + ring_slot * kStage;
@@ -330,16 +332,15 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
   }
 }
 
-template <int kRing, int kStep, int kSplit>
+template <int kRing, int kStep, int kSplit, int kNarrow>
 hipError_t LaunchMma(hipStream_t stream, const GemvI8Args& args) {
-  constexpr size_t lds_bytes = size_t(kSplit) * (size_t(kRing) * kMmaVectors * kStep + 16);
-  auto kernel = GemvI8MmaKernel<kRing, kStep, kSplit>;
-  static bool attr_set = false;
-  if (lds_bytes > 48 * 1024 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
-    if (e != hipSuccess) return e;
-    attr_set = true;
+  constexpr size_t lds_bytes = size_t(kSplit) * (size_t(kRing) * (kMmaRows + kNarrow) * kStep + 16);
+  auto kernel = GemvI8MmaKernel<kRing, kStep, kSplit, kNarrow>;
+  if (lds_bytes > 48 * 1024) {
+    // Once per process (thread-safe static initialisation).
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    if (attr != hipSuccess) return attr;
   }
   const dim3 grid((args.rows + kMmaRows - 1) / kMmaRows);
   hipLaunchKernelGGL(kernel, grid, dim3(64 * kSplit), lds_bytes, stream, args);
@@ -350,9 +351,9 @@ hipError_t LaunchMma(hipStream_t stream, const GemvI8Args& args) {
 
 hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
   if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
-  // What the kernels assume: at most 8 narrow vectors, 16-byte granularity of
+  // What the kernels assume: at most 16 narrow vectors, 16-byte granularity of
   // the depth, of both pitches and of both base addresses.
-  if (args.narrow_count > 8 || args.K % 16 != 0 || args.ld_wide % 16 != 0 ||
+  if (args.narrow_count > 16 || args.K % 16 != 0 || args.ld_wide % 16 != 0 ||
       (args.narrow_count > 1 && args.ld_narrow % 16 != 0) ||
       (reinterpret_cast<uintptr_t>(args.wide) | reinterpret_cast<uintptr_t>(args.narrow)) % 16 != 0)
     return hipErrorInvalidValue;
@@ -367,9 +368,15 @@ hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
   // over the waves of a workgroup to get enough loads in flight.
   const int groups = (args.rows + kMmaRows - 1) / kMmaRows;
   const int steps = (args.K + 511) / 512;
-  if (groups >= 512 || steps < 4) return LaunchMma<2, 512, 1>(stream, args);
-  if (steps < 8) return LaunchMma<2, 512, 2>(stream, args);
-  return LaunchMma<2, 512, 4>(stream, args);
+  const int split = groups >= 512 || steps < 4 ? 1 : steps < 8 ? 2 : 4;
+  if (args.narrow_count <= 8) {
+    if (split == 1) return LaunchMma<2, 512, 1, 8>(stream, args);
+    if (split == 2) return LaunchMma<2, 512, 2, 8>(stream, args);
+    return LaunchMma<2, 512, 4, 8>(stream, args);
+  }
+  if (split == 1) return LaunchMma<2, 512, 1, 16>(stream, args);
+  if (split == 2) return LaunchMma<2, 512, 2, 16>(stream, args);
+  return LaunchMma<2, 512, 4, 16>(stream, args);
 }
 
 }  // namespace ruyamd

@@ -12,6 +12,9 @@ namespace {
 // kCacheIfLargeSpeedup means "the other side is narrow enough for the
 // bandwidth-bound kernel".
 constexpr int kSkinnyWidth = 8;
+// The int8 streaming kernel itself takes up to 16 vectors on the narrow side
+// (all 16 columns of its matrix instruction).
+constexpr int kSkinnyWidthInt8 = 16;
 
 bool SetupDestination(const MulCall& call, GemmArgs* args);
 
@@ -172,10 +175,10 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     return rc;
   const int32_t zp_product_depth =
       static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
-  if (N <= kSkinnyWidth || M <= kSkinnyWidth) {
-    // Bandwidth-bound shapes: stream the wide side once, no matrix instructions.
+  if (N <= kSkinnyWidthInt8 || M <= kSkinnyWidthInt8) {
+    // Bandwidth-bound shapes: stream the wide side exactly once.
     GemvI8Args g;
-    g.swapped = !(N <= kSkinnyWidth && (M > kSkinnyWidth || M >= N));
+    g.swapped = !(N <= kSkinnyWidthInt8 && (M > kSkinnyWidthInt8 || M >= N));
     const Operand8& wide = g.swapped ? b : a;
     const Operand8& narrow = g.swapped ? a : b;
     g.wide = wide.data;

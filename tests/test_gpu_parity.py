@@ -410,6 +410,23 @@ def test_skinny_shapes_both_orientations(device_ctx, tup):
             assert device_ctx.last_kernel_name() == ("f32_gemv" if tup[0] == S.F32 else "i8_gemv")
 
 
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I16),
+                                 (S.U8, S.U8, S.I32, S.I32)], ids=cases.tuple_name)
+def test_skinny_nine_to_sixteen_vectors(device_ctx, tup):
+    """8-bit products whose narrow side has 9..16 vectors also go to the
+    streaming kernel (all 16 columns of its matrix instruction in use)."""
+    rng = np.random.default_rng(321)
+    for shape in [(300, 1500, 9), (16, 1500, 300), (1031, 2048, 16), (12, 4100, 513), (8200, 2099, 13),
+                  (10, 5000, 8195), (64, 9000, 11), (16, 64, 16), (9, 16, 9), (500, 520, 15)]:
+        for orders in (cases.RCC, cases.ALL_ORDERS[int(rng.integers(8))]):
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=bool(rng.integers(2)),
+                                 name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
+            assert device_ctx.last_kernel_name() == "i8_gemv"
+
+
 def test_caller_stream_asynchronous_calls_and_kernel_timing(device_ctx):
     """Device-side controls without a counterpart in the reference: launching on
     a caller-owned stream, returning before completion, per-kernel timing."""
