@@ -111,8 +111,14 @@ def cpu_baseline_gemm(problem, n_slice):
         rc = O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, cores,
                                          2.0, 2, C.byref(lat), C.byref(used))
         if rc == 0 and lat.value > 0:
-            return {"value": ops / lat.value / 1e12, "unit": "TOP/s", "cores": cores,
-                    "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
+            out = {"value": ops / lat.value / 1e12, "unit": "TOP/s", "cores": cores,
+                   "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
+            # ruy never picks a thread count itself (ruy/context.h:68-73): also one thread.
+            lat1 = C.c_double(0)
+            if O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, 1,
+                                           1.0, 1, C.byref(lat1), C.byref(used)) == 0 and lat1.value > 0:
+                out["value_1_thread"] = ops / lat1.value / 1e12
+            return out
     t0 = time.perf_counter()
     O.oracle_mul(sub)
     dt = time.perf_counter() - t0
@@ -133,8 +139,13 @@ def cpu_baseline_gemv(problem):
         rc = O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, cores,
                                          1.0, 3, C.byref(lat), C.byref(used))
         if rc == 0 and lat.value > 0:
-            return {"value": nbytes / lat.value / 1e9, "unit": "GB/s", "cores": cores,
-                    "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
+            out = {"value": nbytes / lat.value / 1e9, "unit": "GB/s", "cores": cores,
+                   "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
+            lat1 = C.c_double(0)
+            if O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, 1,
+                                           1.0, 1, C.byref(lat1), C.byref(used)) == 0 and lat1.value > 0:
+                out["value_1_thread"] = nbytes / lat1.value / 1e9
+            return out
     t0 = time.perf_counter()
     O.oracle_mul(problem)
     dt = time.perf_counter() - t0

@@ -484,12 +484,11 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int grid = ((total + 7) / 8) * 8;
   const size_t lds_bytes = C::kLdsBytes;
   auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES>;
-  static bool attr_set = false;
-  if (!attr_set && lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
-    if (e != hipSuccess) return e;
-    attr_set = true;
+  if (lds_bytes > 48 * 1024) {
+    // Once per process; static initialisation is safe against concurrent callers.
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    if (attr != hipSuccess) return attr;
   }
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::kThreads), lds_bytes, stream, args);
   return hipGetLastError();

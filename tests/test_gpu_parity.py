@@ -42,8 +42,8 @@ def compare(problem, got, want, exact_fp=False):
             problem.name, bad.size, bad[0], got[bad[0]], want[bad[0]])
 
 
-def run_both(ctx, problem, fill=0x5A):
-    import device_runner as D
+def expected(problem, fill=0x5A):
+    """The checker's destination storage, untouched elements holding the fill byte."""
     want = O.oracle_mul(problem)
     # give the checker's untouched elements the same fill pattern
     filled = np.zeros_like(want)
@@ -54,8 +54,12 @@ def run_both(ctx, problem, fill=0x5A):
         strides = (it, d.stride * it) if d.order == S.ORDER_COL_MAJOR else (d.stride * it, it)
         np.lib.stride_tricks.as_strided(filled, (d.rows, d.cols), strides)[...] = \
             np.lib.stride_tricks.as_strided(want, (d.rows, d.cols), strides)
-    got = D.device_mul(ctx, problem, fill)
-    return got, filled
+    return filled
+
+
+def run_both(ctx, problem, fill=0x5A):
+    import device_runner as D
+    return D.device_mul(ctx, problem, fill), expected(problem, fill)
 
 
 def test_requantizer_known_answers_on_device(device_ctx):
@@ -408,6 +412,44 @@ def test_skinny_shapes_both_orientations(device_ctx, tup):
             got, want = run_both(device_ctx, p)
             compare(p, got, want)
             assert device_ctx.last_kernel_name() == ("f32_gemv" if tup[0] == S.F32 else "i8_gemv")
+
+
+def test_two_contexts_on_two_threads():
+    """The reference's rule (ruy/ruy.h:82-95): a Context serves one thread, and
+    concurrent Mul calls need distinct Contexts. Two threads, each with its own
+    context (hence its own stream, scratch and cache), multiply concurrently."""
+    import threading
+    import device_runner as D
+    from ruy_amd import api
+    rng = np.random.default_rng(99)
+    jobs = []
+    for t in range(2):
+        probs = [W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, 300 + 7 * t, 400, 500, *cases.RCC, name="gemm"),
+                 W.random_problem(rng, S.U8, S.U8, S.I32, S.U8, 129, 77 + t, 65, *cases.ALL_ORDERS[3], strided=True, name="packed"),
+                 W.random_problem(rng, S.I8, S.I8, S.I32, S.I32, 2000, 1500 + 16 * t, 6, *cases.RCC, name="skinny"),
+                 W.random_problem(rng, S.F32, S.F32, S.F32, S.F32, 200, 100, 150 + t, *cases.RCC, name="f32"),
+                 W.config_int8_gemv(1024, N=1, weight_seed=t)]
+        jobs.append([(p, expected(p)) for p in probs])
+    errors = []
+
+    def worker(my_jobs):
+        try:
+            ctx = api.Context()
+            try:
+                for _ in range(6):
+                    for p, want in my_jobs:
+                        compare(p, D.device_mul(ctx, p), want)
+            finally:
+                ctx.close()
+        except BaseException as e:  # reported by the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(j,)) for j in jobs]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
 
 
 @pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I16),
