@@ -209,8 +209,21 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // the end of the depth are issued too (they fetch zeros) so that the number
   // of loads in flight, which the vmcnt waits count, never depends on K.
   // Load number n (0 .. kLoadsPerStage-1) of depth step kt: A loads first.
+  // Small tiles only (grids of one round of workgroups): every tile row walks
+  // the depth from its own starting step and wraps around, so that workgroups
+  // running side by side do not ask the same memory channels at the same
+  // time. The order of the steps does not matter for the sums. Steps past the
+  // end keep their index, which puts them out of range as before.
+  const int k_tiles = (K + kBK - 1) / kBK;
+  constexpr bool kRotateDepth = WM * WN <= 4;
+  const int rot = kRotateDepth && K % kBK == 0 ? (tile_m * 5) % k_tiles : 0;
+  auto phys = [&](int kt) {
+    if constexpr (!kRotateDepth) return kt;
+    const int p = kt + rot;
+    return kt >= k_tiles ? kt : p >= k_tiles ? p - k_tiles : p;
+  };
   auto issue_one = [&](int kt, int n) {
-    const int kbase = kt * kBK;
+    const int kbase = phys(kt) * kBK;
     const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
     if (n < C::kALoads) {
       const uint32_t off = (kbase + a_k[n] < K) ? a_goff[n] + kbase : kOutOfRange;
@@ -225,7 +238,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // per-granule test, and the step's depth offset travels as the instruction's
   // scalar offset, so nothing but the load itself is issued.
   auto issue_one_full = [&](int kt, int n) {
-    const uint32_t kbase = kt * kBK;
+    const uint32_t kbase = phys(kt) * kBK;
     const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
     if (n < C::kALoads) {
       LoadToLds16(stage + (wave * C::kALoads + n) * 1024, a_goff[n], kbase, a_rsrc);
@@ -316,8 +329,6 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-
-  const int k_tiles = (K + kBK - 1) / kBK;
 
   // ---- software pipeline ----
   // Fragments are double-buffered in registers: while the matrix instructions
@@ -498,13 +509,29 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
   return ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
 }
 
-// Largest tile that still gives every CU something to do.
+// Picks the tile by a small cost model: workgroups are dealt to the CUs in
+// rounds, a round of a given tile costs its area divided by how well that tile
+// feeds the matrix cores (a wave of the 64x64 tile reads one LDS fragment pair
+// per matrix instruction and is LDS-bound at about half rate; 128x128 reaches
+// about 0.8 of the 256x256 tile). Large tiles win when there are many rounds,
+// small tiles when the last (or only) round would leave most CUs idle.
 template <typename Traits>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
-  if (TileCount(args, 256, 256) >= num_cus) return Launch<Traits, 4, 4, 128, 2>(stream, args);
-  if (TileCount(args, 128, 128) >= num_cus || Traits::kSplitB) return Launch<Traits, 2, 2, 128, 3>(stream, args);
-  if constexpr (!Traits::kSplitB) return Launch<Traits, 1, 1, 128, 4>(stream, args);
-  return hipErrorInvalidValue;
+  auto cost = [&](int bm, int bn, double efficiency) {
+    const int rounds = (TileCount(args, bm, bn) + num_cus - 1) / num_cus;
+    return rounds * double(bm) * double(bn) / efficiency;
+  };
+  const double c256 = cost(256, 256, 1.0);
+  const double c128 = cost(128, 128, 0.8);
+  if constexpr (Traits::kSplitB) {
+    // The split-operand form has no 64x64 instantiation.
+    return c256 <= c128 ? Launch<Traits, 4, 4, 128, 2>(stream, args) : Launch<Traits, 2, 2, 128, 3>(stream, args);
+  } else {
+    const double c64 = cost(64, 64, 0.5);
+    if (c256 <= c128 && c256 <= c64) return Launch<Traits, 4, 4, 128, 2>(stream, args);
+    if (c128 <= c64) return Launch<Traits, 2, 2, 128, 3>(stream, args);
+    return Launch<Traits, 1, 1, 128, 4>(stream, args);
+  }
 }
 
 }  // namespace mfma_gemm
