@@ -76,17 +76,29 @@ __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
 #pragma unroll
     for (int j = 0; j < NB; ++j) acc[r][j] = 0;
 
+  // The depth is walked in steps of 1024 bytes starting from a step that
+  // differs from wave to wave and wrapping around (the order does not matter
+  // for the sums), so that waves running side by side spread over the memory
+  // channels. Logical positions past the depth stay out of range.
+  const int k_ceil = (K + 1023) & ~1023;
+  const int rot = (((blockIdx.x * kWaves + wave) * 5) % max(k_ceil >> 10, 1)) << 10;
+  auto phys = [&](int k0) {
+    const int p = k0 + rot;
+    return k0 >= k_ceil ? k0 : p >= k_ceil ? p - k_ceil : p;
+  };
   auto load_wide = [&](int k0, v4i (&w)[kRowsPerWave]) {
-    const bool in = k0 + lane * 16 < K;
+    const int kp = phys(k0);
+    const bool in = kp + lane * 16 < K;
 #pragma unroll
     for (int r = 0; r < kRowsPerWave; ++r)
-      w[r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, in ? w_off[r] + k0 : kOutOfRange, 0, 0);
+      w[r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, in ? w_off[r] + kp : kOutOfRange, 0, 0);
   };
   auto load_narrow = [&](int k0, v4i (&n)[NB]) {
-    const bool in = k0 + lane * 16 < K;
+    const int kp = phys(k0);
+    const bool in = kp + lane * 16 < K;
 #pragma unroll
     for (int j = 0; j < NB; ++j)
-      n[j] = __builtin_amdgcn_raw_buffer_load_b128(n_rsrc, in ? n_off[j] + k0 : kOutOfRange, 0, 0);
+      n[j] = __builtin_amdgcn_raw_buffer_load_b128(n_rsrc, in ? n_off[j] + kp : kOutOfRange, 0, 0);
   };
   auto fma_all = [&](const v4i (&w)[kRowsPerWave], const v4i (&n)[NB]) {
 #pragma unroll
