@@ -511,9 +511,9 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
 
 // Picks the tile by a small cost model: workgroups are dealt to the CUs in
 // rounds, a round of a given tile costs its area divided by how well that tile
-// feeds the matrix cores (a wave of the 64x64 tile reads one LDS fragment pair
-// per matrix instruction and is LDS-bound at about half rate; 128x128 reaches
-// about 0.8 of the 256x256 tile). Large tiles win when there are many rounds,
+// feeds the matrix cores (measured on int8: the 128x128 tile sustains about
+// 0.65 and the 64x64 tile, whose waves read one LDS fragment pair per matrix
+// instruction, about 0.45 of the 256x256 tile's rate). Large tiles win when there are many rounds,
 // small tiles when the last (or only) round would leave most CUs idle.
 template <typename Traits>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
@@ -522,14 +522,14 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
     return rounds * double(bm) * double(bn) / efficiency;
   };
   const double c256 = cost(256, 256, 1.0);
-  const double c128 = cost(128, 128, 0.8);
+  const double c128 = cost(128, 128, 0.65);
   if constexpr (Traits::kSplitB) {
     // The split-operand form has no 64x64 instantiation.
-    return c256 <= c128 ? Launch<Traits, 4, 4, 128, 2>(stream, args) : Launch<Traits, 2, 2, 128, 3>(stream, args);
+    return c256 <= c128 ? Launch<Traits, 4, 4, 128, 2>(stream, args) : Launch<Traits, 2, 2, 128, 4>(stream, args);
   } else {
-    const double c64 = cost(64, 64, 0.5);
+    const double c64 = cost(64, 64, 0.45);
     if (c256 <= c128 && c256 <= c64) return Launch<Traits, 4, 4, 128, 2>(stream, args);
-    if (c128 <= c64) return Launch<Traits, 2, 2, 128, 3>(stream, args);
+    if (c128 <= c64) return Launch<Traits, 2, 2, 128, 4>(stream, args);
     return Launch<Traits, 1, 1, 128, 4>(stream, args);
   }
 }
