@@ -40,6 +40,8 @@
 
 #include <type_traits>
 
+#include <algorithm>
+
 #include "../epilogue.h"
 #include "../internal.h"
 #include "gemm_i8.h"
@@ -209,13 +211,13 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // the end of the depth are issued too (they fetch zeros) so that the number
   // of loads in flight, which the vmcnt waits count, never depends on K.
   // Load number n (0 .. kLoadsPerStage-1) of depth step kt: A loads first.
-  // Small tiles only (grids of one round of workgroups): every tile row walks
+  // All tiles but the largest (grids of few rounds of workgroups): every tile row walks
   // the depth from its own starting step and wraps around, so that workgroups
   // running side by side do not ask the same memory channels at the same
   // time. The order of the steps does not matter for the sums. Steps past the
   // end keep their index, which puts them out of range as before.
   const int k_tiles = (K + kBK - 1) / kBK;
-  constexpr bool kRotateDepth = WM * WN <= 4;
+  constexpr bool kRotateDepth = WM * WN < 16;
   const int rot = kRotateDepth && K % kBK == 0 ? (tile_m * 5) % k_tiles : 0;
   auto phys = [&](int kt) {
     if constexpr (!kRotateDepth) return kt;
@@ -515,6 +517,7 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
 // 0.65 and the 64x64 tile, whose waves read one LDS fragment pair per matrix
 // instruction, about 0.45 of the 256x256 tile's rate). Large tiles win when there are many rounds,
 // small tiles when the last (or only) round would leave most CUs idle.
+constexpr double kEff256x128 = 0.75;  // measured, like the figures below
 template <typename Traits>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
   auto cost = [&](int bm, int bn, double efficiency) {
@@ -528,8 +531,13 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
     return c256 <= c128 ? Launch<Traits, 4, 4, 128, 2>(stream, args) : Launch<Traits, 2, 2, 128, 4>(stream, args);
   } else {
     const double c64 = cost(64, 64, 0.45);
-    if (c256 <= c128 && c256 <= c64) return Launch<Traits, 4, 4, 128, 2>(stream, args);
-    if (c128 <= c64) return Launch<Traits, 2, 2, 128, 4>(stream, args);
+    const double c256x128 = cost(256, 128, kEff256x128);
+    const double c128x256 = cost(128, 256, kEff256x128);
+    const double best = std::min(std::min(c256, c128), std::min(c64, std::min(c256x128, c128x256)));
+    if (c256 == best) return Launch<Traits, 4, 4, 128, 2>(stream, args);
+    if (c256x128 == best) return Launch<Traits, 4, 2, 128, 3>(stream, args);
+    if (c128x256 == best) return Launch<Traits, 2, 4, 128, 3>(stream, args);
+    if (c128 == best) return Launch<Traits, 2, 2, 128, 4>(stream, args);
     return Launch<Traits, 1, 1, 128, 4>(stream, args);
   }
 }

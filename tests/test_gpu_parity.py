@@ -414,6 +414,22 @@ def test_skinny_shapes_both_orientations(device_ctx, tup):
             assert device_ctx.last_kernel_name() == ("f32_gemv" if tup[0] == S.F32 else "i8_gemv")
 
 
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I32),
+                                 (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
+def test_shapes_that_take_the_rectangular_and_large_tiles(device_ctx, tup):
+    """Destination sizes for which the tile cost model picks the 256x128, the
+    128x256, the 128x128 and the 256x256 tile (on 256 CUs), with shallow depths
+    so that the checker stays fast; ragged edges in both dimensions."""
+    rng = np.random.default_rng(77)
+    for shape in [(4096, 200, 2048), (1920, 136, 4352), (1790, 100, 1795), (4000, 72, 4100), (4096, 64, 4096)]:
+        for orders in (cases.RCC, cases.ALL_ORDERS[int(rng.integers(8))]):
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=bool(rng.integers(2)),
+                                 name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
+
+
 def test_two_contexts_on_two_threads():
     """The reference's rule (ruy/ruy.h:82-95): a Context serves one thread, and
     concurrent Mul calls need distinct Contexts. Two threads, each with its own
