@@ -186,6 +186,17 @@ RUYAMD_API void ruyamd_ctx_set_explicit_tuning(ruyamd_ctx* ctx, int value);
 RUYAMD_API int ruyamd_ctx_num_threads_strategy(const ruyamd_ctx* ctx);
 RUYAMD_API void ruyamd_ctx_set_num_threads_strategy(ruyamd_ctx* ctx,
                                                     int value);
+/* Advisory bits of the last ruyamd_mul (ruy/performance_advisory.h:21-38,
+ * cleared at the start of each call like ruy/frontend.h:86). Bit 0x1,
+ * kReallocatedPerChannelBuffer, is never raised here. Bit 0x100 has no
+ * counterpart in the reference: an operand or the destination was host memory
+ * and travelled over PCIe inside the call (a cached operand that was found in
+ * the prepacked cache does not travel and does not raise it). */
+enum {
+  RUYAMD_ADVISORY_NONE = 0,
+  RUYAMD_ADVISORY_REALLOCATED_PERCHANNEL_BUFFER = 0x1,
+  RUYAMD_ADVISORY_STAGED_THROUGH_HOST = 0x100
+};
 RUYAMD_API int ruyamd_ctx_performance_advisory(const ruyamd_ctx* ctx,
                                                int advisory);
 

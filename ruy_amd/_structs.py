@@ -10,6 +10,7 @@ U8, I8, I16, I32, F32, F64 = 1, 2, 3, 4, 5, 6
 CACHE_NEVER, CACHE_IF_LARGE_SPEEDUP, CACHE_IF_SIGNIFICANT_SPEEDUP, CACHE_ALWAYS = 0, 1, 2, 3
 CHANNEL_ROW, CHANNEL_COL = 0, 1
 PATH_NONE, PATH_STANDARD_CPP, PATH_GFX950 = 0, 0x1, 0x10
+ADVISORY_REALLOCATED_PERCHANNEL_BUFFER, ADVISORY_STAGED_THROUGH_HOST = 0x1, 0x100
 OK, E_INVALID, E_UNSUPPORTED, E_HIP, E_NO_PATH, E_NO_DEVICE = 0, 1, 2, 3, 4, 5
 
 KERNEL_NAMES = {

@@ -56,6 +56,154 @@ void Workspace::Reset() {
   for (auto& b : blocks_) b.used = 0;
 }
 
+HostStaging::~HostStaging() {
+  if (!pinned_) return;
+  for (int c = 0; c < kChunks; ++c) (void)hipEventDestroy(done_[c]);
+  (void)hipHostFree(pinned_);
+}
+
+bool HostStaging::Init() {
+  if (pinned_) return true;
+  void* p = nullptr;
+  if (hipHostMalloc(&p, kChunks * kChunkBytes, hipHostMallocDefault) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  for (int c = 0; c < kChunks; ++c) {
+    if (hipEventCreateWithFlags(&done_[c], hipEventDisableTiming) != hipSuccess) {
+      for (int d = 0; d < c; ++d) (void)hipEventDestroy(done_[d]);
+      (void)hipHostFree(p);
+      return false;
+    }
+  }
+  pinned_ = static_cast<char*>(p);
+  return true;
+}
+
+bool HostStaging::WaitFree(int c) {
+  if (!busy_[c]) return true;
+  if (hipEventSynchronize(done_[c]) != hipSuccess) return false;
+  busy_[c] = false;
+  return true;
+}
+
+bool HostStaging::RetireCurrent(hipStream_t stream) {
+  if (fill_ == 0) return true;
+  if (hipEventRecord(done_[current_], stream) != hipSuccess) return false;
+  busy_[current_] = true;
+  current_ = (current_ + 1) % kChunks;
+  fill_ = 0;
+  return true;
+}
+
+namespace {
+// Page-locked host memory (hipHostMalloc, torch's pinned tensors): the copy
+// engine reaches it directly, no staging needed.
+bool IsPinnedHost(const void* p) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+    (void)hipGetLastError();  // ordinary pageable memory
+    return false;
+  }
+  return attr.type == hipMemoryTypeHost;
+}
+}  // namespace
+
+bool HostStaging::ToDevice(void* dst_dev, const void* src_host, std::size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return true;
+  if (IsPinnedHost(src_host))
+    return hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, stream) == hipSuccess;
+  if (!Init()) return false;
+  const char* src = static_cast<const char*>(src_host);
+  char* dst = static_cast<char*>(dst_dev);
+  while (bytes > 0) {
+    // Keep pieces 256-byte aligned inside a chunk.
+    const std::size_t at = (fill_ + 255) & ~std::size_t(255);
+    if (at >= kChunkBytes || (bytes <= kChunkBytes && at + bytes > kChunkBytes)) {
+      // Does not fit behind what the chunk already holds: move on to the next.
+      if (!RetireCurrent(stream)) return false;
+      continue;
+    }
+    if (at == 0 && fill_ == 0 && !WaitFree(current_)) return false;
+    const std::size_t n = bytes < kChunkBytes - at ? bytes : kChunkBytes - at;
+    char* piece = pinned_ + std::size_t(current_) * kChunkBytes + at;
+    std::memcpy(piece, src, n);
+    if (hipMemcpyAsync(dst, piece, n, hipMemcpyHostToDevice, stream) != hipSuccess) return false;
+    fill_ = at + n;
+    src += n;
+    dst += n;
+    bytes -= n;
+    if (fill_ >= kChunkBytes && !RetireCurrent(stream)) return false;
+  }
+  return true;
+}
+
+bool HostStaging::ToHost2D(void* dst_host, const void* src_dev, std::size_t pitch, std::size_t inner_bytes,
+                           std::size_t outer, hipStream_t stream) {
+  if (inner_bytes == 0 || outer == 0) return true;
+  if (IsPinnedHost(dst_host)) {
+    // Stream-ordered; complete once the caller has synchronised the stream.
+    if (pitch == inner_bytes || outer == 1)
+      return hipMemcpyAsync(dst_host, src_dev, pitch * (outer - 1) + inner_bytes, hipMemcpyDeviceToHost,
+                            stream) == hipSuccess;
+    return hipMemcpy2DAsync(dst_host, pitch, src_dev, pitch, inner_bytes, outer, hipMemcpyDeviceToHost,
+                            stream) == hipSuccess;
+  }
+  if (!Init()) return false;
+  // The chunk that ToDevice was filling carries copies that are still in flight.
+  if (!RetireCurrent(stream)) return false;
+  const std::size_t total = pitch * (outer - 1) + inner_bytes;  // extent of the image
+  const char* src = static_cast<const char*>(src_dev);
+  char* dst = static_cast<char*>(dst_host);
+  struct Piece {
+    std::size_t begin, size;
+    int chunk;
+  };
+  Piece in_flight[kChunks];
+  int head = 0, count = 0;  // ring of pieces whose device-to-host copy was issued
+  std::size_t issued = 0;
+  auto land = [&](const Piece& pc) {
+    if (hipEventSynchronize(done_[pc.chunk]) != hipSuccess) return false;
+    busy_[pc.chunk] = false;
+    const char* from = pinned_ + std::size_t(pc.chunk) * kChunkBytes;
+    // Copy the parts of the runs that lie inside [begin, begin + size).
+    const std::size_t end = pc.begin + pc.size;
+    for (std::size_t run = pc.begin / pitch; run < outer && run * pitch < end; ++run) {
+      const std::size_t lo = run * pitch > pc.begin ? run * pitch : pc.begin;
+      const std::size_t run_end = run * pitch + inner_bytes;
+      const std::size_t hi = run_end < end ? run_end : end;
+      if (hi > lo) std::memcpy(dst + lo, from + (lo - pc.begin), hi - lo);
+    }
+    return true;
+  };
+  while (issued < total || count > 0) {
+    if (issued < total && count < kChunks - 1) {
+      const int c = current_;
+      if (!WaitFree(c)) return false;
+      const std::size_t n = total - issued < kChunkBytes ? total - issued : kChunkBytes;
+      if (hipMemcpyAsync(pinned_ + std::size_t(c) * kChunkBytes, src + issued, n, hipMemcpyDeviceToHost,
+                         stream) != hipSuccess)
+        return false;
+      if (hipEventRecord(done_[c], stream) != hipSuccess) return false;
+      busy_[c] = true;
+      in_flight[(head + count) % kChunks] = Piece{issued, n, c};
+      ++count;
+      issued += n;
+      current_ = (current_ + 1) % kChunks;
+      continue;
+    }
+    if (!land(in_flight[head])) return false;
+    head = (head + 1) % kChunks;
+    --count;
+  }
+  return true;
+}
+
+void HostStaging::Reset() {
+  for (int c = 0; c < kChunks; ++c) busy_[c] = false;
+  fill_ = 0;
+}
+
 }  // namespace ruyamd
 
 using ruyamd::PrepackedCache;

@@ -48,6 +48,42 @@ class Workspace {
   bool growth_allowed_ = true;
 };
 
+// Moves pageable host memory to and from the device through a small ring of
+// pinned chunks: the CPU copies into (out of) a chunk while the copy engine
+// works on the previous ones, and every transfer the engine sees is a true
+// asynchronous pinned copy. Small operands share a chunk. Host memory that is
+// already page-locked skips the chunks and is copied directly. Used only by calls
+// that were handed host pointers; such a call ends with a stream
+// synchronisation, after which Reset() makes all chunks available again.
+class HostStaging {
+ public:
+  ~HostStaging();
+  // dst_dev[0, bytes) = src_host[0, bytes), ordered on `stream`.
+  bool ToDevice(void* dst_dev, const void* src_host, std::size_t bytes, hipStream_t stream);
+  // Copies `outer` runs of `inner_bytes`, `pitch` bytes apart in both images,
+  // from device to host after everything already enqueued on `stream`; the
+  // bytes between the runs of the host image are not written. The host image
+  // is complete when this returns (pageable destination) or once the stream
+  // has been synchronised (page-locked destination, copied directly).
+  bool ToHost2D(void* dst_host, const void* src_dev, std::size_t pitch, std::size_t inner_bytes,
+                std::size_t outer, hipStream_t stream);
+  // Call after the stream has been synchronised.
+  void Reset();
+
+ private:
+  static constexpr std::size_t kChunkBytes = std::size_t(4) << 20;
+  static constexpr int kChunks = 4;
+  bool Init();
+  // Makes chunk c reusable: waits for the transfer that last used it.
+  bool WaitFree(int c);
+  bool RetireCurrent(hipStream_t stream);
+  char* pinned_ = nullptr;
+  hipEvent_t done_[kChunks] = {};
+  bool busy_[kChunks] = {};
+  int current_ = 0;            // chunk being filled by ToDevice
+  std::size_t fill_ = 0;       // bytes of it already handed to the copy engine
+};
+
 }  // namespace ruyamd
 
 struct ruyamd_ctx {
@@ -66,6 +102,7 @@ struct ruyamd_ctx {
   bool force_generic = false;
   std::string last_error;
   ruyamd::Workspace workspace;
+  ruyamd::HostStaging staging;
   std::unique_ptr<ruyamd::PrepackedCache> cache;
   int multiprocessor_count = 0;
   // Optional timing of the dominant kernel of each call.

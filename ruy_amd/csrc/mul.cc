@@ -112,7 +112,7 @@ int64_t StorageElements(const ruyamd_mat& m) {
 const void* StageIn(ruyamd_ctx* ctx, const void* p, std::size_t bytes, bool* staged_any, bool* ok) {
   if (!p || bytes == 0 || IsDevicePointer(p)) return p;
   void* d = ctx->workspace.Alloc(bytes);
-  if (!d || hipMemcpyAsync(d, p, bytes, hipMemcpyHostToDevice, ctx->stream) != hipSuccess) {
+  if (!d || !ctx->staging.ToDevice(d, p, bytes, ctx->stream)) {
     *ok = false;
     return nullptr;
   }
@@ -280,14 +280,18 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
     const std::size_t inner = dst->order == RUYAMD_ORDER_COL_MAJOR ? dst->rows : dst->cols;
     const std::size_t outer = dst->order == RUYAMD_ORDER_COL_MAJOR ? dst->cols : dst->rows;
     const std::size_t pitch = std::size_t(dst->stride) * dst_elt;
-    if (hipMemcpy2DAsync(dst->data, pitch, dst_d, pitch, inner * dst_elt, outer,
-                         hipMemcpyDeviceToHost, ctx->stream) != hipSuccess)
-      return Fail(ctx, RUYAMD_E_HIP, "copying the destination back to the host failed");
+    if (!ctx->staging.ToHost2D(dst->data, dst_d, pitch, inner * dst_elt, outer, ctx->stream))
+      return Fail(ctx, RUYAMD_E_HIP, std::string("copying the destination back to the host failed: ") +
+                                         hipGetErrorString(hipGetLastError()));
     staged = true;
   }
   if ((ctx->synchronous || staged) && !ctx->capturing) {
     if (hipStreamSynchronize(ctx->stream) != hipSuccess)
       return Fail(ctx, RUYAMD_E_HIP, std::string("kernel execution failed: ") + hipGetErrorString(hipGetLastError()));
+  }
+  if (staged) {
+    ctx->staging.Reset();
+    ctx->performance_advisories |= RUYAMD_ADVISORY_STAGED_THROUGH_HOST;
   }
   return RUYAMD_OK;
 }
@@ -310,8 +314,9 @@ extern "C" int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x, const 
   if (!od) return Fail(ctx, RUYAMD_E_HIP, "device allocation failed");
   if (LaunchApplyMultiplier(ctx->stream, xd, md, ed, od, n) != hipSuccess)
     return Fail(ctx, RUYAMD_E_HIP, "launch failed");
-  if (!out_dev && hipMemcpyAsync(out, od, bytes, hipMemcpyDeviceToHost, ctx->stream) != hipSuccess)
+  if (!out_dev && !ctx->staging.ToHost2D(out, od, bytes, bytes, 1, ctx->stream))
     return Fail(ctx, RUYAMD_E_HIP, "copy back failed");
   if (hipStreamSynchronize(ctx->stream) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "kernel execution failed");
+  ctx->staging.Reset();
   return RUYAMD_OK;
 }

@@ -464,7 +464,7 @@ int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
   std::size_t& bytes = side == 0 ? call->lhs_host_bytes : call->rhs_host_bytes;
   if (bytes == 0) return RUYAMD_OK;
   void* d = ctx->workspace.Alloc(bytes);
-  if (!d || hipMemcpyAsync(d, m.data, bytes, hipMemcpyHostToDevice, ctx->stream) != hipSuccess) {
+  if (!d || !ctx->staging.ToDevice(d, m.data, bytes, ctx->stream)) {
     *err = "staging a host operand to the device failed";
     return RUYAMD_E_HIP;
   }

@@ -159,6 +159,40 @@ def test_host_pointer_operands(device_ctx):
         assert all(got.view(np.uint8).reshape(got.size, -1)[g, 0] == 0x77 for g in gaps)
 
 
+def test_large_host_pointer_operands_and_the_staging_advisory(device_ctx):
+    """Host operands larger than one pinned staging chunk (4 MiB) on both the
+    way in and the way out, a strided destination whose padding must survive,
+    and the advisory bit that tells a caller its data crossed PCIe in the call."""
+    import device_runner as D
+    rng = np.random.default_rng(55)
+    big = W.random_problem(rng, S.I8, S.I8, S.I32, S.I32, 1500, 5000, 1100, *cases.RCC, strided=True, name="big host")
+    want = expected(big, fill=0x33)
+    got = D.host_pointer_mul(device_ctx, big, dst_fill=0x33)   # 7.5 MB + 5.5 MB in, 6.6 MB out
+    compare(big, got, want)
+    assert device_ctx.performance_advisory(S.ADVISORY_STAGED_THROUGH_HOST)
+    assert not device_ctx.performance_advisory(S.ADVISORY_REALLOCATED_PERCHANNEL_BUFFER)
+    small = W.config_int8_gemm(64)
+    got, want = run_both(device_ctx, small)                     # device-resident: bit cleared again
+    compare(small, got, want)
+    assert not device_ctx.performance_advisory(S.ADVISORY_STAGED_THROUGH_HOST)
+    for _ in range(3):                                          # repeated host calls reuse the chunks
+        compare(small, D.host_pointer_mul(device_ctx, small, dst_fill=0x5A), want)
+    # page-locked host memory is copied directly, without the staging chunks
+    import ctypes as C
+    import torch
+    from ruy_amd import api
+    lhs_p, rhs_p = (torch.from_numpy(m.storage).clone().pin_memory() for m in (big.lhs, big.rhs))
+    out_p = torch.full((big.dst.n_storage,), 0x33333333, dtype=torch.int32).pin_memory()
+    l, r = big.lhs.struct(lhs_p.data_ptr()), big.rhs.struct(rhs_p.data_ptr())
+    d, ps = big.dst.struct(out_p.data_ptr()), big.params_struct()
+    device_ctx._check(api.lib.ruyamd_mul(device_ctx._h, C.byref(l), C.byref(r), C.byref(ps), C.byref(d)))
+    compare(big, out_p.numpy(), expected(big, fill=0x33))
+    assert device_ctx.performance_advisory(S.ADVISORY_STAGED_THROUGH_HOST)
+    # fp32 with a row-major strided destination, > 4 MiB out
+    f = W.random_problem(rng, S.F32, S.F32, S.F32, S.F32, 1200, 300, 1300, 1, 0, 1, strided=True, name="f32 host")
+    compare(f, D.host_pointer_mul(device_ctx, f, dst_fill=0), O.oracle_mul(f, fill=0))
+
+
 def test_empty_and_degenerate_shapes(device_ctx):
     import device_runner as D
     rng = np.random.default_rng(6)
