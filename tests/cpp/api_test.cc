@@ -53,6 +53,9 @@ static void TestExamples(ruy::Context* ctx) {
     ruy::MulParams<float, float> p;
     ruy::Mul(lhs, rhs, p, ctx, &dst);
     EXPECT(Is(d, 5, 11, 11, 25));
+    // Host vectors were handed over: the call staged them and says so.
+    EXPECT(ctx->performance_advisory(ruy::PerformanceAdvisory::kStagedThroughHost));
+    EXPECT(!ctx->performance_advisory(ruy::PerformanceAdvisory::kReallocatedPerChannelBuffer));
     const float bias[] = {1, 0};
     p.set_bias(bias);
     p.set_clamp_min(0);
