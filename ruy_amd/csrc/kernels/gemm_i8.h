@@ -36,8 +36,19 @@ struct GemmArgs {
   DevMat dst;
   int32_t dst_elt = 1;
   int32_t dst_vector_ok = 0;
+  // int8 kernel, small problems only (GemmI8CanFuseSums): when fuse_sums is
+  // set the kernel forms the depth sums of a's rows and b's columns itself
+  // and subtracts fused_a_factor * rowsum(i) + fused_b_factor * colsum(j)
+  // from accumulator (i, j); the caller then leaves the corresponding zero
+  // point of `ep` at 0 so that the write-back does not look for sums arrays.
+  int32_t fuse_sums = 0;
+  int32_t fused_a_factor = 0;
+  int32_t fused_b_factor = 0;
 };
 
+// True if LaunchGemmI8 would run these arguments on its smallest tile, the
+// one that has a variant with the sums fused in.
+bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmF32(hipStream_t stream, const GemmArgs& args, int num_cus);
 // int8 x int16: `b` is the int16 operand split by LaunchPackI16Split.

@@ -121,7 +121,15 @@ hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus
   return mfma_gemm::LaunchBest<Int8SplitTraits>(stream, args, num_cus);
 }
 
+bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
+  return mfma_gemm::PickTile(args, num_cus, false) == mfma_gemm::Tile::k64x64;
+}
+
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
+  if (args.fuse_sums) {
+    if (!GemmI8CanFuseSums(args, num_cus)) return hipErrorInvalidValue;
+    return mfma_gemm::Launch<Int8Traits, 1, 1, 128, 4, true>(stream, args);
+  }
   return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);
 }
 

@@ -143,8 +143,17 @@ struct Cfg {
       kStages * kStageBytes > kEpilogueBytes ? kStages * kStageBytes : kEpilogueBytes;
 };
 
-template <typename Traits, int WM, int WN, int BK, int STAGES>
+// kFusedSums (64x64 tile of the int8 kernel only): the kernel also forms the
+// depth sums of its rows of `a` and columns of `b` - one more matrix
+// instruction each per depth sub-step, against a fragment of ones - and
+// subtracts args.fused_a_factor * rowsum + args.fused_b_factor * colsum from
+// every accumulator before the write-back. This is the zero-point correction
+// of ruy/kernel.h:219-232 without a separate pass over the operands, for
+// problems so small that a second kernel launch would cost more than the
+// extra matrix instructions.
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false>
 __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
+  static_assert(!kFusedSums || WM * WN == 1, "fused sums exist for the single-block tile only");
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   constexpr int kBK = BK;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -296,6 +305,14 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
+  typename Traits::Acc sum_a, sum_b;  // kFusedSums: row sums of a / column sums of b, in every column / row
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    sum_a[v] = 0;
+    sum_b[v] = 0;
+  }
+  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+
   // One depth sub-step: the WM*WN matrix instructions on `cur`, with the LDS
   // reads of the next fragments (depth sub-step ks_next of ring step kt_next)
   // and, if kt_dma >= 0, the direct-to-LDS loads of ring step kt_dma dealt out
@@ -313,6 +330,10 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
     for (int n = 0; n < kMmas; ++n) {
       __builtin_amdgcn_sched_barrier(0);
       Traits::Mma(cur.a[n / WN], cur.b[n % WN], acc[n / WN][n % WN]);
+      if constexpr (kFusedSums) {
+        Traits::Mma(cur.a[0], ones, sum_a);
+        Traits::Mma(ones, cur.b[0], sum_b);
+      }
       __builtin_amdgcn_sched_barrier(0);
       if (n < kReadSlots) {
 #pragma unroll
@@ -367,6 +388,14 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type());
   WaitVmcnt<0>();
   __syncthreads();  // every wave is done with the operand ring
+  if constexpr (kFusedSums) {
+    const uint32_t fa = static_cast<uint32_t>(args.fused_a_factor);
+    const uint32_t fb = static_cast<uint32_t>(args.fused_b_factor);
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      acc[0][0][v] = static_cast<int>(static_cast<uint32_t>(acc[0][0][v]) - fa * static_cast<uint32_t>(sum_a[v]) -
+                                      fb * static_cast<uint32_t>(sum_b[v]));
+  }
 
   // ---- fused write-back ----
   // The destination is column-major here (rows contiguous; the host swaps the
@@ -488,7 +517,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   }
 }
 
-template <typename Traits, int WM, int WN, int BK, int STAGES>
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
@@ -496,7 +525,7 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int total = tiles_m * tiles_n;
   const int grid = ((total + 7) / 8) * 8;
   const size_t lds_bytes = C::kLdsBytes;
-  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES>;
+  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums>;
   if (lds_bytes > 48 * 1024) {
     // Once per process; static initialisation is safe against concurrent callers.
     static const hipError_t attr = hipFuncSetAttribute(
@@ -511,35 +540,56 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
   return ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
 }
 
+enum class Tile { k256x256, k256x128, k128x256, k128x128, k64x64 };
+
 // Picks the tile by a small cost model: workgroups are dealt to the CUs in
 // rounds, a round of a given tile costs its area divided by how well that tile
-// feeds the matrix cores (measured on int8: the 128x128 tile sustains about
-// 0.65 and the 64x64 tile, whose waves read one LDS fragment pair per matrix
-// instruction, about 0.45 of the 256x256 tile's rate). Large tiles win when there are many rounds,
-// small tiles when the last (or only) round would leave most CUs idle.
-constexpr double kEff256x128 = 0.75;  // measured, like the figures below
-template <typename Traits>
-hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
+// feeds the matrix cores (measured on int8: 256x128 sustains about 0.75, the
+// 128x128 tile about 0.65 and the 64x64 tile, whose waves read one LDS
+// fragment pair per matrix instruction, about 0.45 of the 256x256 tile's
+// rate). Large tiles win when there are many rounds, small tiles when the last
+// (or only) round would leave most CUs idle. `split_b`: the plane-split form
+// of the int16 kernel, which has the two square large tiles only.
+inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   auto cost = [&](int bm, int bn, double efficiency) {
     const int rounds = (TileCount(args, bm, bn) + num_cus - 1) / num_cus;
     return rounds * double(bm) * double(bn) / efficiency;
   };
   const double c256 = cost(256, 256, 1.0);
   const double c128 = cost(128, 128, 0.65);
-  if constexpr (Traits::kSplitB) {
-    // The split-operand form has no 64x64 instantiation.
-    return c256 <= c128 ? Launch<Traits, 4, 4, 128, 2>(stream, args) : Launch<Traits, 2, 2, 128, 4>(stream, args);
-  } else {
-    const double c64 = cost(64, 64, 0.45);
-    const double c256x128 = cost(256, 128, kEff256x128);
-    const double c128x256 = cost(128, 256, kEff256x128);
-    const double best = std::min(std::min(c256, c128), std::min(c64, std::min(c256x128, c128x256)));
-    if (c256 == best) return Launch<Traits, 4, 4, 128, 2>(stream, args);
-    if (c256x128 == best) return Launch<Traits, 4, 2, 128, 3>(stream, args);
-    if (c128x256 == best) return Launch<Traits, 2, 4, 128, 3>(stream, args);
-    if (c128 == best) return Launch<Traits, 2, 2, 128, 4>(stream, args);
-    return Launch<Traits, 1, 1, 128, 4>(stream, args);
+  if (split_b) return c256 <= c128 ? Tile::k256x256 : Tile::k128x128;
+  const double c64 = cost(64, 64, 0.45);
+  const double c256x128 = cost(256, 128, 0.75);
+  const double c128x256 = cost(128, 256, 0.75);
+  const double best = std::min(std::min(c256, c128), std::min(c64, std::min(c256x128, c128x256)));
+  if (c256 == best) return Tile::k256x256;
+  if (c256x128 == best) return Tile::k256x128;
+  if (c128x256 == best) return Tile::k128x256;
+  if (c128 == best) return Tile::k128x128;
+  return Tile::k64x64;
+}
+
+template <typename Traits>
+hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
+  switch (PickTile(args, num_cus, Traits::kSplitB)) {
+    case Tile::k256x256:
+      return Launch<Traits, 4, 4, 128, 2>(stream, args);
+    case Tile::k128x128:
+      return Launch<Traits, 2, 2, 128, 4>(stream, args);
+    default:
+      break;
   }
+  if constexpr (!Traits::kSplitB) {
+    switch (PickTile(args, num_cus, false)) {
+      case Tile::k256x128:
+        return Launch<Traits, 4, 2, 128, 3>(stream, args);
+      case Tile::k128x256:
+        return Launch<Traits, 2, 4, 128, 3>(stream, args);
+      default:
+        return Launch<Traits, 1, 1, 128, 4>(stream, args);
+    }
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace mfma_gemm

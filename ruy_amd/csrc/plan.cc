@@ -43,7 +43,27 @@ struct Operand8 {
   const int32_t* sums = nullptr;
   int32_t zero_point = 0;  // of the int8 form (uint8 zero point minus 128)
   uint32_t bytes = 0;
+  // An operand used in place whose sums are needed but have not been computed:
+  // the dispatcher either lets the kernel form them or calls MaterializeSums.
+  bool sums_pending = false;
+  int32_t count = 0;
 };
+
+int MaterializeSums(ruyamd_ctx* ctx, Operand8* op, int32_t K, std::string* err) {
+  if (!op->sums_pending) return RUYAMD_OK;
+  int32_t* sums = static_cast<int32_t*>(ctx->workspace.Alloc(std::size_t(op->count) * 4));
+  if (!sums) {
+    *err = "workspace allocation failed";
+    return RUYAMD_E_HIP;
+  }
+  if (LaunchSumsI8(ctx->stream, op->data, op->ld, op->count, K, sums) != hipSuccess) {
+    *err = "sums kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  op->sums = sums;
+  op->sums_pending = false;
+  return RUYAMD_OK;
+}
 
 // While the stream records a graph the cache may neither allocate nor eject:
 // a hit is pinned (the recorded kernels keep reading its buffers on every
@@ -126,18 +146,8 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
     out->data = static_cast<const int8_t*>(src.data);
     out->ld = src.count == 1 ? ld : static_cast<int32_t>(src.stride_c);
     out->bytes = static_cast<uint32_t>(extent);
-    if (need_sums) {
-      int32_t* sums = static_cast<int32_t*>(ctx->workspace.Alloc(std::size_t(src.count) * 4));
-      if (!sums) {
-        *err = "workspace allocation failed";
-        return RUYAMD_E_HIP;
-      }
-      if (LaunchSumsI8(ctx->stream, out->data, out->ld, src.count, K, sums) != hipSuccess) {
-        *err = "sums kernel launch failed";
-        return RUYAMD_E_HIP;
-      }
-      out->sums = sums;
-    }
+    out->sums_pending = need_sums;
+    out->count = src.count;
     return RUYAMD_OK;
   }
 
@@ -177,6 +187,8 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
       static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
   if (N <= kSkinnyWidthInt8 || M <= kSkinnyWidthInt8) {
     // Bandwidth-bound shapes: stream the wide side exactly once.
+    if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
+    if (int rc = MaterializeSums(ctx, &b, K, err)) return rc;
     GemvI8Args g;
     g.swapped = !(N <= kSkinnyWidthInt8 && (M > kSkinnyWidthInt8 || M >= N));
     const Operand8& wide = g.swapped ? b : a;
@@ -222,10 +234,27 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.M = swap ? N : M;
   args.N = swap ? M : N;
   args.n_logical = args.N;
-  args.ep.lhs_sums = x.sums;
-  args.ep.rhs_sums = y.sums;
   args.ep.lhs_zero_point = swap ? rzp : lzp;
   args.ep.rhs_zero_point = swap ? lzp : rzp;
+  if ((a.sums_pending || b.sums_pending) && GemmI8CanFuseSums(args, ctx->multiprocessor_count)) {
+    // A small problem on operands used in place: the kernel forms the pending
+    // sums itself (one launch instead of two or three). The zero point that
+    // multiplies a side's sums moves from the write-back to the fused factor.
+    args.fuse_sums = 1;
+    if (x.sums_pending) {
+      args.fused_a_factor = args.ep.rhs_zero_point;
+      args.ep.rhs_zero_point = 0;
+    }
+    if (y.sums_pending) {
+      args.fused_b_factor = args.ep.lhs_zero_point;
+      args.ep.lhs_zero_point = 0;
+    }
+  } else {
+    if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
+    if (int rc = MaterializeSums(ctx, &b, K, err)) return rc;
+  }
+  args.ep.lhs_sums = x.sums;
+  args.ep.rhs_sums = y.sums;
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
@@ -411,6 +440,7 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
                                side8 == 0 ? call->lhs_src_key : call->rhs_src_key,
                                side8 == 0 ? N : M, &a, err))
     return rc;
+  if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
   if (int rc = EnsureOnDevice(ctx, call, side16, err)) return rc;
   const DevMat& m16 = side16 == 0 ? call->lhs : call->rhs;
   const PackSource src = side16 == 0 ? PackSource{m16.data, m16.rs, m16.cs, m16.rows, m16.cols, m16.dtype}

@@ -70,11 +70,12 @@ def test_captured_calls_replay_correctly():
         dps = [D.DeviceProblem(p, dst_fill=0) for p in probs]
 
         # A capture before the first eager call has neither scratch memory nor
-        # cache entries to work with: the call must refuse and record nothing.
+        # cache entries to work with: a call that needs either (the packed
+        # uint8 product, the cached weight) must refuse and record nothing.
         cold = torch.cuda.CUDAGraph()
         refused = []
         with torch.cuda.graph(cold, stream=stream):
-            for dp in (dps[0], dps[4]):
+            for dp in (dps[1], dps[4]):
                 try:
                     dp.run(ctx)
                 except api.RuyAmdError as e:
