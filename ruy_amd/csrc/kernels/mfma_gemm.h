@@ -326,6 +326,15 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   constexpr int kReadSlots = kMmas < kFrags ? kMmas : kFrags;
   auto sub_step = [&](const Frags& cur, Frags& next, int kt_next, int ks_next, int kt_dma,
                       auto dma_is_full_step) {
+    // Few matrix instructions per sub-step: their run time does not cover the
+    // latency of an LDS read issued behind them, so the next fragments are
+    // requested first.
+    constexpr bool kReadsFirst = kMmas <= 4;
+    if constexpr (kReadsFirst) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < kFrags; ++r) read_one(kt_next, ks_next, r, next);
+    }
 #pragma unroll
     for (int n = 0; n < kMmas; ++n) {
       __builtin_amdgcn_sched_barrier(0);
@@ -335,7 +344,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
         Traits::Mma(ones, cur.b[0], sum_b);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (n < kReadSlots) {
+      if (!kReadsFirst && n < kReadSlots) {
 #pragma unroll
         for (int r = n * kFrags / kReadSlots; r < (n + 1) * kFrags / kReadSlots; ++r)
           read_one(kt_next, ks_next, r, next);
