@@ -220,8 +220,8 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
   if (!ok) return Fail(ctx, RUYAMD_E_HIP, "staging host operands to the device failed");
 
   // Destination: device memory is written in place; host memory gets a device
-  // image with the same stride that is copied back row by row (column by
-  // column), so the padding between them is never touched.
+  // image with the same stride of which only the rows (columns) themselves are
+  // copied back, so the padding between them is never touched.
   const bool dst_on_device = IsDevicePointer(dst->data);
   void* dst_d = dst->data;
   const std::size_t dst_elt = DtypeSize(dst->dtype);
