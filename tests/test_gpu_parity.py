@@ -568,3 +568,36 @@ def test_reference_slow_shape_list(device_ctx, tup):
             announce(p.name)
             got, want = run_both(device_ctx, p)
             compare(p, got, want)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_seeded_random_shapes(device_ctx, seed):
+    """A seeded random walk over the space the dispatcher divides up: sizes
+    around the tile and step edges (multiples of 16, 64, 128, 512 plus or minus
+    a little), every type tuple, random orders, strides, zero points, bias,
+    multipliers, channel dimension and cache policy. 60 problems per seed."""
+    rng = np.random.default_rng(1000 + seed)
+    edges = [1, 7, 8, 9, 16, 17, 31, 33, 63, 64, 65, 127, 128, 129, 255, 257, 511, 513]
+
+    def size(limit):
+        if rng.integers(3) == 0:
+            return int(rng.integers(1, limit + 1))
+        return int(min(limit, max(1, edges[int(rng.integers(len(edges)))] * int(rng.integers(1, 3))
+                                  + int(rng.integers(-2, 3)))))
+
+    for i in range(60):
+        tup = cases.TYPE_TUPLES[int(rng.integers(len(cases.TYPE_TUPLES)))]
+        fp64 = S.F64 in tup
+        limit = 200 if fp64 else 700
+        M, K, N = size(limit), size(1100 if not fp64 else 200), size(limit)
+        orders = cases.ALL_ORDERS[int(rng.integers(8))]
+        p = W.random_problem(rng, *tup, M, K, N, *orders, strided=bool(rng.integers(2)),
+                             name="seed %d #%d %s %dx%dx%d %s" % (seed, i, cases.tuple_name(tup), M, K, N, orders))
+        p.lhs.cache_policy = int(rng.integers(4))
+        p.rhs.cache_policy = int(rng.integers(4))
+        announce(p.name)
+        got, want = run_both(device_ctx, p)
+        compare(p, got, want)
+        # The cache trusts pointer equality (ruy/matrix.h:160-166) and the next
+        # problem's buffers may reuse these addresses.
+        device_ctx.clear_prepacked_cache()
