@@ -15,6 +15,10 @@ namespace ruyamd {
 // `a_bytes` / `b_bytes` (< 2^31) bound the buffer descriptors, so rows at or
 // past M / N read as zero. Elements are int8 (LaunchGemmI8) or fp32
 // (LaunchGemmF32).
+// uint8 data used in place: value - 128, which is what the int8 arithmetic
+// works on (ruy/pack_common.h:36-58), is the byte with its top bit flipped.
+constexpr uint32_t kFlipU8 = 0x80808080u;
+
 struct GemmArgs {
   const void* a = nullptr;
   const void* b = nullptr;
@@ -44,6 +48,12 @@ struct GemmArgs {
   int32_t fuse_sums = 0;
   int32_t fused_a_factor = 0;
   int32_t fused_b_factor = 0;
+  // int8 kernel, smallest tile only (GemmI8CanFuseSums): kFlipU8 for an
+  // operand that is uint8 data used in place, else 0. Bytes that the kernel
+  // reads as zero (past the depth) would turn into -128, so k_bytes must then
+  // be a multiple of 128, the kernel's depth step.
+  uint32_t a_flip = 0;
+  uint32_t b_flip = 0;
 };
 
 // True if LaunchGemmI8 would run these arguments on its smallest tile, the
@@ -71,9 +81,18 @@ struct GemvI8Args {
   int32_t narrow_count = 0;
   int32_t K = 0;
   int32_t swapped = 0;
+  // kFlipU8 for a side that is uint8 data used in place, else 0. K must then
+  // be a multiple of the kernel's depth step (GemvI8DepthStep), because bytes
+  // past the depth are read as zero and would turn into -128.
+  uint32_t wide_flip = 0;
+  uint32_t narrow_flip = 0;
   Epilogue ep;
   DevMat dst;
 };
+
+// Depth step of the skinny kernel that LaunchGemvI8 picks for this many
+// narrow vectors.
+int GemvI8DepthStep(int narrow_count);
 
 hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args);
 // fp32 version: the same argument block with K, ld_wide and ld_narrow counted
@@ -113,9 +132,10 @@ hipError_t LaunchPackI16Split(hipStream_t stream, const PackSource& src, int8_t*
 hipError_t LaunchPackF32(hipStream_t stream, const PackSource& src, float* dst, int32_t ld);
 
 // sums[c] = sum_k data[c*ld + k] for depth-contiguous int8 data with 16-byte
-// aligned base and ld, K a multiple of 16.
+// aligned base and ld, K a multiple of 16. With flip = kFlipU8 the bytes are
+// uint8 and the sums are those of value - 128.
 hipError_t LaunchSumsI8(hipStream_t stream, const int8_t* data, int32_t ld, int32_t count,
-                        int32_t K, int32_t* sums);
+                        int32_t K, int32_t* sums, uint32_t flip = 0);
 
 }  // namespace ruyamd
 

@@ -126,8 +126,14 @@ bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
 }
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
-  if (args.fuse_sums) {
-    if (!GemmI8CanFuseSums(args, num_cus)) return hipErrorInvalidValue;
+  const bool flip = args.a_flip != 0 || args.b_flip != 0;
+  if (args.fuse_sums || flip) {
+    // Both exist for the smallest tile only; flipped bytes need a whole number of depth steps.
+    if (!GemmI8CanFuseSums(args, num_cus) || (flip && args.k_bytes % 128 != 0)) return hipErrorInvalidValue;
+    if (flip) {
+      return args.fuse_sums ? mfma_gemm::Launch<Int8Traits, 1, 1, 128, 4, true, true>(stream, args)
+                            : mfma_gemm::Launch<Int8Traits, 1, 1, 128, 4, false, true>(stream, args);
+    }
     return mfma_gemm::Launch<Int8Traits, 1, 1, 128, 4, true>(stream, args);
   }
   return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);

@@ -49,7 +49,9 @@ __device__ __forceinline__ int WaveSum(int v) {
   return v;
 }
 
-template <int NB, int kRowsPerWave>
+// kFlip: args.wide_flip / args.narrow_flip are applied to the loaded bytes
+// (uint8 data used in place; the depth is then a whole number of steps).
+template <int NB, int kRowsPerWave, bool kFlip>
 __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -104,7 +106,13 @@ __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
 #pragma unroll
     for (int r = 0; r < kRowsPerWave; ++r)
 #pragma unroll
-      for (int j = 0; j < NB; ++j) acc[r][j] = Dot16(w[r], n[j], acc[r][j]);
+      for (int j = 0; j < NB; ++j) {
+        if constexpr (kFlip)
+          acc[r][j] = Dot16(w[r] ^ static_cast<int>(args.wide_flip), n[j] ^ static_cast<int>(args.narrow_flip),
+                            acc[r][j]);
+        else
+          acc[r][j] = Dot16(w[r], n[j], acc[r][j]);
+      }
   };
 
   // Two depth steps are in flight: the loads of step s+1 are issued before the
@@ -146,11 +154,11 @@ __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
   }
 }
 
-template <int NB, int R>
+template <int NB, int R, bool kFlip>
 void Launch(hipStream_t stream, const GemvI8Args& args) {
   const int rows_per_block = R * kWaves;
   const dim3 grid((args.rows + rows_per_block - 1) / rows_per_block);
-  hipLaunchKernelGGL((GemvI8Kernel<NB, R>), grid, dim3(64 * kWaves), 0, stream, args);
+  hipLaunchKernelGGL((GemvI8Kernel<NB, R, kFlip>), grid, dim3(64 * kWaves), 0, stream, args);
 }
 
 // 16 bytes per lane from the buffer straight to LDS at lds_base + 16*lane.
@@ -207,7 +215,7 @@ __device__ __forceinline__ void WaitVmcnt() {
 // workgroup; wave w walks the w-th part of the depth and the partial result
 // blocks are added through LDS at the end. kNarrow: narrow vectors staged, 8
 // or 16 (with 16 every column of the matrix instruction is a real one).
-template <int kRing, int kStep, int kSplit, int kNarrow>
+template <int kRing, int kStep, int kSplit, int kNarrow, bool kFlip>
 __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) {
   static_assert(kNarrow == 8 || kNarrow == 16, "");
   constexpr int kMmaVectors = kMmaRows + kNarrow;  // vectors per stage
@@ -271,6 +279,10 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
   const int q = lane >> 4;
   const bool narrow_lane = mv < kNarrow;
   v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+  // kFlip (uint8 data used in place): the lanes that read the slot of zeros
+  // keep their zeros.
+  const int a_flip = static_cast<int>(args.wide_flip);
+  const int b_flip = narrow_lane ? static_cast<int>(args.narrow_flip) : 0;
   auto consume = [&](int ring_slot) {
     const char* stage = lds + ring_slot * kStage;
     const char* a_row = stage + mv * kStep;
@@ -278,8 +290,12 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
 #pragma unroll
     for (int kb = 0; kb < kStep / 64; ++kb) {
       const int sl = ((kb * 4 + q) ^ (mv & 7)) * 16;
-      const v4i a = *reinterpret_cast<const v4i*>(a_row + sl);
-      const v4i b = *reinterpret_cast<const v4i*>(narrow_lane ? b_row + sl : lds + kZeroSlot);
+      v4i a = *reinterpret_cast<const v4i*>(a_row + sl);
+      v4i b = *reinterpret_cast<const v4i*>(narrow_lane ? b_row + sl : lds + kZeroSlot);
+      if constexpr (kFlip) {
+        a ^= a_flip;
+        b ^= b_flip;
+      }
       if (kb & 1)
         acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc1, 0, 0, 0);
       else
@@ -344,10 +360,10 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
   }
 }
 
-template <int kRing, int kStep, int kSplit, int kNarrow>
+template <int kRing, int kStep, int kSplit, int kNarrow, bool kFlip>
 hipError_t LaunchMma(hipStream_t stream, const GemvI8Args& args) {
   constexpr size_t lds_bytes = size_t(kSplit) * (size_t(kRing) * (kMmaRows + kNarrow) * kStep + 16);
-  auto kernel = GemvI8MmaKernel<kRing, kStep, kSplit, kNarrow>;
+  auto kernel = GemvI8MmaKernel<kRing, kStep, kSplit, kNarrow, kFlip>;
   if (lds_bytes > 48 * 1024) {
     // Once per process (thread-safe static initialisation).
     static const hipError_t attr = hipFuncSetAttribute(
@@ -359,21 +375,35 @@ hipError_t LaunchMma(hipStream_t stream, const GemvI8Args& args) {
   return hipGetLastError();
 }
 
+template <int kSplit, int kNarrow>
+hipError_t LaunchMmaFlip(hipStream_t stream, const GemvI8Args& args, bool flip) {
+  return flip ? LaunchMma<2, 512, kSplit, kNarrow, true>(stream, args)
+              : LaunchMma<2, 512, kSplit, kNarrow, false>(stream, args);
+}
+
 }  // namespace
+
+int GemvI8DepthStep(int narrow_count) { return narrow_count == 1 ? 1024 : 512; }
 
 hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
   if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
   // What the kernels assume: at most 16 narrow vectors, 16-byte granularity of
-  // the depth, of both pitches and of both base addresses.
+  // the depth, of both pitches and of both base addresses; whole depth steps
+  // when bytes are flipped on the way in.
+  const bool flip = args.wide_flip != 0 || args.narrow_flip != 0;
   if (args.narrow_count > 16 || args.K % 16 != 0 || args.ld_wide % 16 != 0 ||
       (args.narrow_count > 1 && args.ld_narrow % 16 != 0) ||
-      (reinterpret_cast<uintptr_t>(args.wide) | reinterpret_cast<uintptr_t>(args.narrow)) % 16 != 0)
+      (reinterpret_cast<uintptr_t>(args.wide) | reinterpret_cast<uintptr_t>(args.narrow)) % 16 != 0 ||
+      (flip && args.K % GemvI8DepthStep(args.narrow_count) != 0))
     return hipErrorInvalidValue;
   if (args.narrow_count == 1) {
     // One column: the dot-product kernel. Its many small waves are scheduled
     // dynamically and it streams a little faster than the matrix-core kernel
     // at every size measured.
-    Launch<1, 2>(stream, args);
+    if (flip)
+      Launch<1, 2, true>(stream, args);
+    else
+      Launch<1, 2, false>(stream, args);
     return hipGetLastError();
   }
   // Matrix-core kernel. With few groups of 16 wide vectors the depth is split
@@ -382,13 +412,13 @@ hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
   const int steps = (args.K + 511) / 512;
   const int split = groups >= 512 || steps < 4 ? 1 : steps < 8 ? 2 : 4;
   if (args.narrow_count <= 8) {
-    if (split == 1) return LaunchMma<2, 512, 1, 8>(stream, args);
-    if (split == 2) return LaunchMma<2, 512, 2, 8>(stream, args);
-    return LaunchMma<2, 512, 4, 8>(stream, args);
+    if (split == 1) return LaunchMmaFlip<1, 8>(stream, args, flip);
+    if (split == 2) return LaunchMmaFlip<2, 8>(stream, args, flip);
+    return LaunchMmaFlip<4, 8>(stream, args, flip);
   }
-  if (split == 1) return LaunchMma<2, 512, 1, 16>(stream, args);
-  if (split == 2) return LaunchMma<2, 512, 2, 16>(stream, args);
-  return LaunchMma<2, 512, 4, 16>(stream, args);
+  if (split == 1) return LaunchMmaFlip<1, 16>(stream, args, flip);
+  if (split == 2) return LaunchMmaFlip<2, 16>(stream, args, flip);
+  return LaunchMmaFlip<4, 16>(stream, args, flip);
 }
 
 }  // namespace ruyamd

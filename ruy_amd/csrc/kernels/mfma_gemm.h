@@ -151,9 +151,14 @@ struct Cfg {
 // of ruy/kernel.h:219-232 without a separate pass over the operands, for
 // problems so small that a second kernel launch would cost more than the
 // extra matrix instructions.
-template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false>
+//
+// kFlip (same tile only): args.a_flip / args.b_flip are applied to every
+// fragment before use, which turns uint8 data used in place into the int8
+// values the arithmetic is defined on.
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false>
 __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   static_assert(!kFusedSums || WM * WN == 1, "fused sums exist for the single-block tile only");
+  static_assert(!kFlip || WM * WN == 1, "in-place uint8 operands exist for the single-block tile only");
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   constexpr int kBK = BK;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -324,8 +329,14 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // The fragment reads go behind the first matrix instructions of the
   // sub-step, so that they have landed well before the next sub-step starts.
   constexpr int kReadSlots = kMmas < kFrags ? kMmas : kFrags;
-  auto sub_step = [&](const Frags& cur, Frags& next, int kt_next, int ks_next, int kt_dma,
+  auto sub_step = [&](const Frags& cur_raw, Frags& next, int kt_next, int ks_next, int kt_dma,
                       auto dma_is_full_step) {
+    Frags flipped;
+    if constexpr (kFlip) {
+      flipped.a[0] = cur_raw.a[0] ^ static_cast<int>(args.a_flip);
+      flipped.b[0] = cur_raw.b[0] ^ static_cast<int>(args.b_flip);
+    }
+    const Frags& cur = kFlip ? flipped : cur_raw;
     // Few matrix instructions per sub-step: their run time does not cover the
     // latency of an LDS read issued behind them, so the next fragments are
     // requested first.
@@ -526,7 +537,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   }
 }
 
-template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false>
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
@@ -534,7 +545,7 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int total = tiles_m * tiles_n;
   const int grid = ((total + 7) / 8) * 8;
   const size_t lds_bytes = C::kLdsBytes;
-  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums>;
+  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip>;
   if (lds_bytes > 48 * 1024) {
     // Once per process; static initialisation is safe against concurrent callers.
     static const hipError_t attr = hipFuncSetAttribute(

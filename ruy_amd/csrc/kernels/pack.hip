@@ -107,9 +107,140 @@ __global__ __launch_bounds__(256) void PackI8Kernel(PackSource src, int8_t* dst,
   }
 }
 
+// Depth-contiguous source (any alignment, any depth): one wave per vector (or
+// per part of a vector when there are few vectors) streams it 1024 bytes at a
+// time, 16 output bytes per lane. The source is read as aligned dwords - up
+// to five around the lane's 16 bytes - and brought into place with
+// v_alignbyte_b32, so no byte loads are needed for unaligned rows. A dword
+// may reach up to three bytes before or past the row, always inside an
+// aligned dword that also holds a byte of the row.
+__global__ __launch_bounds__(256) void PackI8RowsKernel(PackSource src, int8_t* dst, int32_t ld,
+                                                       int32_t* sums, int k_span) {
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (c >= src.count) return;
+  const uint8_t* row = static_cast<const uint8_t*>(src.data) + int64_t(c) * src.stride_c;
+  const uint32_t flip = src.dtype == RUYAMD_DTYPE_U8 ? 0x80808080u : 0u;
+  const int K = src.K;
+  const int k_begin = blockIdx.y * k_span;
+  const int k_end = min(k_begin + k_span, ld);
+  int8_t* out_row = dst + int64_t(c) * ld;
+  int32_t sum = 0;
+  for (int k = k_begin + lane * 16; k < k_end; k += 1024) {
+    v4i out = {0, 0, 0, 0};
+    if (k < K) {
+      const uintptr_t address = reinterpret_cast<uintptr_t>(row + k);
+      const int shift = static_cast<int>(address & 3);
+      const uint32_t* p = reinterpret_cast<const uint32_t*>(address - shift);
+      const int n = min(16, K - k);             // source bytes this lane needs
+      const int words = (shift + n + 3) >> 2;   // aligned dwords that hold them, 1..5
+      uint32_t d[5];
+#pragma unroll
+      for (int i = 0; i < 5; ++i) d[i] = i < words ? p[i] : 0u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t w = __builtin_amdgcn_alignbyte(d[i + 1], d[i], shift);
+        const int kd = k + 4 * i;
+        // Bytes past the depth are padding and stay 0 (they are not flipped either).
+        const uint32_t mask = kd + 4 <= K ? 0xffffffffu : kd >= K ? 0u : (0xffffffffu >> (8 * (kd + 4 - K)));
+        w = (w & mask) ^ (flip & mask);
+        out[i] = static_cast<int>(w);
+        sum = __builtin_amdgcn_sdot4(static_cast<int>(w), 0x01010101, sum, false);
+      }
+    }
+    *reinterpret_cast<v4i*>(out_row + k) = out;
+  }
+  if (sums) {
+    const int32_t total = WaveSum(sum);
+    if (lane == 0) {
+      if (gridDim.y == 1)
+        sums[c] = total;
+      else
+        atomicAdd(&sums[c], total);
+    }
+  }
+}
+
+// Source contiguous along the vectors (the transposed case) with a 4-byte
+// aligned base and pitch: a block moves a 64-vector x 64-depth tile per step.
+// Each thread loads four dwords (4 vectors x 4 consecutive depth positions),
+// transposes the 4x4 bytes in registers with v_perm_b32 and writes four
+// dwords to the LDS tile, from which the block writes depth-contiguous
+// 16-byte pieces as in the generic kernel.
+__global__ __launch_bounds__(256) void PackI8TransposeKernel(PackSource src, int8_t* dst, int32_t ld,
+                                                            int32_t* sums, int k_span) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kPitch];
+  const int tid = threadIdx.x;
+  const int c0 = blockIdx.x * kTileC;
+  const int k_begin = blockIdx.y * k_span;
+  const int k_end = min(k_begin + k_span, ld);
+  const uint8_t* s = static_cast<const uint8_t*>(src.data);
+  const uint32_t flip = src.dtype == RUYAMD_DTYPE_U8 ? 0x80808080u : 0u;
+  const int cq = tid & 15;   // quad of vectors
+  const int kq = tid >> 4;   // quad of depth positions
+  const int wc = tid >> 2;   // writer role: vector wc, 16-byte granule wg
+  const int wg = tid & 3;
+  int32_t sum = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += kTileK) {
+    uint32_t r[4];
+    const int cfirst = c0 + cq * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + kq * 4 + i;
+      r[i] = (cfirst < src.count && k < src.K)
+                 ? *reinterpret_cast<const uint32_t*>(s + int64_t(k) * src.stride_k + cfirst)
+                 : 0u;
+    }
+    // 4x4 byte transpose: t[j] = depth bytes k..k+3 of vector cfirst + j.
+    const uint32_t x0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);
+    const uint32_t x1 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
+    const uint32_t y0 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u);
+    const uint32_t y1 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+    uint32_t t[4];
+    t[0] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);
+    t[1] = __builtin_amdgcn_perm(y0, x0, 0x07060302u);
+    t[2] = __builtin_amdgcn_perm(y1, x1, 0x05040100u);
+    t[3] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<uint32_t*>(tile + (cq * 4 + j) * kPitch + kq * 4) = t[j];
+    __syncthreads();
+    const int c = c0 + wc;
+    const int k = k0 + wg * 16;
+    if (c < src.count && k < ld) {
+      const uint32_t* row = reinterpret_cast<const uint32_t*>(tile + wc * kPitch + wg * 16);
+      v4i out;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        uint32_t w = row[d];
+        const int kd = k + 4 * d;
+        const uint32_t mask = kd + 4 <= src.K ? 0xffffffffu : kd >= src.K ? 0u : (0xffffffffu >> (8 * (kd + 4 - src.K)));
+        w = (w & mask) ^ (flip & mask);
+        out[d] = static_cast<int>(w);
+        sum = __builtin_amdgcn_sdot4(static_cast<int>(w), 0x01010101, sum, false);
+      }
+      *reinterpret_cast<v4i*>(dst + int64_t(c) * ld + k) = out;
+    }
+    __syncthreads();
+  }
+  if (sums) {
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    const int c = c0 + wc;
+    if (wg == 0 && c < src.count) {
+      if (gridDim.y == 1)
+        sums[c] = sum;
+      else
+        atomicAdd(&sums[c], sum);
+    }
+  }
+}
+
 // One wave per vector, 16 bytes per lane per step.
+// `flip` = 0x80808080 for uint8 data used in place (value - 128 is the byte
+// with its top bit flipped, read as int8), 0 for int8 data.
 __global__ __launch_bounds__(256) void SumsI8Kernel(const int8_t* data, int32_t ld, int32_t count,
-                                                   int32_t K, int32_t* sums) {
+                                                   int32_t K, int32_t* sums, int32_t flip) {
   const int lane = threadIdx.x & 63;
   const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= count) return;
@@ -121,14 +252,14 @@ __global__ __launch_bounds__(256) void SumsI8Kernel(const int8_t* data, int32_t 
     const v4i y = *reinterpret_cast<const v4i*>(row + k + 1024);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      s0 = __builtin_amdgcn_sdot4(x[d], 0x01010101, s0, false);
-      s1 = __builtin_amdgcn_sdot4(y[d], 0x01010101, s1, false);
+      s0 = __builtin_amdgcn_sdot4(x[d] ^ flip, 0x01010101, s0, false);
+      s1 = __builtin_amdgcn_sdot4(y[d] ^ flip, 0x01010101, s1, false);
     }
   }
   for (; k < K; k += 1024) {
     const v4i x = *reinterpret_cast<const v4i*>(row + k);
 #pragma unroll
-    for (int d = 0; d < 4; ++d) s0 = __builtin_amdgcn_sdot4(x[d], 0x01010101, s0, false);
+    for (int d = 0; d < 4; ++d) s0 = __builtin_amdgcn_sdot4(x[d] ^ flip, 0x01010101, s0, false);
   }
   const int32_t total = WaveSum(s0 + s1);
   if (lane == 0) sums[c] = total;
@@ -240,6 +371,22 @@ hipError_t LaunchPackF32(hipStream_t stream, const PackSource& src, float* dst, 
 hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld,
                         int32_t* sums) {
   if (src.count == 0 || ld == 0) return hipSuccess;
+  if (src.stride_k == 1) {
+    // Depth-contiguous source: one wave per vector; with few vectors the depth
+    // is split so that some two thousand waves are in flight.
+    const int steps = (ld + 1023) / 1024;
+    int k_split = 1;
+    if (src.count < 2048 && steps > 1) k_split = min((2048 + src.count - 1) / src.count, steps);
+    const int steps_per = (steps + k_split - 1) / k_split;
+    k_split = (steps + steps_per - 1) / steps_per;
+    if (sums && k_split > 1) {
+      hipLaunchKernelGGL(ZeroI32Kernel, dim3((src.count + 255) / 256), dim3(256), 0, stream, sums,
+                         src.count);
+    }
+    hipLaunchKernelGGL(PackI8RowsKernel, dim3((src.count + 3) / 4, k_split), dim3(256), 0, stream, src,
+                       dst, ld, sums, steps_per * 1024);
+    return hipGetLastError();
+  }
   const int blocks_c = (src.count + kTileC - 1) / kTileC;
   // Split the depth when there are too few vector slabs to fill the device.
   int k_split = 1;
@@ -255,16 +402,24 @@ hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, 
     hipLaunchKernelGGL(ZeroI32Kernel, dim3((src.count + 255) / 256), dim3(256), 0, stream, sums,
                        src.count);
   }
-  hipLaunchKernelGGL(PackI8Kernel, dim3(blocks_c, k_split), dim3(256), 0, stream, src, dst, ld, sums,
-                     k_span);
+  // The transposed case: dword loads if base and pitch allow, bytes otherwise.
+  const bool aligned = src.stride_c == 1 && (reinterpret_cast<uintptr_t>(src.data) & 3) == 0 &&
+                       src.stride_k % 4 == 0;
+  if (aligned) {
+    hipLaunchKernelGGL(PackI8TransposeKernel, dim3(blocks_c, k_split), dim3(256), 0, stream, src, dst, ld,
+                       sums, k_span);
+  } else {
+    hipLaunchKernelGGL(PackI8Kernel, dim3(blocks_c, k_split), dim3(256), 0, stream, src, dst, ld, sums,
+                       k_span);
+  }
   return hipGetLastError();
 }
 
 hipError_t LaunchSumsI8(hipStream_t stream, const int8_t* data, int32_t ld, int32_t count, int32_t K,
-                        int32_t* sums) {
+                        int32_t* sums, uint32_t flip) {
   if (count == 0) return hipSuccess;
   hipLaunchKernelGGL(SumsI8Kernel, dim3((count + 3) / 4), dim3(256), 0, stream, data, ld, count, K,
-                     sums);
+                     sums, static_cast<int32_t>(flip));
   return hipGetLastError();
 }
 

@@ -47,6 +47,8 @@ struct Operand8 {
   // the dispatcher either lets the kernel form them or calls MaterializeSums.
   bool sums_pending = false;
   int32_t count = 0;
+  // kFlipU8 if `data` is the caller's uint8 storage used in place.
+  uint32_t flip = 0;
 };
 
 int MaterializeSums(ruyamd_ctx* ctx, Operand8* op, int32_t K, std::string* err) {
@@ -56,7 +58,7 @@ int MaterializeSums(ruyamd_ctx* ctx, Operand8* op, int32_t K, std::string* err) 
     *err = "workspace allocation failed";
     return RUYAMD_E_HIP;
   }
-  if (LaunchSumsI8(ctx->stream, op->data, op->ld, op->count, K, sums) != hipSuccess) {
+  if (LaunchSumsI8(ctx->stream, op->data, op->ld, op->count, K, sums, op->flip) != hipSuccess) {
     *err = "sums kernel launch failed";
     return RUYAMD_E_HIP;
   }
@@ -77,9 +79,11 @@ const char kCaptureCacheMiss[] =
 
 // Prepares one side: from the cache, in place, or packed into the workspace.
 // `src` views the side as `count` depth vectors (LHS rows / RHS columns).
+// `u8_depth_step`: uint8 data may be used in place (the kernel flips the top
+// bit of every byte) if the depth is a multiple of this; 0 = never.
 int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point, bool need_sums,
-                    int cache_policy, const void* src_key, int other_width, Operand8* out,
-                    std::string* err) {
+                    int cache_policy, const void* src_key, int other_width, int u8_depth_step,
+                    Operand8* out, std::string* err) {
   // View of the side as `count` depth vectors; its data pointer is only valid
   // on the device after EnsureOnDevice.
   auto view = [&]() {
@@ -139,7 +143,8 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
   // In place: already int8, depth-contiguous, 16-byte aligned base and pitch,
   // depth a multiple of 16, and small enough for a buffer descriptor.
   const uint64_t extent = src.count > 0 ? uint64_t(src.count - 1) * uint64_t(src.stride_c) + K : 0;
-  const bool direct = !is_u8 && src.stride_k == 1 && K % 16 == 0 && K > 0 &&
+  const bool u8_ok = !is_u8 || (u8_depth_step > 0 && K % u8_depth_step == 0);
+  const bool direct = u8_ok && src.stride_k == 1 && K % 16 == 0 && K > 0 &&
                       (reinterpret_cast<uintptr_t>(src.data) & 15) == 0 &&
                       (src.stride_c % 16 == 0 || src.count == 1) && extent < (uint64_t(1) << 31);
   if (direct) {
@@ -148,6 +153,7 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
     out->bytes = static_cast<uint32_t>(extent);
     out->sums_pending = need_sums;
     out->count = src.count;
+    out->flip = is_u8 ? kFlipU8 : 0;
     return RUYAMD_OK;
   }
 
@@ -175,17 +181,31 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const int32_t lzp = lhs.dtype == RUYAMD_DTYPE_U8 ? lhs.zero_point - 128 : lhs.zero_point;
   const int32_t rzp = rhs.dtype == RUYAMD_DTYPE_U8 ? rhs.zero_point - 128 : rhs.zero_point;
   Operand8 a, b;
+  // Which kernel will run decides whether uint8 storage can be used in place:
+  // the skinny kernels and the smallest tile of the tiled kernel flip bytes on
+  // the way in, provided the depth is a whole number of their depth steps.
+  const bool skinny = N <= kSkinnyWidthInt8 || M <= kSkinnyWidthInt8;
+  int u8_depth_step = 0;
+  if (skinny) {
+    const bool swapped = !(N <= kSkinnyWidthInt8 && (M > kSkinnyWidthInt8 || M >= N));
+    u8_depth_step = GemvI8DepthStep(swapped ? M : N);
+  } else {
+    GemmArgs shape;
+    shape.M = M;
+    shape.N = N;
+    if (GemmI8CanFuseSums(shape, ctx->multiprocessor_count)) u8_depth_step = 128;
+  }
   // Row sums of one side are needed iff the other side's zero point is not 0
   // (ruy/kernel.h:219-232).
   if (int rc = PrepareOperand8(ctx, call, 0, lhs.zero_point, rzp != 0, call->lhs_cache_policy,
-                               call->lhs_src_key, N, &a, err))
+                               call->lhs_src_key, N, u8_depth_step, &a, err))
     return rc;
   if (int rc = PrepareOperand8(ctx, call, 1, rhs.zero_point, lzp != 0, call->rhs_cache_policy,
-                               call->rhs_src_key, M, &b, err))
+                               call->rhs_src_key, M, u8_depth_step, &b, err))
     return rc;
   const int32_t zp_product_depth =
       static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
-  if (N <= kSkinnyWidthInt8 || M <= kSkinnyWidthInt8) {
+  if (skinny) {
     // Bandwidth-bound shapes: stream the wide side exactly once.
     if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
     if (int rc = MaterializeSums(ctx, &b, K, err)) return rc;
@@ -199,6 +219,8 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     g.narrow_bytes = narrow.bytes;
     g.ld_wide = wide.ld;
     g.ld_narrow = narrow.ld;
+    g.wide_flip = wide.flip;
+    g.narrow_flip = narrow.flip;
     g.rows = g.swapped ? N : M;
     g.narrow_count = g.swapped ? M : N;
     g.K = RoundUp(K, 16);
@@ -231,6 +253,8 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.b_bytes = y.bytes;
   args.lda = x.ld;
   args.ldb = y.ld;
+  args.a_flip = x.flip;
+  args.b_flip = y.flip;
   args.M = swap ? N : M;
   args.N = swap ? M : N;
   args.n_logical = args.N;
@@ -438,7 +462,7 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   if (int rc = PrepareOperand8(ctx, call, side8, 0, /*need_sums=*/true,
                                side8 == 0 ? call->lhs_cache_policy : call->rhs_cache_policy,
                                side8 == 0 ? call->lhs_src_key : call->rhs_src_key,
-                               side8 == 0 ? N : M, &a, err))
+                               side8 == 0 ? N : M, /*u8_depth_step=*/0, &a, err))
     return rc;
   if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
   if (int rc = EnsureOnDevice(ctx, call, side16, err)) return rc;

@@ -601,3 +601,30 @@ def test_seeded_random_shapes(device_ctx, seed):
         # The cache trusts pointer equality (ruy/matrix.h:160-166) and the next
         # problem's buffers may reuse these addresses.
         device_ctx.clear_prepacked_cache()
+
+
+@pytest.mark.parametrize("tup", [(S.U8, S.U8, S.I32, S.U8), (S.I8, S.U8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I32),
+                                 (S.U8, S.U8, S.I32, S.I16)], ids=cases.tuple_name)
+def test_uint8_operands_used_in_place(device_ctx, tup):
+    """uint8 operands whose depth is a whole number of the kernel's depth steps
+    are read where they lie (the kernels flip the top bit of every byte)
+    instead of being converted by a pack kernel first: the small tile of the
+    tiled kernel (depth % 128), the 2..16-column skinny kernel (depth % 512),
+    the one-column kernel (depth % 1024); neighbouring depths take the packed
+    route. Zero points are non-zero on both sides, so the sums see the flip too."""
+    rng = np.random.default_rng(4242)
+    shapes = [(200, 128, 300), (64, 1024, 64), (333, 384, 129), (200, 144, 300),          # tiled, small tile
+              (700, 512, 5), (5, 1024, 700), (900, 2048, 12), (16, 1536, 400), (700, 528, 5),  # 2..16 columns
+              (1000, 1024, 1), (1, 3072, 900), (1000, 1536, 1)]                           # one column
+    for shape in shapes:
+        for orders in (cases.RCC, (1, 0, 1)):
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=False,
+                                 name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+            # make sure the corrections that involve the sums are exercised
+            if p.lhs.zero_point in (0, 128) and tup[0] == S.U8:
+                p.lhs.zero_point = 121
+            if p.rhs.zero_point in (0, 128) and tup[1] == S.U8:
+                p.rhs.zero_point = 3
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
