@@ -131,6 +131,10 @@ hipError_t LaunchPackI16Split(hipStream_t stream, const PackSource& src, int8_t*
 // multiple of 4), zero-filled from K up to ld. `src.dtype` is fp32.
 hipError_t LaunchPackF32(hipStream_t stream, const PackSource& src, float* dst, int32_t ld);
 
+// dst(i, j) = src(i, j): same shape and element size, any two storage orders
+// (strides in elements).
+hipError_t LaunchReorder(hipStream_t stream, const DevMat& src, const DevMat& dst);
+
 // sums[c] = sum_k data[c*ld + k] for depth-contiguous int8 data with 16-byte
 // aligned base and ld, K a multiple of 16. With flip = kFlipU8 the bytes are
 // uint8 and the sums are those of value - 128.

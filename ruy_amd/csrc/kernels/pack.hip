@@ -348,7 +348,59 @@ __global__ __launch_bounds__(256) void PackI16SplitKernel(PackSource src, int8_t
   }
 }
 
+// dst(i, j) = src(i, j) for two views of the same shape with different storage
+// orders, 32x32 elements per block through LDS: reads run along the source's
+// contiguous dimension, writes along the destination's.
+template <typename T>
+__global__ __launch_bounds__(256) void ReorderKernel(const T* src, int64_t src_rs, int64_t src_cs, T* dst,
+                                                    int64_t dst_rs, int64_t dst_cs, int rows, int cols) {
+  __shared__ T tile[32][33];
+  const int tx = threadIdx.x & 31;
+  const int ty = threadIdx.x >> 5;  // 0..7
+  const int i0 = blockIdx.x * 32;
+  const int j0 = blockIdx.y * 32;
+  const bool src_rows_contiguous = src_rs == 1;
+  const bool dst_rows_contiguous = dst_rs == 1;
+#pragma unroll
+  for (int t = ty; t < 32; t += 8) {
+    const int i = i0 + (src_rows_contiguous ? tx : t);
+    const int j = j0 + (src_rows_contiguous ? t : tx);
+    if (i < rows && j < cols) tile[i - i0][j - j0] = src[i * src_rs + j * src_cs];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int t = ty; t < 32; t += 8) {
+    const int i = i0 + (dst_rows_contiguous ? tx : t);
+    const int j = j0 + (dst_rows_contiguous ? t : tx);
+    if (i < rows && j < cols) dst[i * dst_rs + j * dst_cs] = tile[i - i0][j - j0];
+  }
+}
+
 }  // namespace
+
+hipError_t LaunchReorder(hipStream_t stream, const DevMat& src, const DevMat& dst) {
+  if (dst.rows == 0 || dst.cols == 0) return hipSuccess;
+  const dim3 grid((dst.rows + 31) / 32, (dst.cols + 31) / 32);
+  switch (DtypeSize(dst.dtype)) {
+    case 1:
+      hipLaunchKernelGGL(ReorderKernel<uint8_t>, grid, dim3(256), 0, stream, static_cast<const uint8_t*>(src.data),
+                         src.rs, src.cs, static_cast<uint8_t*>(dst.data), dst.rs, dst.cs, dst.rows, dst.cols);
+      break;
+    case 2:
+      hipLaunchKernelGGL(ReorderKernel<uint16_t>, grid, dim3(256), 0, stream,
+                         static_cast<const uint16_t*>(src.data), src.rs, src.cs, static_cast<uint16_t*>(dst.data),
+                         dst.rs, dst.cs, dst.rows, dst.cols);
+      break;
+    case 4:
+      hipLaunchKernelGGL(ReorderKernel<uint32_t>, grid, dim3(256), 0, stream,
+                         static_cast<const uint32_t*>(src.data), src.rs, src.cs, static_cast<uint32_t*>(dst.data),
+                         dst.rs, dst.cs, dst.rows, dst.cols);
+      break;
+    default:
+      return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
 
 hipError_t LaunchPackI16Split(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld) {
   if (src.count == 0 || ld == 0) return hipSuccess;

@@ -551,6 +551,29 @@ int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
       const DevMat& side16 = dst_col_major ? rhs : lhs;
       if (side8.dtype == RUYAMD_DTYPE_I8 && side16.dtype == RUYAMD_DTYPE_I16)
         return RunI8I16(ctx, call, err);
+      // (A single-column destination has no storage order to flip.)
+      if (side8.dtype == RUYAMD_DTYPE_I16 && side16.dtype == RUYAMD_DTYPE_I8 &&
+          !(dst_col_major && call->dst.cols == 1)) {
+        // The other way round: compute into a scratch destination of the
+        // opposite storage order, for which the int8 side is the contiguous
+        // one, and reorder that into the caller's destination.
+        MulCall flipped = *call;
+        DevMat& t = flipped.dst;
+        t.data = ctx->workspace.Alloc(std::size_t(t.rows) * t.cols * DtypeSize(t.dtype));
+        if (!t.data) {
+          *err = "workspace allocation failed";
+          return RUYAMD_E_HIP;
+        }
+        t.rs = dst_col_major ? t.cols : 1;
+        t.cs = dst_col_major ? 1 : t.rows;
+        if (int rc = RunI8I16(ctx, &flipped, err)) return rc;
+        call->staged_any = call->staged_any || flipped.staged_any;
+        if (LaunchReorder(ctx->stream, t, call->dst) != hipSuccess) {
+          *err = "reorder kernel launch failed";
+          return RUYAMD_E_HIP;
+        }
+        return RUYAMD_OK;
+      }
     }
     if (lhs.dtype == RUYAMD_DTYPE_F32 && rhs.dtype == RUYAMD_DTYPE_F32 &&
         call->dst.dtype == RUYAMD_DTYPE_F32 && call->accum_dtype == RUYAMD_DTYPE_F32)
