@@ -1,5 +1,6 @@
 #include "plan.h"
 
+#include <algorithm>
 #include <cstdint>
 
 #include "kernels/gemm_i8.h"
@@ -528,57 +529,34 @@ int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
   return RUYAMD_OK;
 }
 
-int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
-  const DevMat& lhs = call->lhs;
-  const DevMat& rhs = call->rhs;
-  // The tuned kernels address operands through 32-bit buffer offsets; anything
-  // of 2 GiB or more goes to the generic kernel, which uses 64-bit offsets.
-  auto extent_bytes = [](const DevMat& m) {
-    if (m.rows == 0 || m.cols == 0) return uint64_t(0);
-    return (uint64_t(m.rows - 1) * uint64_t(m.rs) + uint64_t(m.cols - 1) * uint64_t(m.cs) + 1) *
-           uint64_t(DtypeSize(m.dtype));
-  };
-  const uint64_t kLimit = (uint64_t(1) << 31) - (uint64_t(1) << 20);
-  const bool huge = extent_bytes(lhs) >= kLimit || extent_bytes(rhs) >= kLimit ||
-                    uint64_t(lhs.rows) * (uint64_t(lhs.cols) + 16) * DtypeSize(lhs.dtype) >= kLimit ||
-                    uint64_t(rhs.cols) * (uint64_t(rhs.rows) + 16) * DtypeSize(rhs.dtype) >= kLimit / 2;
-  if (!ctx->force_generic && !huge) {
-    if (Is8Bit(lhs.dtype) && Is8Bit(rhs.dtype)) return RunInt8(ctx, call, err);
-    {
-      // The int8 side must run along the destination's contiguous dimension.
-      const bool dst_col_major = call->dst.rs == 1;
-      const DevMat& side8 = dst_col_major ? lhs : rhs;
-      const DevMat& side16 = dst_col_major ? rhs : lhs;
-      if (side8.dtype == RUYAMD_DTYPE_I8 && side16.dtype == RUYAMD_DTYPE_I16)
-        return RunI8I16(ctx, call, err);
-      // (A single-column destination has no storage order to flip.)
-      if (side8.dtype == RUYAMD_DTYPE_I16 && side16.dtype == RUYAMD_DTYPE_I8 &&
-          !(dst_col_major && call->dst.cols == 1)) {
-        // The other way round: compute into a scratch destination of the
-        // opposite storage order, for which the int8 side is the contiguous
-        // one, and reorder that into the caller's destination.
-        MulCall flipped = *call;
-        DevMat& t = flipped.dst;
-        t.data = ctx->workspace.Alloc(std::size_t(t.rows) * t.cols * DtypeSize(t.dtype));
-        if (!t.data) {
-          *err = "workspace allocation failed";
-          return RUYAMD_E_HIP;
-        }
-        t.rs = dst_col_major ? t.cols : 1;
-        t.cs = dst_col_major ? 1 : t.rows;
-        if (int rc = RunI8I16(ctx, &flipped, err)) return rc;
-        call->staged_any = call->staged_any || flipped.staged_any;
-        if (LaunchReorder(ctx->stream, t, call->dst) != hipSuccess) {
-          *err = "reorder kernel launch failed";
-          return RUYAMD_E_HIP;
-        }
-        return RUYAMD_OK;
-      }
-    }
-    if (lhs.dtype == RUYAMD_DTYPE_F32 && rhs.dtype == RUYAMD_DTYPE_F32 &&
-        call->dst.dtype == RUYAMD_DTYPE_F32 && call->accum_dtype == RUYAMD_DTYPE_F32)
-      return RunF32(ctx, call, err);
-  }
+namespace {
+
+enum class TunedPath { kNone, kInt8, kInt8Int16, kF32 };
+
+TunedPath TunedPathFor(const MulCall& call) {
+  const int l = call.lhs.dtype, r = call.rhs.dtype;
+  if (Is8Bit(l) && Is8Bit(r)) return TunedPath::kInt8;
+  if ((l == RUYAMD_DTYPE_I8 && r == RUYAMD_DTYPE_I16) || (l == RUYAMD_DTYPE_I16 && r == RUYAMD_DTYPE_I8))
+    return TunedPath::kInt8Int16;
+  if (l == RUYAMD_DTYPE_F32 && r == RUYAMD_DTYPE_F32 && call.dst.dtype == RUYAMD_DTYPE_F32 &&
+      call.accum_dtype == RUYAMD_DTYPE_F32)
+    return TunedPath::kF32;
+  return TunedPath::kNone;
+}
+
+// The tuned kernels address an operand through 32-bit buffer offsets, so its
+// depth-contiguous form (used in place or packed) must stay below 2 GiB; the
+// int16 operand is split into two planes, hence half of that. Counts of rows
+// (columns) that fit, with the depth padding the pack kernels may add.
+constexpr uint64_t kOperandLimit = (uint64_t(1) << 31) - (uint64_t(1) << 20);
+
+uint64_t VectorsThatFit(const DevMat& m, int depth) {
+  const uint64_t vector_bytes = (uint64_t(depth) + 16) * uint64_t(DtypeSize(m.dtype));
+  const uint64_t limit = m.dtype == RUYAMD_DTYPE_I16 ? kOperandLimit / 2 : kOperandLimit;
+  return limit / vector_bytes;
+}
+
+int RunGeneric(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   if (int rc = EnsureOnDevice(ctx, call, 0, err)) return rc;
   if (int rc = EnsureOnDevice(ctx, call, 1, err)) return rc;
   if (LaunchGeneric(ctx->stream, call->lhs, call->rhs, call->ep, call->dst, call->accum_dtype) != hipSuccess) {
@@ -586,6 +564,90 @@ int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     return RUYAMD_E_HIP;
   }
   ctx->last_kernel = RUYAMD_KERNEL_GENERIC;
+  return RUYAMD_OK;
+}
+
+// One call whose operands both fit the tuned kernels.
+int RunTuned(ruyamd_ctx* ctx, MulCall* call, TunedPath path, std::string* err) {
+  switch (path) {
+    case TunedPath::kInt8:
+      return RunInt8(ctx, call, err);
+    case TunedPath::kF32:
+      return RunF32(ctx, call, err);
+    case TunedPath::kInt8Int16: {
+      // The kernel wants the int8 side along the destination's contiguous dimension.
+      const bool dst_col_major = call->dst.rs == 1;
+      const DevMat& contiguous_side = dst_col_major ? call->lhs : call->rhs;
+      if (contiguous_side.dtype == RUYAMD_DTYPE_I8) return RunI8I16(ctx, call, err);
+      // The other way round: compute into a scratch destination of the
+      // opposite storage order and reorder that into the caller's destination.
+      // (A single-column destination has no storage order to flip.)
+      if (dst_col_major && call->dst.cols == 1) return RunGeneric(ctx, call, err);
+      MulCall flipped = *call;
+      DevMat& t = flipped.dst;
+      t.data = ctx->workspace.Alloc(std::size_t(t.rows) * t.cols * DtypeSize(t.dtype));
+      if (!t.data) {
+        *err = "workspace allocation failed";
+        return RUYAMD_E_HIP;
+      }
+      t.rs = dst_col_major ? t.cols : 1;
+      t.cs = dst_col_major ? 1 : t.rows;
+      if (int rc = RunI8I16(ctx, &flipped, err)) return rc;
+      call->staged_any = call->staged_any || flipped.staged_any;
+      if (LaunchReorder(ctx->stream, t, call->dst) != hipSuccess) {
+        *err = "reorder kernel launch failed";
+        return RUYAMD_E_HIP;
+      }
+      return RUYAMD_OK;
+    }
+    default:
+      return RunGeneric(ctx, call, err);
+  }
+}
+
+const void* Advance(const void* p, int64_t elements, int element_size) {
+  return p ? static_cast<const char*>(p) + elements * element_size : nullptr;
+}
+
+}  // namespace
+
+int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
+  const TunedPath path = ctx->force_generic ? TunedPath::kNone : TunedPathFor(*call);
+  if (path == TunedPath::kNone) return RunGeneric(ctx, call, err);
+  const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
+  const uint64_t rows_fit = VectorsThatFit(call->lhs, K);
+  const uint64_t cols_fit = VectorsThatFit(call->rhs, K);
+  if (rows_fit == 0 || cols_fit == 0) return RunGeneric(ctx, call, err);  // a single vector of 2 GiB
+  if (uint64_t(M) <= rows_fit && uint64_t(N) <= cols_fit) return RunTuned(ctx, call, path, err);
+
+  // An operand of 2 GiB or more: the destination is computed in blocks of
+  // rows and columns whose operands fit. Each block is an ordinary call on
+  // sub-views (its cached operands are keyed by the sub-view's address).
+  if (int rc = EnsureOnDevice(ctx, call, 0, err)) return rc;
+  if (int rc = EnsureOnDevice(ctx, call, 1, err)) return rc;
+  const int row_step = static_cast<int>(std::min<uint64_t>(rows_fit, uint64_t(M)));
+  const int col_step = static_cast<int>(std::min<uint64_t>(cols_fit, uint64_t(N)));
+  const int accum_size = DtypeSize(call->accum_dtype);
+  for (int r0 = 0; r0 < M; r0 += row_step) {
+    for (int c0 = 0; c0 < N; c0 += col_step) {
+      MulCall block = *call;
+      block.lhs.rows = std::min(row_step, M - r0);
+      block.rhs.cols = std::min(col_step, N - c0);
+      block.dst.rows = block.lhs.rows;
+      block.dst.cols = block.rhs.cols;
+      block.lhs.data = const_cast<void*>(Advance(call->lhs.data, int64_t(r0) * call->lhs.rs, DtypeSize(call->lhs.dtype)));
+      block.rhs.data = const_cast<void*>(Advance(call->rhs.data, int64_t(c0) * call->rhs.cs, DtypeSize(call->rhs.dtype)));
+      block.dst.data = const_cast<void*>(Advance(call->dst.data, int64_t(r0) * call->dst.rs + int64_t(c0) * call->dst.cs,
+                                                 DtypeSize(call->dst.dtype)));
+      block.lhs_src_key = Advance(call->lhs_src_key, int64_t(r0) * call->lhs.rs, DtypeSize(call->lhs.dtype));
+      block.rhs_src_key = Advance(call->rhs_src_key, int64_t(c0) * call->rhs.cs, DtypeSize(call->rhs.dtype));
+      const int64_t channel0 = call->ep.channel_is_col ? c0 : r0;
+      block.ep.bias = Advance(call->ep.bias, channel0, accum_size);
+      block.ep.mult_fixedpoint = static_cast<const int32_t*>(Advance(call->ep.mult_fixedpoint, channel0, 4));
+      block.ep.mult_exponent = static_cast<const int32_t*>(Advance(call->ep.mult_exponent, channel0, 4));
+      if (int rc = RunTuned(ctx, &block, path, err)) return rc;
+    }
+  }
   return RUYAMD_OK;
 }
 

@@ -628,3 +628,37 @@ def test_uint8_operands_used_in_place(device_ctx, tup):
             announce(p.name)
             got, want = run_both(device_ctx, p)
             compare(p, got, want)
+
+
+def test_operand_of_more_than_2_gib(device_ctx):
+    """A 2.18 GB int8 LHS (66560 x 32768): the tuned kernels address an
+    operand through 32-bit offsets, so the library computes the destination in
+    row blocks whose operands fit (here 65472 + 1088 rows), each an ordinary
+    call on a sub-view; bias and per-channel multipliers follow the rows. One,
+    three and seventeen columns: both skinny kernels and the tiled kernel."""
+    import device_runner as D
+    rng = np.random.default_rng(2024)
+    K, rows = 32768, 66560
+    block = rng.integers(-127, 128, (1024, K), dtype=np.int8)
+    lhs = W.HostMatrix(S.I8, rows, K, S.ORDER_ROW_MAJOR, zero_point=3)
+    lhs.storage.reshape(rows, K)[:] = np.tile(block, (rows // 1024, 1))
+    # make the rows differ from block to block
+    lhs.storage.reshape(rows, K)[:, 0] = (np.arange(rows) % 251 - 125).astype(np.int8)
+    for N in (1, 3, 17):
+        rhs = W.HostMatrix(S.I8, K, N, S.ORDER_COL_MAJOR, zero_point=-5)
+        rhs.storage[:] = rng.integers(-128, 128, rhs.storage.size, dtype=np.int8)
+        bias = rng.integers(-100000, 100000, rows, dtype=np.int32)
+        mf = rng.integers(1 << 30, (1 << 31) - 1, rows, dtype=np.int32)
+        me = rng.integers(-14, -9, rows, dtype=np.int32)
+        for dst_dtype in (S.I32, S.I8):
+            dst = W.HostMatrix(dst_dtype, rows, N, S.ORDER_COL_MAJOR, zero_point=0 if dst_dtype == S.I32 else 7)
+            if dst_dtype == S.I32:
+                p = W.Problem("huge raw N=%d" % N, lhs, rhs, dst, S.I32, bias=bias)
+            else:
+                p = W.Problem("huge requantized N=%d" % N, lhs, rhs, dst, S.I32, bias=bias,
+                              multiplier_fixedpoint_perchannel=mf, multiplier_exponent_perchannel=me,
+                              clamp_min=-128, clamp_max=127)
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
+            assert device_ctx.last_kernel_name() == ("i8_mfma" if N == 17 else "i8_gemv")
