@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the int8 GEMM")
     ap.add_argument("--gemv-size", type=int, default=16384, help="M=K of the int8 GEMV")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the HIP-graph replay timing of the small configurations")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies, so that a counter run "
                          "(FETCH_SIZE / WRITE_SIZE) has a dispatch of known traffic to scale by")
@@ -303,7 +305,7 @@ def bench_gemv(ctx, args):
     return out
 
 
-def bench_other_configs(ctx, steps, warmup):
+def bench_other_configs(ctx, steps, warmup, with_graph=True):
     """Time (not roofline) of the remaining configurations: small or
     latency-bound shapes whose gate is parity; reported for completeness."""
     from ruy_amd import workloads as W
@@ -320,7 +322,7 @@ def bench_other_configs(ctx, steps, warmup):
         step_s, _, _ = time_steps(lambda: dp.run(ctx), steps, warmup, ctx)
         entry = {"config": name, "kernel": kernel, "us_per_step": step_s * 1e6,
                  "Top/s": problem.ops() / step_s / 1e12}
-        if problem.ops() < 1e9:
+        if with_graph and problem.ops() < 1e9:
             entry["us_per_step_graph"] = graph_replay_us(ctx, dp)
         out.append(entry)
     ctx.set_kernel_timing(True)
@@ -411,7 +413,7 @@ def main():
         else:
             line["gemv"] = gv
     if args.workload == "all":
-        line["other_configs"] = bench_other_configs(ctx, args.steps, args.warmup)
+        line["other_configs"] = bench_other_configs(ctx, args.steps, args.warmup, not args.no_graph)
     if args.copy_calibration:
         a = torch.full((256 << 20,), 3, dtype=torch.uint8, device="cuda")
         b = torch.empty_like(a)
