@@ -560,7 +560,7 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
   return ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
 }
 
-enum class Tile { k256x256, k256x128, k128x256, k128x128, k64x64 };
+enum class Tile { k256x256, k256x128, k128x256, k128x128, k64x128, k64x64 };
 
 // Picks the tile by a small cost model: workgroups are dealt to the CUs in
 // rounds, a round of a given tile costs its area divided by how well that tile
@@ -569,7 +569,7 @@ enum class Tile { k256x256, k256x128, k128x256, k128x128, k64x64 };
 // fragment pair per matrix instruction, about 0.45 of the 256x256 tile's
 // rate). Large tiles win when there are many rounds, small tiles when the last
 // (or only) round would leave most CUs idle. `split_b`: the plane-split form
-// of the int16 kernel, which has the two square large tiles only.
+// of the int16 kernel, which has the two square large tiles and a 64x128 one.
 inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   auto cost = [&](int bm, int bn, double efficiency) {
     const int rounds = (TileCount(args, bm, bn) + num_cus - 1) / num_cus;
@@ -577,7 +577,12 @@ inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   };
   const double c256 = cost(256, 256, 1.0);
   const double c128 = cost(128, 128, 0.65);
-  if (split_b) return c256 <= c128 ? Tile::k256x256 : Tile::k128x128;
+  if (split_b) {
+    // Plane-split operand: the smallest tile is 64 rows x 128 plane columns (64 destination columns).
+    const double c64x128 = cost(64, 128, 0.5);
+    if (c256 <= c128 && c256 <= c64x128) return Tile::k256x256;
+    return c128 <= c64x128 ? Tile::k128x128 : Tile::k64x128;
+  }
   const double c64 = cost(64, 64, 0.45);
   const double c256x128 = cost(256, 128, 0.75);
   const double c128x256 = cost(128, 256, 0.75);
@@ -596,6 +601,8 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
       return Launch<Traits, 4, 4, 128, 2>(stream, args);
     case Tile::k128x128:
       return Launch<Traits, 2, 2, 128, 4>(stream, args);
+    case Tile::k64x128:
+      return Launch<Traits, 1, 2, 128, 4>(stream, args);
     default:
       break;
   }
