@@ -61,7 +61,10 @@ struct GemmArgs {
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmF32(hipStream_t stream, const GemmArgs& args, int num_cus);
-// int8 x int16: `b` is the int16 operand split by LaunchPackI16Split.
+// int8 x int16: `b` is the int16 operand split by LaunchPackI16Split. On the
+// smallest tile (GemmI8I16CanFuseSums) fuse_sums / fused_a_factor work as in
+// the int8 kernel; fused_b_factor is ignored.
+bool GemmI8I16CanFuseSums(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus);
 
 // Skinny multiplication: `rows` wide-side vectors against narrow_count <= 8

@@ -157,7 +157,8 @@ struct Cfg {
 // values the arithmetic is defined on.
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false>
 __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
-  static_assert(!kFusedSums || WM * WN == 1, "fused sums exist for the single-block tile only");
+  static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
+                "fused sums exist for the tiles with one block (one block per plane) per wave only");
   static_assert(!kFlip || WM * WN == 1, "in-place uint8 operands exist for the single-block tile only");
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   constexpr int kBK = BK;
@@ -351,8 +352,12 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
       __builtin_amdgcn_sched_barrier(0);
       Traits::Mma(cur.a[n / WN], cur.b[n % WN], acc[n / WN][n % WN]);
       if constexpr (kFusedSums) {
-        Traits::Mma(cur.a[0], ones, sum_a);
-        Traits::Mma(ones, cur.b[0], sum_b);
+        // Once per sub-step. The plane-split operand has zero point 0 by
+        // definition, so its column sums are never needed.
+        if (n == 0) {
+          Traits::Mma(cur.a[0], ones, sum_a);
+          if constexpr (!Traits::kSplitB) Traits::Mma(ones, cur.b[0], sum_b);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       if (!kReadsFirst && n < kReadSlots) {
@@ -411,10 +416,13 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   if constexpr (kFusedSums) {
     const uint32_t fa = static_cast<uint32_t>(args.fused_a_factor);
     const uint32_t fb = static_cast<uint32_t>(args.fused_b_factor);
+    // Plane-split operand: the correction belongs to the low plane's block
+    // (the write-back combines 256 * high + low).
+    constexpr int kBlock = Traits::kSplitB ? 1 : 0;
 #pragma unroll
     for (int v = 0; v < 16; ++v)
-      acc[0][0][v] = static_cast<int>(static_cast<uint32_t>(acc[0][0][v]) - fa * static_cast<uint32_t>(sum_a[v]) -
-                                      fb * static_cast<uint32_t>(sum_b[v]));
+      acc[0][kBlock][v] = static_cast<int>(static_cast<uint32_t>(acc[0][kBlock][v]) -
+                                           fa * static_cast<uint32_t>(sum_a[v]) - fb * static_cast<uint32_t>(sum_b[v]));
   }
 
   // ---- fused write-back ----

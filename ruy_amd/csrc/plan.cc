@@ -465,7 +465,6 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
                                side8 == 0 ? call->lhs_src_key : call->rhs_src_key,
                                side8 == 0 ? N : M, /*u8_depth_step=*/0, &a, err))
     return rc;
-  if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
   if (int rc = EnsureOnDevice(ctx, call, side16, err)) return rc;
   const DevMat& m16 = side16 == 0 ? call->lhs : call->rhs;
   const PackSource src = side16 == 0 ? PackSource{m16.data, m16.rs, m16.cs, m16.rows, m16.cols, m16.dtype}
@@ -496,11 +495,19 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.M = swap ? N : M;
   args.N = n_phys;
   args.n_logical = src.count;
-  args.ep.lhs_sums = a.sums;
   args.ep.rhs_sums = nullptr;
   args.ep.lhs_zero_point = 0;
   args.ep.rhs_zero_point = -128;  // the low plane stores (v & 0xff) - 128
   args.ep.zp_product_depth = 0;
+  if (a.sums_pending && GemmI8I16CanFuseSums(args, ctx->multiprocessor_count)) {
+    // Small problem, int8 side used in place: the kernel forms its row sums.
+    args.fuse_sums = 1;
+    args.fused_a_factor = args.ep.rhs_zero_point;
+    args.ep.rhs_zero_point = 0;
+  } else if (int rc = MaterializeSums(ctx, &a, K, err)) {
+    return rc;
+  }
+  args.ep.lhs_sums = a.sums;
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8I16(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
