@@ -7,6 +7,8 @@
 // Operands that already have that layout are used in place and only summed.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "../internal.h"
 #include "gemm_i8.h"
 
@@ -348,6 +350,37 @@ __global__ __launch_bounds__(256) void PackI16SplitKernel(PackSource src, int8_t
   }
 }
 
+// The same split for a depth-contiguous, 16-byte aligned int16 source whose
+// depth is a multiple of 16: pure streaming, one wave per vector part, each
+// lane turns 16 int16 (two 16-byte loads) into 16 high bytes and 16 low bytes
+// with v_perm_b32 (the low plane is the low byte with its top bit flipped).
+__global__ __launch_bounds__(256) void PackI16SplitRowsKernel(PackSource src, int8_t* dst, int32_t ld) {
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int count_padded = (src.count + 31) / 32 * 32;  // vectors of the last group that do not exist are zero
+  if (c >= count_padded) return;
+  int8_t* hi_row = dst + (int64_t(c / 32) * 64 + c % 32) * ld;
+  int8_t* lo_row = hi_row + int64_t(32) * ld;
+  const int16_t* row = static_cast<const int16_t*>(src.data) + int64_t(c) * src.stride_c;
+  for (int k = blockIdx.y * 1024 + lane * 16; k < ld; k += gridDim.y * 1024) {
+    v4i hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
+    if (c < src.count && k < src.K) {
+      const v4i x = *reinterpret_cast<const v4i*>(row + k);
+      const v4i y = *reinterpret_cast<const v4i*>(row + k + 8);
+      hi[0] = __builtin_amdgcn_perm(x[1], x[0], 0x07050301u);
+      hi[1] = __builtin_amdgcn_perm(x[3], x[2], 0x07050301u);
+      hi[2] = __builtin_amdgcn_perm(y[1], y[0], 0x07050301u);
+      hi[3] = __builtin_amdgcn_perm(y[3], y[2], 0x07050301u);
+      lo[0] = __builtin_amdgcn_perm(x[1], x[0], 0x06040200u) ^ 0x80808080u;
+      lo[1] = __builtin_amdgcn_perm(x[3], x[2], 0x06040200u) ^ 0x80808080u;
+      lo[2] = __builtin_amdgcn_perm(y[1], y[0], 0x06040200u) ^ 0x80808080u;
+      lo[3] = __builtin_amdgcn_perm(y[3], y[2], 0x06040200u) ^ 0x80808080u;
+    }
+    *reinterpret_cast<v4i*>(hi_row + k) = hi;
+    *reinterpret_cast<v4i*>(lo_row + k) = lo;
+  }
+}
+
 // dst(i, j) = src(i, j) for two views of the same shape with different storage
 // orders, 32x32 elements per block through LDS: reads run along the source's
 // contiguous dimension, writes along the destination's.
@@ -405,6 +438,12 @@ hipError_t LaunchReorder(hipStream_t stream, const DevMat& src, const DevMat& ds
 hipError_t LaunchPackI16Split(hipStream_t stream, const PackSource& src, int8_t* dst, int32_t ld) {
   if (src.count == 0 || ld == 0) return hipSuccess;
   const int groups = (src.count + 31) / 32;
+  if (src.stride_k == 1 && src.K % 16 == 0 && (reinterpret_cast<uintptr_t>(src.data) & 15) == 0 &&
+      (src.stride_c * 2) % 16 == 0) {
+    const int k_blocks = std::min((ld + 1023) / 1024, std::max(1, 2048 / (groups * 32)));
+    hipLaunchKernelGGL(PackI16SplitRowsKernel, dim3(groups * 8, k_blocks), dim3(256), 0, stream, src, dst, ld);
+    return hipGetLastError();
+  }
   int blocks_k = (ld + 31) / 32;
   if (blocks_k > 64) blocks_k = 64;
   hipLaunchKernelGGL(PackI16SplitKernel, dim3(groups, blocks_k), dim3(256), 0, stream, src, dst, ld);
