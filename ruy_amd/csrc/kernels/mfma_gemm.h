@@ -568,7 +568,7 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
   return ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
 }
 
-enum class Tile { k256x256, k256x128, k128x256, k128x128, k64x128, k64x64 };
+enum class Tile { k256x256, k256x128, k128x256, k128x128, k128x64, k64x128, k64x64 };
 
 // Picks the tile by a small cost model: workgroups are dealt to the CUs in
 // rounds, a round of a given tile costs its area divided by how well that tile
@@ -578,6 +578,7 @@ enum class Tile { k256x256, k256x128, k128x256, k128x128, k64x128, k64x64 };
 // rate). Large tiles win when there are many rounds, small tiles when the last
 // (or only) round would leave most CUs idle. `split_b`: the plane-split form
 // of the int16 kernel, which has the two square large tiles and a 64x128 one.
+constexpr double kEffHalf = 0.55;
 inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   auto cost = [&](int bm, int bn, double efficiency) {
     const int rounds = (TileCount(args, bm, bn) + num_cus - 1) / num_cus;
@@ -594,11 +595,15 @@ inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   const double c64 = cost(64, 64, 0.45);
   const double c256x128 = cost(256, 128, 0.75);
   const double c128x256 = cost(128, 256, 0.75);
-  const double best = std::min(std::min(c256, c128), std::min(c64, std::min(c256x128, c128x256)));
+  const double c128x64 = cost(128, 64, kEffHalf);
+  const double c64x128 = cost(64, 128, kEffHalf);
+  const double best = std::min({c256, c128, c64, c256x128, c128x256, c128x64, c64x128});
   if (c256 == best) return Tile::k256x256;
   if (c256x128 == best) return Tile::k256x128;
   if (c128x256 == best) return Tile::k128x256;
   if (c128 == best) return Tile::k128x128;
+  if (c128x64 == best) return Tile::k128x64;
+  if (c64x128 == best) return Tile::k64x128;
   return Tile::k64x64;
 }
 
@@ -620,6 +625,8 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
         return Launch<Traits, 4, 2, 128, 3>(stream, args);
       case Tile::k128x256:
         return Launch<Traits, 2, 4, 128, 3>(stream, args);
+      case Tile::k128x64:
+        return Launch<Traits, 2, 1, 128, 4>(stream, args);
       default:
         return Launch<Traits, 1, 1, 128, 4>(stream, args);
     }

@@ -452,10 +452,11 @@ def test_skinny_shapes_both_orientations(device_ctx, tup):
                                  (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
 def test_shapes_that_take_the_rectangular_and_large_tiles(device_ctx, tup):
     """Destination sizes for which the tile cost model picks the 256x128, the
-    128x256, the 128x128 and the 256x256 tile (on 256 CUs), with shallow depths
+    128x256, the 128x128, the 256x256, the 64x128 and the 128x64 tile (on 256 CUs), with shallow depths
     so that the checker stays fast; ragged edges in both dimensions."""
     rng = np.random.default_rng(77)
-    for shape in [(4096, 200, 2048), (1920, 136, 4352), (1790, 100, 1795), (4000, 72, 4100), (4096, 64, 4096)]:
+    for shape in [(4096, 200, 2048), (1920, 136, 4352), (1790, 100, 1795), (4000, 72, 4100), (4096, 64, 4096),
+                  (16384, 80, 128), (120, 64, 16380)]:  # the 64x128 and 128x64 tiles
         for orders in (cases.RCC, cases.ALL_ORDERS[int(rng.integers(8))]):
             p = W.random_problem(rng, *tup, *shape, *orders, strided=bool(rng.integers(2)),
                                  name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
