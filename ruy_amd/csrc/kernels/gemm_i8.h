@@ -89,6 +89,14 @@ struct GemvI8Args {
   // past the depth are read as zero and would turn into -128.
   uint32_t wide_flip = 0;
   uint32_t narrow_flip = 0;
+  // int8 kernels: with fuse_sums set the kernel forms the depth sums of the
+  // wide and narrow vectors itself (a few extra instructions on data it holds
+  // anyway) and subtracts fused_wide_factor * sum(wide vector) +
+  // fused_narrow_factor * sum(narrow vector) from every product before the
+  // write-back; the caller then leaves the matching zero point of `ep` at 0.
+  int32_t fuse_sums = 0;
+  int32_t fused_wide_factor = 0;
+  int32_t fused_narrow_factor = 0;
   Epilogue ep;
   DevMat dst;
 };

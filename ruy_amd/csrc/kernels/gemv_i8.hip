@@ -77,6 +77,13 @@ __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
   for (int r = 0; r < kRowsPerWave; ++r)
 #pragma unroll
     for (int j = 0; j < NB; ++j) acc[r][j] = 0;
+  // args.fuse_sums: depth sums of the wide and narrow vectors, per lane.
+  int wide_sum[kRowsPerWave], narrow_sum[NB];
+#pragma unroll
+  for (int r = 0; r < kRowsPerWave; ++r) wide_sum[r] = 0;
+#pragma unroll
+  for (int j = 0; j < NB; ++j) narrow_sum[j] = 0;
+  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
 
   // The depth is walked in steps of 1024 bytes starting from a step that
   // differs from wave to wave and wrapping around (the order does not matter
@@ -113,6 +120,14 @@ __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
         else
           acc[r][j] = Dot16(w[r], n[j], acc[r][j]);
       }
+    if (args.fuse_sums) {  // wave-uniform
+#pragma unroll
+      for (int r = 0; r < kRowsPerWave; ++r)
+        wide_sum[r] = Dot16(kFlip ? w[r] ^ static_cast<int>(args.wide_flip) : w[r], ones, wide_sum[r]);
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        narrow_sum[j] = Dot16(kFlip ? n[j] ^ static_cast<int>(args.narrow_flip) : n[j], ones, narrow_sum[j]);
+    }
   };
 
   // Two depth steps are in flight: the loads of step s+1 are issued before the
@@ -139,7 +154,11 @@ __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
   for (int r = 0; r < kRowsPerWave; ++r)
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-      const int total = WaveSum(acc[r][j]);
+      // The per-lane correction is linear, so it can be applied before the reduction.
+      const uint32_t corrected = static_cast<uint32_t>(acc[r][j]) -
+                                 static_cast<uint32_t>(args.fused_wide_factor) * static_cast<uint32_t>(wide_sum[r]) -
+                                 static_cast<uint32_t>(args.fused_narrow_factor) * static_cast<uint32_t>(narrow_sum[j]);
+      const int total = WaveSum(static_cast<int>(corrected));
       if (lane == r * NB + j) mine = total;
     }
   const int r = lane / NB;
@@ -279,6 +298,11 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
   const int q = lane >> 4;
   const bool narrow_lane = mv < kNarrow;
   v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+  // args.fuse_sums: sum of each wide vector (in every column) and of each
+  // narrow vector (in every row), by multiplying with a fragment of ones.
+  v4i wide_sum = {0, 0, 0, 0}, narrow_sum = {0, 0, 0, 0};
+  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+  const bool fuse_sums = args.fuse_sums != 0;  // wave-uniform
   // kFlip (uint8 data used in place): the lanes that read the slot of zeros
   // keep their zeros.
   const int a_flip = static_cast<int>(args.wide_flip);
@@ -300,6 +324,10 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
         acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc1, 0, 0, 0);
       else
         acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc0, 0, 0, 0);
+      if (fuse_sums) {
+        wide_sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, ones, wide_sum, 0, 0, 0);
+        narrow_sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, b, narrow_sum, 0, 0, 0);
+      }
     }
   };
 
@@ -335,6 +363,14 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
     ring_slot = ring_slot + 1 == kRing ? 0 : ring_slot + 1;
   }
   v4i acc = acc0 + acc1;
+  if (fuse_sums) {
+    // Linear in the depth, so each wave corrects its own partial block.
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      acc[v] = static_cast<int>(static_cast<uint32_t>(acc[v]) -
+                                static_cast<uint32_t>(args.fused_wide_factor) * static_cast<uint32_t>(wide_sum[v]) -
+                                static_cast<uint32_t>(args.fused_narrow_factor) * static_cast<uint32_t>(narrow_sum[v]));
+  }
   if (kSplit > 1) {
     // Every load of this wave has landed; its ring now carries its partial block.
     if (wave > 0) reinterpret_cast<v4i*>(lds)[lane] = acc;

@@ -207,9 +207,8 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const int32_t zp_product_depth =
       static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
   if (skinny) {
-    // Bandwidth-bound shapes: stream the wide side exactly once.
-    if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
-    if (int rc = MaterializeSums(ctx, &b, K, err)) return rc;
+    // Bandwidth-bound shapes: stream the wide side exactly once. Sums that are
+    // still pending (operands used in place) are formed by the kernel itself.
     GemvI8Args g;
     g.swapped = !(N <= kSkinnyWidthInt8 && (M > kSkinnyWidthInt8 || M >= N));
     const Operand8& wide = g.swapped ? b : a;
@@ -231,6 +230,16 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     g.ep.lhs_zero_point = lzp;
     g.ep.rhs_zero_point = rzp;
     g.ep.zp_product_depth = zp_product_depth;
+    if (a.sums_pending) {  // the LHS sums are multiplied by the RHS zero point
+      g.fuse_sums = 1;
+      (g.swapped ? g.fused_narrow_factor : g.fused_wide_factor) = rzp;
+      g.ep.rhs_zero_point = 0;
+    }
+    if (b.sums_pending) {
+      g.fuse_sums = 1;
+      (g.swapped ? g.fused_wide_factor : g.fused_narrow_factor) = lzp;
+      g.ep.lhs_zero_point = 0;
+    }
     g.dst = call->dst;
     const bool timed = ctx->TimingBegin();
     const hipError_t launched = LaunchGemvI8(ctx->stream, g);
