@@ -1,8 +1,4 @@
-"""ctypes mirrors of the plain structs of include/ruy_amd/c_api.h.
-
-The same layouts are used by the CPU checker under oracle/ (its header repeats
-the definitions), so tests can pass one descriptor to both.
-"""
+"""ctypes mirrors of the plain structs of include/ruy_amd/c_api.h."""
 import ctypes as C
 
 ORDER_COL_MAJOR, ORDER_ROW_MAJOR = 0, 1
@@ -27,7 +23,7 @@ INT_RANGES = {U8: (0, 255), I8: (-128, 127), I16: (-32768, 32767),
 
 
 class Mat(C.Structure):
-    """ruyamd_mat / oracle_mat."""
+    """ruyamd_mat."""
     _fields_ = [
         ("data", C.c_void_p),
         ("rows", C.c_int32),
@@ -42,7 +38,7 @@ class Mat(C.Structure):
 
 
 class MulParamsStruct(C.Structure):
-    """ruyamd_mul_params / oracle_mul_params."""
+    """ruyamd_mul_params."""
     _fields_ = [
         ("bias", C.c_void_p),
         ("multiplier_fixedpoint_perchannel", C.c_void_p),

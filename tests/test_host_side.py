@@ -134,3 +134,24 @@ def test_context_creation_fails_loudly_without_a_gpu():
     from ruy_amd import api
     with pytest.raises(api.RuyAmdError):
         api.Context()
+
+
+def test_product_code_never_touches_the_checker():
+    """The CPU checker under oracle/ is test infrastructure: nothing in the
+    package or in the public headers may include, import, load or name it, and
+    the package has no CPU fallback to route through."""
+    roots = [os.path.join(ROOT, "ruy_amd"), os.path.join(ROOT, "include")]
+    pattern = re.compile(r"oracle|libstock_ruy|libruy_oracle|_ref/")
+    offenders = []
+    for root in roots:
+        for dirpath, dirnames, filenames in os.walk(root):
+            dirnames[:] = [d for d in dirnames if d not in ("__pycache__", "_obj")]
+            for name in filenames:
+                if not name.endswith((".py", ".h", ".cc", ".hip")):
+                    continue
+                path = os.path.join(dirpath, name)
+                with open(path, encoding="utf-8") as f:
+                    for number, line in enumerate(f, 1):
+                        if pattern.search(line):
+                            offenders.append("%s:%d: %s" % (os.path.relpath(path, ROOT), number, line.strip()))
+    assert not offenders, "\n".join(offenders)
