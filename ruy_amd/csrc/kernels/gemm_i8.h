@@ -67,7 +67,7 @@ hipError_t LaunchGemmF32(hipStream_t stream, const GemmArgs& args, int num_cus);
 bool GemmI8I16CanFuseSums(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus);
 
-// Skinny multiplication: `rows` wide-side vectors against narrow_count <= 8
+// Skinny multiplication: `rows` wide-side vectors against narrow_count <= 16
 // narrow-side vectors, all depth-contiguous int8 with the same alignment rules
 // as GemmI8Args. `swapped` = 0: the wide side is the LHS (rows of dst), the
 // narrow side the RHS columns; 1: the wide side is the RHS (columns of dst) and
@@ -109,6 +109,9 @@ hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args);
 // fp32 version: the same argument block with K, ld_wide and ld_narrow counted
 // in bytes of fp32 data, an fp32 destination and the float write-back.
 hipError_t LaunchGemvF32(hipStream_t stream, const GemvI8Args& args);
+// Its 2..16-vector case: the matrix-core streaming kernel of the int8 path on
+// fp32 matrix instructions.
+hipError_t LaunchGemvF32Mma(hipStream_t stream, const GemvI8Args& args);
 
 // A matrix seen as `count` depth-vectors of length K: vector c, depth k is
 // data[c * stride_c + k * stride_k] (elements of `dtype`, uint8 or int8).

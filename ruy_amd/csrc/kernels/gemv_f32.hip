@@ -1,7 +1,8 @@
-// fp32 skinny multiplication (at most 8 vectors on the narrow side): the
-// floating-point counterpart of the int8 streaming kernel, replacing the
-// reference's single-column float kernels (ruy/kernel_avx512.cc:1238-1320,
-// dispatch ruy/kernel_x86.h:101-110) and extending them to 8 columns.
+// fp32 skinny multiplication: the floating-point counterpart of the int8
+// streaming kernels, replacing the reference's single-column float kernels
+// (ruy/kernel_avx512.cc:1238-1320, dispatch ruy/kernel_x86.h:101-110). One
+// narrow vector runs on the kernel below; 2..16 narrow vectors go to the
+// matrix-core streaming kernel shared with int8 (LaunchGemvF32Mma).
 //
 // Each wave owns kRows wide vectors (weight rows) and walks the depth 256
 // floats at a time; a lane keeps 4 consecutive depth values of every narrow
@@ -136,14 +137,9 @@ void Launch(hipStream_t stream, const GemvI8Args& args) {
 
 hipError_t LaunchGemvF32(hipStream_t stream, const GemvI8Args& args) {
   if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
-  if (args.narrow_count <= 1)
-    Launch<1, 2>(stream, args);
-  else if (args.narrow_count <= 2)
-    Launch<2, 4>(stream, args);
-  else if (args.narrow_count <= 4)
-    Launch<4, 4>(stream, args);
-  else
-    Launch<8, 4>(stream, args);
+  // Two and more narrow vectors: the matrix-core streaming kernel.
+  if (args.narrow_count >= 2) return LaunchGemvF32Mma(stream, args);
+  Launch<1, 2>(stream, args);
   return hipGetLastError();
 }
 

@@ -230,13 +230,55 @@ __device__ __forceinline__ void WaitVmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// What differs between the int8 and the fp32 instantiation: the accumulator,
+// the matrix instruction(s) for one 16-byte fragment pair, and the write-back.
+struct Int8Elements {
+  using Acc = v4i;
+  static constexpr bool kInteger = true;
+  // One v_mfma_i32_16x16x64_i8 per fragment pair; consecutive blocks alternate
+  // between two accumulators.
+  static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& c0, Acc& c1, int kb) {
+    if (kb & 1)
+      c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c1, 0, 0, 0);
+    else
+      c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c0, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void Store(int32_t acc, int di, int dj, const GemvI8Args& args) {
+    const int32_t out = FinishInt<true>(acc, di, dj, args.ep);
+    StoreInt(args.dst.data, args.dst.dtype, int64_t(di) * args.dst.rs + int64_t(dj) * args.dst.cs, out);
+  }
+};
+
+struct F32Elements {
+  using Acc = v4f;
+  static constexpr bool kInteger = false;
+  // A 16-byte fragment is 4 consecutive depth values: four v_mfma_f32_16x16x4f32
+  // (lane l supplies row l%16 at depth position l/16 of each), two accumulators.
+  static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& c0, Acc& c1, int) {
+    c0 = __builtin_amdgcn_mfma_f32_16x16x4f32(__int_as_float(a[0]), __int_as_float(b[0]), c0, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(__int_as_float(a[1]), __int_as_float(b[1]), c1, 0, 0, 0);
+    c0 = __builtin_amdgcn_mfma_f32_16x16x4f32(__int_as_float(a[2]), __int_as_float(b[2]), c0, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(__int_as_float(a[3]), __int_as_float(b[3]), c1, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void Store(float acc, int di, int dj, const GemvI8Args& args) {
+    static_cast<float*>(args.dst.data)[int64_t(di) * args.dst.rs + int64_t(dj) * args.dst.cs] =
+        FinishF32(acc, di, dj, args.ep);
+  }
+};
+
 // kStep: depth bytes per ring stage (256, 512 or 1024). kSplit: waves per
 // workgroup; wave w walks the w-th part of the depth and the partial result
 // blocks are added through LDS at the end. kNarrow: narrow vectors staged, 8
 // or 16 (with 16 every column of the matrix instruction is a real one).
-template <int kRing, int kStep, int kSplit, int kNarrow, bool kFlip>
-__global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) {
+// For fp32 (Elements = F32Elements) the arguments are byte-addressed: K and
+// both pitches count bytes of fp32 data.
+template <typename Elements, int kRing, int kStep, int kSplit, int kNarrow, bool kFlip>
+__global__ __launch_bounds__(64 * kSplit) void GemvMmaKernel(GemvI8Args args) {
   static_assert(kNarrow == 8 || kNarrow == 16, "");
+  static_assert(Elements::kInteger || !kFlip, "byte flipping is for uint8 data");
+  using Acc = typename Elements::Acc;
   constexpr int kMmaVectors = kMmaRows + kNarrow;  // vectors per stage
   constexpr int kStage = kMmaVectors * kStep;
   constexpr int kRunsPerLoad = 1024 / kStep;       // runs of kStep bytes moved by one load
@@ -297,12 +339,12 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
   const int mv = lane & 15;
   const int q = lane >> 4;
   const bool narrow_lane = mv < kNarrow;
-  v4i acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+  Acc acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
   // args.fuse_sums: sum of each wide vector (in every column) and of each
   // narrow vector (in every row), by multiplying with a fragment of ones.
   v4i wide_sum = {0, 0, 0, 0}, narrow_sum = {0, 0, 0, 0};
   const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-  const bool fuse_sums = args.fuse_sums != 0;  // wave-uniform
+  const bool fuse_sums = Elements::kInteger && args.fuse_sums != 0;  // wave-uniform
   // kFlip (uint8 data used in place): the lanes that read the slot of zeros
   // keep their zeros.
   const int a_flip = static_cast<int>(args.wide_flip);
@@ -320,10 +362,7 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
         a ^= a_flip;
         b ^= b_flip;
       }
-      if (kb & 1)
-        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc1, 0, 0, 0);
-      else
-        acc0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc0, 0, 0, 0);
+      Elements::Mma(a, b, acc0, acc1, kb);
       if (fuse_sums) {
         wide_sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, ones, wide_sum, 0, 0, 0);
         narrow_sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, b, narrow_sum, 0, 0, 0);
@@ -362,22 +401,24 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
     if (next < n_steps) issue_next(ring_slot);
     ring_slot = ring_slot + 1 == kRing ? 0 : ring_slot + 1;
   }
-  v4i acc = acc0 + acc1;
-  if (fuse_sums) {
-    // Linear in the depth, so each wave corrects its own partial block.
+  Acc acc = acc0 + acc1;
+  if constexpr (Elements::kInteger) {
+    if (fuse_sums) {
+      // Linear in the depth, so each wave corrects its own partial block.
 #pragma unroll
-    for (int v = 0; v < 4; ++v)
-      acc[v] = static_cast<int>(static_cast<uint32_t>(acc[v]) -
-                                static_cast<uint32_t>(args.fused_wide_factor) * static_cast<uint32_t>(wide_sum[v]) -
-                                static_cast<uint32_t>(args.fused_narrow_factor) * static_cast<uint32_t>(narrow_sum[v]));
+      for (int v = 0; v < 4; ++v)
+        acc[v] = static_cast<int>(static_cast<uint32_t>(acc[v]) -
+                                  static_cast<uint32_t>(args.fused_wide_factor) * static_cast<uint32_t>(wide_sum[v]) -
+                                  static_cast<uint32_t>(args.fused_narrow_factor) * static_cast<uint32_t>(narrow_sum[v]));
+    }
   }
   if (kSplit > 1) {
     // Every load of this wave has landed; its ring now carries its partial block.
-    if (wave > 0) reinterpret_cast<v4i*>(lds)[lane] = acc;
+    if (wave > 0) reinterpret_cast<Acc*>(lds)[lane] = acc;
     __syncthreads();
     if (wave > 0) return;
 #pragma unroll
-    for (int w = 1; w < kSplit; ++w) acc += reinterpret_cast<const v4i*>(lds_all + w * kWaveLds)[lane];
+    for (int w = 1; w < kSplit; ++w) acc += reinterpret_cast<const Acc*>(lds_all + w * kWaveLds)[lane];
   }
 
   // Result block: lane l holds column l%16, rows 4*(l/16)..+3.
@@ -389,17 +430,16 @@ __global__ __launch_bounds__(64 * kSplit) void GemvI8MmaKernel(GemvI8Args args) 
       if (row < args.rows) {
         const int di = args.swapped ? j : row;
         const int dj = args.swapped ? row : j;
-        const int32_t out = FinishInt<true>(acc[v], di, dj, args.ep);
-        StoreInt(args.dst.data, args.dst.dtype, int64_t(di) * args.dst.rs + int64_t(dj) * args.dst.cs, out);
+        Elements::Store(acc[v], di, dj, args);
       }
     }
   }
 }
 
-template <int kRing, int kStep, int kSplit, int kNarrow, bool kFlip>
+template <typename Elements, int kRing, int kStep, int kSplit, int kNarrow, bool kFlip>
 hipError_t LaunchMma(hipStream_t stream, const GemvI8Args& args) {
   constexpr size_t lds_bytes = size_t(kSplit) * (size_t(kRing) * (kMmaRows + kNarrow) * kStep + 16);
-  auto kernel = GemvI8MmaKernel<kRing, kStep, kSplit, kNarrow, kFlip>;
+  auto kernel = GemvMmaKernel<Elements, kRing, kStep, kSplit, kNarrow, kFlip>;
   if (lds_bytes > 48 * 1024) {
     // Once per process (thread-safe static initialisation).
     static const hipError_t attr = hipFuncSetAttribute(
@@ -413,8 +453,18 @@ hipError_t LaunchMma(hipStream_t stream, const GemvI8Args& args) {
 
 template <int kSplit, int kNarrow>
 hipError_t LaunchMmaFlip(hipStream_t stream, const GemvI8Args& args, bool flip) {
-  return flip ? LaunchMma<2, 512, kSplit, kNarrow, true>(stream, args)
-              : LaunchMma<2, 512, kSplit, kNarrow, false>(stream, args);
+  return flip ? LaunchMma<Int8Elements, 2, 512, kSplit, kNarrow, true>(stream, args)
+              : LaunchMma<Int8Elements, 2, 512, kSplit, kNarrow, false>(stream, args);
+}
+
+// Depth split: with few groups of 16 wide vectors the depth is divided over
+// the waves of a workgroup to get enough loads in flight.
+int MmaDepthSplit(const GemvI8Args& args) {
+  const int groups = (args.rows + kMmaRows - 1) / kMmaRows;
+  const int steps = (args.K + 511) / 512;
+  if (groups >= 1024 || steps < 4) return 1;
+  if (groups >= 512) return steps >= 16 ? 2 : 1;
+  return steps < 8 ? 2 : 4;
 }
 
 }  // namespace
@@ -442,11 +492,7 @@ hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
       Launch<1, 2, false>(stream, args);
     return hipGetLastError();
   }
-  // Matrix-core kernel. With few groups of 16 wide vectors the depth is split
-  // over the waves of a workgroup to get enough loads in flight.
-  const int groups = (args.rows + kMmaRows - 1) / kMmaRows;
-  const int steps = (args.K + 511) / 512;
-  const int split = groups >= 512 || steps < 4 ? 1 : steps < 8 ? 2 : 4;
+  const int split = MmaDepthSplit(args);
   if (args.narrow_count <= 8) {
     if (split == 1) return LaunchMmaFlip<1, 8>(stream, args, flip);
     if (split == 2) return LaunchMmaFlip<2, 8>(stream, args, flip);
@@ -455,6 +501,24 @@ hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
   if (split == 1) return LaunchMmaFlip<1, 16>(stream, args, flip);
   if (split == 2) return LaunchMmaFlip<2, 16>(stream, args, flip);
   return LaunchMmaFlip<4, 16>(stream, args, flip);
+}
+
+// fp32 with 2..16 narrow vectors: the same streaming kernel on
+// v_mfma_f32_16x16x4f32 (arguments byte-addressed, see GemvMmaKernel).
+hipError_t LaunchGemvF32Mma(hipStream_t stream, const GemvI8Args& args) {
+  if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
+  if (args.narrow_count > 16 || args.K % 16 != 0 || args.ld_wide % 16 != 0 || args.ld_narrow % 16 != 0 ||
+      (reinterpret_cast<uintptr_t>(args.wide) | reinterpret_cast<uintptr_t>(args.narrow)) % 16 != 0)
+    return hipErrorInvalidValue;
+  const int split = MmaDepthSplit(args);
+  if (args.narrow_count <= 8) {
+    if (split == 1) return LaunchMma<F32Elements, 2, 512, 1, 8, false>(stream, args);
+    if (split == 2) return LaunchMma<F32Elements, 2, 512, 2, 8, false>(stream, args);
+    return LaunchMma<F32Elements, 2, 512, 4, 8, false>(stream, args);
+  }
+  if (split == 1) return LaunchMma<F32Elements, 2, 512, 1, 16, false>(stream, args);
+  if (split == 2) return LaunchMma<F32Elements, 2, 512, 2, 16, false>(stream, args);
+  return LaunchMma<F32Elements, 2, 512, 4, 16, false>(stream, args);
 }
 
 }  // namespace ruyamd

@@ -13,9 +13,9 @@ namespace {
 // kCacheIfLargeSpeedup means "the other side is narrow enough for the
 // bandwidth-bound kernel".
 constexpr int kSkinnyWidth = 8;
-// The int8 streaming kernel itself takes up to 16 vectors on the narrow side
-// (all 16 columns of its matrix instruction).
-constexpr int kSkinnyWidthInt8 = 16;
+// The streaming kernels themselves take up to 16 vectors on the narrow side
+// (all 16 columns of their matrix instruction).
+constexpr int kSkinnyKernelWidth = 16;
 
 bool SetupDestination(const MulCall& call, GemmArgs* args);
 
@@ -185,10 +185,10 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   // Which kernel will run decides whether uint8 storage can be used in place:
   // the skinny kernels and the smallest tile of the tiled kernel flip bytes on
   // the way in, provided the depth is a whole number of their depth steps.
-  const bool skinny = N <= kSkinnyWidthInt8 || M <= kSkinnyWidthInt8;
+  const bool skinny = N <= kSkinnyKernelWidth || M <= kSkinnyKernelWidth;
   int u8_depth_step = 0;
   if (skinny) {
-    const bool swapped = !(N <= kSkinnyWidthInt8 && (M > kSkinnyWidthInt8 || M >= N));
+    const bool swapped = !(N <= kSkinnyKernelWidth && (M > kSkinnyKernelWidth || M >= N));
     u8_depth_step = GemvI8DepthStep(swapped ? M : N);
   } else {
     GemmArgs shape;
@@ -210,7 +210,7 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     // Bandwidth-bound shapes: stream the wide side exactly once. Sums that are
     // still pending (operands used in place) are formed by the kernel itself.
     GemvI8Args g;
-    g.swapped = !(N <= kSkinnyWidthInt8 && (M > kSkinnyWidthInt8 || M >= N));
+    g.swapped = !(N <= kSkinnyKernelWidth && (M > kSkinnyKernelWidth || M >= N));
     const Operand8& wide = g.swapped ? b : a;
     const Operand8& narrow = g.swapped ? a : b;
     g.wide = wide.data;
@@ -408,10 +408,10 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   OperandF32 a, b;
   if (int rc = PrepareOperandF32(ctx, call, 0, call->lhs_cache_policy, call->lhs_src_key, N, &a, err)) return rc;
   if (int rc = PrepareOperandF32(ctx, call, 1, call->rhs_cache_policy, call->rhs_src_key, M, &b, err)) return rc;
-  if (N <= kSkinnyWidth || M <= kSkinnyWidth) {
-    // Bandwidth-bound shapes: stream the wide side once, no matrix instructions.
+  if (N <= kSkinnyKernelWidth || M <= kSkinnyKernelWidth) {
+    // Bandwidth-bound shapes: stream the wide side exactly once.
     GemvI8Args g;
-    g.swapped = !(N <= kSkinnyWidth && (M > kSkinnyWidth || M >= N));
+    g.swapped = !(N <= kSkinnyKernelWidth && (M > kSkinnyKernelWidth || M >= N));
     const OperandF32& wide = g.swapped ? b : a;
     const OperandF32& narrow = g.swapped ? a : b;
     g.wide = reinterpret_cast<const int8_t*>(wide.data);
