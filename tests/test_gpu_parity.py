@@ -504,10 +504,10 @@ def test_two_contexts_on_two_threads():
 
 
 @pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I16),
-                                 (S.U8, S.U8, S.I32, S.I32)], ids=cases.tuple_name)
+                                 (S.U8, S.U8, S.I32, S.I32), (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
 def test_skinny_nine_to_sixteen_vectors(device_ctx, tup):
-    """8-bit products whose narrow side has 9..16 vectors also go to the
-    streaming kernel (all 16 columns of its matrix instruction in use)."""
+    """8-bit and fp32 products whose narrow side has 9..16 vectors also go to
+    the streaming kernel (all 16 columns of its matrix instruction in use)."""
     rng = np.random.default_rng(321)
     for shape in [(300, 1500, 9), (16, 1500, 300), (1031, 2048, 16), (12, 4100, 513), (8200, 2099, 13),
                   (10, 5000, 8195), (64, 9000, 11), (16, 64, 16), (9, 16, 9), (500, 520, 15)]:
@@ -517,7 +517,7 @@ def test_skinny_nine_to_sixteen_vectors(device_ctx, tup):
             announce(p.name)
             got, want = run_both(device_ctx, p)
             compare(p, got, want)
-            assert device_ctx.last_kernel_name() == "i8_gemv"
+            assert device_ctx.last_kernel_name() == ("f32_gemv" if tup[0] == S.F32 else "i8_gemv")
 
 
 def test_caller_stream_asynchronous_calls_and_kernel_timing(device_ctx):
