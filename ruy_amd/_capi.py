@@ -16,6 +16,15 @@ if not os.path.exists(LIB_PATH):
         "%s is missing: build it with `python -m ruy_amd.build` "
         "(hipcc --offload-arch=gfx950); there is no CPU fallback" % LIB_PATH)
 
+# PyTorch's ROCm wheels bring their own copy of the HIP runtime, and a process
+# that ends up with two runtimes finds no device through the one loaded second.
+# Where torch is installed it is therefore imported first, so that this library
+# binds to the runtime torch loaded; without torch the system's runtime is used.
+try:
+    import torch  # noqa: F401
+except ImportError:
+    pass
+
 lib = C.CDLL(LIB_PATH)
 
 _ctx = C.c_void_p
