@@ -407,7 +407,8 @@ def main():
         if args.workload == "gemv":
             line.update({"metric": gv["metric"], "unit": "GB/s", "value": gv["value"],
                          "ms_per_step": gv["ms_per_step"], "roofline": gv["roofline"],
-                         "config": {"workload": gv["metric"], "kernel": gv["kernel"]}})
+                         "config": {"workload": gv["metric"], "kernel": gv["kernel"]},
+                         "more_columns": gv.get("more_columns")})
             if "cpu_baseline" in gv:
                 line["cpu_baseline"] = gv["cpu_baseline"]
         else:

@@ -97,6 +97,10 @@ struct GemvI8Args {
   int32_t fuse_sums = 0;
   int32_t fused_wide_factor = 0;
   int32_t fused_narrow_factor = 0;
+  // Matrix-core kernel: workgroup g starts its walk over the depth at step
+  // (g * rotate_step) mod steps (odd strides between 3 and 17 measured within
+  // 1 % of each other on the 16384^2 weights; 1 is 3 % slower).
+  int32_t rotate_step = 7;
   Epilogue ep;
   DevMat dst;
 };

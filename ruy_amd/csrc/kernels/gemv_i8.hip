@@ -223,7 +223,6 @@ __device__ __forceinline__ v4i RsrcWords(const void* p, uint32_t bytes) {
 // ---------------------------------------------------------------------------
 
 constexpr int kMmaRows = 16;
-constexpr int kRotate = 11;
 
 template <int N>
 __device__ __forceinline__ void WaitVmcnt() {
@@ -379,7 +378,7 @@ __global__ __launch_bounds__(64 * kSplit) void GemvMmaKernel(GemvI8Args args) {
   // side by side do not all ask the same memory channels at the same time.
   const int n_steps = s_end - s_begin;
   int next = 0;  // next step to issue, as an index into the rotated order
-  int phys = n_steps > 0 ? s_begin + (blockIdx.x * kRotate) % n_steps : 0;
+  int phys = n_steps > 0 ? s_begin + (blockIdx.x * args.rotate_step) % n_steps : 0;
   auto issue_next = [&](int ring_slot) {
     issue(phys, ring_slot);
     ++next;
