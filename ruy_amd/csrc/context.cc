@@ -4,6 +4,8 @@
 #include <cstdlib>
 #include <cstring>
 
+#include "kernels/gemm_i8.h"
+
 namespace ruyamd {
 
 Workspace::~Workspace() {
@@ -273,6 +275,15 @@ int ruyamd_ctx_create(ruyamd_ctx** out) {
     return RUYAMD_E_HIP;
   }
   ctx->stream = ctx->own_stream;
+  const std::size_t counter_bytes = std::size_t(ruyamd::GemmDepthSplitCounters()) * sizeof(uint32_t);
+  ctx->split_counters = static_cast<uint32_t*>(DeviceAlloc(counter_bytes));
+  if (!ctx->split_counters || hipMemsetAsync(ctx->split_counters, 0, counter_bytes, ctx->own_stream) != hipSuccess ||
+      hipStreamSynchronize(ctx->own_stream) != hipSuccess) {
+    DeviceFree(ctx->split_counters);
+    (void)hipStreamDestroy(ctx->own_stream);
+    delete ctx;
+    return RUYAMD_E_HIP;
+  }
   ctx->cache = MakeCache(PrepackedCache::kDefaultMaxBuffersBytes);
   *out = ctx;
   return RUYAMD_OK;
@@ -282,6 +293,7 @@ void ruyamd_ctx_destroy(ruyamd_ctx* ctx) {
   if (!ctx) return;
   (void)hipStreamSynchronize(ctx->stream);
   ctx->cache.reset();
+  DeviceFree(ctx->split_counters);
   for (auto* v : {&ctx->timing_pending, &ctx->timing_pool})
     for (auto& ev : *v) {
       (void)hipEventDestroy(ev.first);

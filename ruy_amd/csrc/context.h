@@ -105,6 +105,9 @@ struct ruyamd_ctx {
   ruyamd::HostStaging staging;
   std::unique_ptr<ruyamd::PrepackedCache> cache;
   int multiprocessor_count = 0;
+  // Arrival counters of the depth-split matrix-core kernels: zero between
+  // launches (the kernels leave them so), allocated with the context.
+  uint32_t* split_counters = nullptr;
   // Optional timing of the dominant kernel of each call.
   bool kernel_timing = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pending;

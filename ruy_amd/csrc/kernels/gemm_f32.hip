@@ -25,6 +25,8 @@ struct F32Traits {
   }
   static constexpr bool kSplitB = false;
   static __device__ __forceinline__ int Bits(float x, float) { return __float_as_int(x); }
+  static __device__ __forceinline__ int RawBits(float x) { return __float_as_int(x); }
+  static __device__ __forceinline__ float FromRawBits(int w) { return __int_as_float(w); }
 
   struct RowState {
     float bias[16];

@@ -54,7 +54,27 @@ struct GemmArgs {
   // be a multiple of 128, the kernel's depth step.
   uint32_t a_flip = 0;
   uint32_t b_flip = 0;
+  // Depth split (GemmDepthSplit): split_k > 1 launches that many workgroups
+  // per destination tile, each walking its part of the depth; they add their
+  // accumulators through split_partials (split_k * tile area * 4 bytes per
+  // tile) and elect the one that does the write-back with split_counters (one
+  // zero-initialised word per tile, left at zero by the kernel).
+  int32_t split_k = 1;
+  void* split_partials = nullptr;
+  uint32_t* split_counters = nullptr;
 };
+
+// How a launch of these arguments should split the depth: the number of parts
+// (1 = no split) and the bytes of split_partials it needs. `kind`: which
+// launcher the arguments are for.
+enum class GemmKind { kInt8, kInt8Int16, kF32 };
+struct DepthSplit {
+  int parts = 1;
+  size_t partial_bytes = 0;
+};
+DepthSplit GemmDepthSplit(const GemmArgs& args, int num_cus, GemmKind kind);
+// Number of 32-bit counters split_counters must hold.
+int GemmDepthSplitCounters();
 
 // True if LaunchGemmI8 would run these arguments on its smallest tile, the
 // one that has a variant with the sums fused in.

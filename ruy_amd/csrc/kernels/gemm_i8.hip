@@ -26,6 +26,8 @@ struct Int8Traits {
   }
   static constexpr bool kSplitB = false;
   static __device__ __forceinline__ int Bits(int x, int) { return x; }
+  static __device__ __forceinline__ int RawBits(int x) { return x; }
+  static __device__ __forceinline__ int FromRawBits(int w) { return w; }
 
   struct RowState {
     uint32_t add[16];
@@ -129,6 +131,12 @@ hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus
   return mfma_gemm::LaunchBest<Int8SplitTraits>(stream, args, num_cus);
 }
 
+DepthSplit GemmDepthSplit(const GemmArgs& args, int num_cus, GemmKind kind) {
+  return mfma_gemm::PlanDepthSplit(args, num_cus, kind == GemmKind::kInt8Int16);
+}
+
+int GemmDepthSplitCounters() { return mfma_gemm::kSplitCounters; }
+
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
   return mfma_gemm::PickTile(args, num_cus, false) == mfma_gemm::Tile::k64x64;
 }
@@ -139,10 +147,10 @@ hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
     // Both exist for the smallest tile only; flipped bytes need a whole number of depth steps.
     if (!GemmI8CanFuseSums(args, num_cus) || (flip && args.k_bytes % 128 != 0)) return hipErrorInvalidValue;
     if (flip) {
-      return args.fuse_sums ? mfma_gemm::Launch<Int8Traits, 1, 1, 128, 4, true, true>(stream, args)
-                            : mfma_gemm::Launch<Int8Traits, 1, 1, 128, 4, false, true>(stream, args);
+      return args.fuse_sums ? mfma_gemm::Launch<Int8Traits, 1, 1, 128, mfma_gemm::kSmallestTileStages, true, true>(stream, args)
+                            : mfma_gemm::Launch<Int8Traits, 1, 1, 128, mfma_gemm::kSmallestTileStages, false, true>(stream, args);
     }
-    return mfma_gemm::Launch<Int8Traits, 1, 1, 128, 4, true>(stream, args);
+    return mfma_gemm::Launch<Int8Traits, 1, 1, 128, mfma_gemm::kSmallestTileStages, true>(stream, args);
   }
   return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);
 }

@@ -29,7 +29,8 @@
 // for one 16-byte fragment pair, kSplitB (the B operand holds, for every 32
 // destination columns, 32 high-plane rows followed by 32 low-plane rows whose
 // accumulators are combined), Bits(x, x2) (accumulator element - or combined
-// pair - as raw 32 bits),
+// pair - as raw 32 bits), RawBits(x) / FromRawBits(w) (one accumulator element
+// to and from raw 32 bits),
 // RowState (per-destination-row write-back parameters, gathered once per lane)
 // and Finish(vals, rows, j, ep), which turns 16 raw accumulators of column j
 // into 16 destination values (as raw 32-bit words).
@@ -56,6 +57,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 
 constexpr int kGranule = 16;            // bytes per lane per load
+constexpr int kSmallestTileStages = 4;  // ring depth of the 64x64 tile
+constexpr int kSplitCounters = 1024;    // tiles a depth-split launch may have (one counter each)
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records we accept
 
 // Buffer descriptor words for a raw (stride 0) buffer of `bytes` bytes.
@@ -231,13 +234,24 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // running side by side do not ask the same memory channels at the same
   // time. The order of the steps does not matter for the sums. Steps past the
   // end keep their index, which puts them out of range as before.
-  const int k_tiles = (K + kBK - 1) / kBK;
+  //
+  // Depth split (tiles of at most two blocks per wave, args.split_k > 1): the
+  // workgroups of grid row blockIdx.y walk the blockIdx.y-th part of the depth
+  // steps only; their accumulators are added up before the write-back (below).
+  // k_tiles, kt_first: the steps this workgroup walks.
+  const int k_tiles_all = (K + kBK - 1) / kBK;
+  constexpr bool kCanSplitDepth = WM * WN <= 2;
+  const int split = kCanSplitDepth ? args.split_k : 1;
+  const int split_index = kCanSplitDepth ? blockIdx.y : 0;
+  const int k_tiles_per_split = (k_tiles_all + split - 1) / split;
+  const int kt_first = split_index * k_tiles_per_split;
+  const int k_tiles = max(0, min(k_tiles_per_split, k_tiles_all - kt_first));
   constexpr bool kRotateDepth = WM * WN < 16;
-  const int rot = kRotateDepth && K % kBK == 0 ? (tile_m * 5) % k_tiles : 0;
+  const int rot = kRotateDepth && K % kBK == 0 && k_tiles > 0 ? (tile_m * 5 + split_index * 3) % k_tiles : 0;
   auto phys = [&](int kt) {
     if constexpr (!kRotateDepth) return kt;
     const int p = kt + rot;
-    return kt >= k_tiles ? kt : p >= k_tiles ? p - k_tiles : p;
+    return kt >= k_tiles ? k_tiles_all + kt : kt_first + (p >= k_tiles ? p - k_tiles : p);
   };
   auto issue_one = [&](int kt, int n) {
     const int kbase = phys(kt) * kBK;
@@ -408,7 +422,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // (a partial step and the ones past the end, which fetch zeros) take the
   // bounds-tested form.
   int kt = 0;
-  const int full_end = K / kBK - C::kStages;
+  const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
   for (; kt < full_end; ++kt) ring_step(kt, std::true_type());
   for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type());
   WaitVmcnt<0>();
@@ -423,6 +437,74 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
     for (int v = 0; v < 16; ++v)
       acc[0][kBlock][v] = static_cast<int>(static_cast<uint32_t>(acc[0][kBlock][v]) -
                                            fa * static_cast<uint32_t>(sum_a[v]) - fb * static_cast<uint32_t>(sum_b[v]));
+  }
+
+  // ---- depth split: add up the partial accumulators ----
+  // Every workgroup of a tile stores its accumulators (as they sit in the
+  // registers, 8 bytes per thread and store) and then counts itself in; the
+  // one that arrives last reads all parts back, in the order of the depth
+  // parts so that the fp32 sum does not depend on who was last, and goes on to
+  // the write-back. Nobody waits for anybody. The counter is left at zero for
+  // the next launch.
+  // The parts travel between workgroups that may sit on different XCDs, whose
+  // L2 caches do not see each other's lines: every access to them and to the
+  // counter is a device-scope atomic (relaxed: a plain store or load that goes
+  // past the caches that are not shared), the stores are awaited before the
+  // counter is touched, and the loads are issued after its value is known.
+  // That costs nothing when no split is asked for, where fences at device
+  // scope would write back and invalidate whole caches.
+  if constexpr (kCanSplitDepth) {
+    if (split > 1) {
+      typedef unsigned long long u64;
+      constexpr int kPartWords = C::kBM * C::kBN;  // 32-bit words of one tile's accumulators
+      u64* parts = static_cast<u64*>(args.split_partials) + size_t(t) * split * (kPartWords / 2);
+      u64* mine = parts + size_t(split_index) * (kPartWords / 2) + tid;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+          for (int h = 0; h < 8; ++h) {
+            const u64 w = u64(uint32_t(Traits::RawBits(acc[i][j][2 * h]))) |
+                          (u64(uint32_t(Traits::RawBits(acc[i][j][2 * h + 1]))) << 32);
+            __hip_atomic_store(mine + ((i * WN + j) * 8 + h) * C::kThreads, w, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+          }
+      WaitVmcnt<0>();
+      __syncthreads();
+      unsigned* arrived = reinterpret_cast<unsigned*>(lds);
+      if (tid == 0)
+        *arrived = __hip_atomic_fetch_add(args.split_counters + t, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      const bool last = *arrived == unsigned(split - 1);
+      __syncthreads();  // the flag's LDS word is part of the write-back's staging area
+      if (!last) return;
+      if (tid == 0) __hip_atomic_store(args.split_counters + t, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+      // This workgroup's own part is read back like the others: one code path,
+      // one summation order. A few parts' loads are in flight together.
+      constexpr int kPartsInFlight = 4 / (WM * WN);
+#pragma unroll kPartsInFlight
+      for (int z = 0; z < split; ++z) {
+        const u64* part = parts + size_t(z) * (kPartWords / 2) + tid;
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int h = 0; h < 8; ++h) {
+              const u64 w = __hip_atomic_load(part + ((i * WN + j) * 8 + h) * C::kThreads, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+              acc[i][j][2 * h] += Traits::FromRawBits(static_cast<int>(uint32_t(w)));
+              acc[i][j][2 * h + 1] += Traits::FromRawBits(static_cast<int>(uint32_t(w >> 32)));
+            }
+      }
+    }
   }
 
   // ---- fused write-back ----
@@ -560,7 +642,16 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
         reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
     if (attr != hipSuccess) return attr;
   }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::kThreads), lds_bytes, stream, args);
+  // The depth split exists for the small tiles only, needs its buffers, and
+  // every part must have at least one depth step.
+  const int split = args.split_k;
+  if (split != 1) {
+    const int k_tiles = (args.k_bytes + BK - 1) / BK;
+    if (WM * WN > 2 || split < 1 || !args.split_partials || !args.split_counters || total > kSplitCounters ||
+        (split - 1) * ((k_tiles + split - 1) / split) >= k_tiles)
+      return hipErrorInvalidValue;
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid, split), dim3(C::kThreads), lds_bytes, stream, args);
   return hipGetLastError();
 }
 
@@ -607,6 +698,39 @@ inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   return Tile::k64x64;
 }
 
+// Depth split for a launch of `args` (see GemmArgs::split_k). Only the
+// smallest tile has it (64x64, or 64 rows x 128 plane columns for the
+// plane-split operand): adding up the parts costs time in proportion to the
+// tile's area, and with larger tiles that outweighed the gain at every shape
+// measured. One workgroup streams its operands at a rate that the CU's
+// outstanding-request capacity fixes (about 35 GB/s), whatever the depth of the
+// ring, so a problem with few tiles and a long depth only gets faster by
+// putting more workgroups on it. The split is taken when the tiles alone leave
+// CUs idle, aims at as many workgroups per CU as the ring's LDS lets run
+// together (two, one for the plane-split tile), and keeps at least
+// kMinStepsPerPart depth steps in every part so that filling the ring and
+// adding up the parts (about as long as one depth step per part) stay small
+// against the work shared out.
+inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, bool split_b) {
+  constexpr int kMinStepsPerPart = 8;
+  constexpr int kMaxParts = 32;
+  const Tile tile = PickTile(args, num_cus, split_b);
+  if (tile != (split_b ? Tile::k64x128 : Tile::k64x64)) return DepthSplit();
+  const int bm = 64, bn = split_b ? 128 : 64;
+  const int tiles = TileCount(args, bm, bn);
+  const int k_tiles = (args.k_bytes + 127) / 128;
+  if (tiles == 0 || tiles > kSplitCounters) return DepthSplit();
+  const int resident_per_cu = split_b ? 1 : 2;
+  int parts = std::min({resident_per_cu * num_cus / tiles, k_tiles / kMinStepsPerPart, kMaxParts});
+  if (parts < 2) return DepthSplit();
+  const int steps_per_part = (k_tiles + parts - 1) / parts;
+  parts = (k_tiles + steps_per_part - 1) / steps_per_part;  // no empty part
+  DepthSplit split;
+  split.parts = parts;
+  split.partial_bytes = size_t(parts) * tiles * bm * bn * 4;
+  return split;
+}
+
 template <typename Traits>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
   switch (PickTile(args, num_cus, Traits::kSplitB)) {
@@ -628,7 +752,7 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
       case Tile::k128x64:
         return Launch<Traits, 2, 1, 128, 4>(stream, args);
       default:
-        return Launch<Traits, 1, 1, 128, 4>(stream, args);
+        return Launch<Traits, 1, 1, 128, kSmallestTileStages>(stream, args);
     }
   }
   return hipErrorInvalidValue;

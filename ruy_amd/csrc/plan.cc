@@ -175,6 +175,19 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
   return RUYAMD_OK;
 }
 
+// Few destination tiles and a long depth: lets the kernel split the depth over
+// several workgroups per tile if the workspace has (or may get) room for their
+// partial accumulators. Without room the launch simply stays unsplit.
+void PlanDepthSplit(ruyamd_ctx* ctx, GemmKind kind, GemmArgs* args) {
+  const DepthSplit split = GemmDepthSplit(*args, ctx->multiprocessor_count, kind);
+  if (split.parts < 2) return;
+  void* partials = ctx->workspace.Alloc(split.partial_bytes);
+  if (!partials) return;
+  args->split_k = split.parts;
+  args->split_partials = partials;
+  args->split_counters = ctx->split_counters;
+}
+
 int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const DevMat& lhs = call->lhs;
   const DevMat& rhs = call->rhs;
@@ -289,6 +302,7 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   }
   args.ep.lhs_sums = x.sums;
   args.ep.rhs_sums = y.sums;
+  PlanDepthSplit(ctx, GemmKind::kInt8, &args);
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
@@ -449,6 +463,7 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.M = swap ? N : M;
   args.N = swap ? M : N;
   args.n_logical = args.N;
+  PlanDepthSplit(ctx, GemmKind::kF32, &args);
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmF32(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
@@ -517,6 +532,7 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     return rc;
   }
   args.ep.lhs_sums = a.sums;
+  PlanDepthSplit(ctx, GemmKind::kInt8Int16, &args);
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8I16(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();

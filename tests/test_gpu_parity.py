@@ -631,6 +631,32 @@ def test_uint8_operands_used_in_place(device_ctx, tup):
             compare(p, got, want)
 
 
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.U8), (S.I8, S.I8, S.I32, S.I32),
+                                 (S.I8, S.I16, S.I32, S.I16), (S.I16, S.I8, S.I32, S.I16),
+                                 (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
+def test_deep_shapes_that_split_the_depth(device_ctx, tup):
+    """Few destination tiles and a long depth: the tiled kernels put several
+    workgroups on every tile, each walking a part of the depth, and add the
+    parts up before the write-back. One tile and several, whole and ragged
+    depths (the last part then ends in a partial step), depths that divide
+    unevenly over the parts, operands used in place (sums formed by the kernel,
+    uint8 bytes flipped on the way in) and packed ones. Every problem runs
+    three times on the same context: the arrival counters must be back at
+    zero after each launch."""
+    rng = np.random.default_rng(909)
+    shapes = [(64, 4096, 64), (100, 5016, 70), (256, 8192, 256), (200, 3088, 130), (128, 16400, 128),
+              (64, 1024, 64), (17, 3000, 33), (320, 2176, 192)]
+    for shape in shapes:
+        for orders in (cases.RCC, (1, 0, 1)):
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=False,
+                                 name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+            announce(p.name)
+            import device_runner as D
+            want = expected(p)
+            for _ in range(3):
+                compare(p, D.device_mul(device_ctx, p), want)
+
+
 def test_operand_of_more_than_2_gib(device_ctx):
     """A 2.18 GB int8 LHS (66560 x 32768): the tuned kernels address an
     operand through 32-bit offsets, so the library computes the destination in
