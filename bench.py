@@ -37,8 +37,11 @@ HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E peak, GB/s
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # The card's clock takes about 50 ms of load to settle after an idle period
+    # (the 8192^3 step measures 5 % slower in the first tens of steps), so the
+    # default warm-up is long enough to time the sustained rate.
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="all", choices=["all", "gemm", "gemv"])
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the int8 GEMM")
     ap.add_argument("--gemv-size", type=int, default=16384, help="M=K of the int8 GEMV")

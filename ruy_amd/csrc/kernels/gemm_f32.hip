@@ -24,6 +24,9 @@ struct F32Traits {
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[e]), __int_as_float(b[e]), acc, 0, 0, 0);
   }
   static constexpr bool kSplitB = false;
+  // Time between two dependent launches (about 5 us) in depth steps of the
+  // 256x256 tile (32 floats deep, 7.8 us each).
+  static constexpr double kLaunchGapInDepthSteps = 0.65;
   static __device__ __forceinline__ int Bits(float x, float) { return __float_as_int(x); }
   static __device__ __forceinline__ int RawBits(float x) { return __float_as_int(x); }
   static __device__ __forceinline__ float FromRawBits(int w) { return __int_as_float(w); }

@@ -670,7 +670,11 @@ enum class Tile { k256x256, k256x128, k128x256, k128x128, k128x64, k64x128, k64x
 // (or only) round would leave most CUs idle. `split_b`: the plane-split form
 // of the int16 kernel, which has the two square large tiles and a 64x128 one.
 constexpr double kEffHalf = 0.55;
-inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
+struct TileChoice {
+  Tile tile;
+  double cost;  // rounds x tile area / efficiency
+};
+inline TileChoice BestTile(const GemmArgs& args, int num_cus, bool split_b) {
   auto cost = [&](int bm, int bn, double efficiency) {
     const int rounds = (TileCount(args, bm, bn) + num_cus - 1) / num_cus;
     return rounds * double(bm) * double(bn) / efficiency;
@@ -680,8 +684,8 @@ inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   if (split_b) {
     // Plane-split operand: the smallest tile is 64 rows x 128 plane columns (64 destination columns).
     const double c64x128 = cost(64, 128, 0.5);
-    if (c256 <= c128 && c256 <= c64x128) return Tile::k256x256;
-    return c128 <= c64x128 ? Tile::k128x128 : Tile::k64x128;
+    if (c256 <= c128 && c256 <= c64x128) return {Tile::k256x256, c256};
+    return c128 <= c64x128 ? TileChoice{Tile::k128x128, c128} : TileChoice{Tile::k64x128, c64x128};
   }
   const double c64 = cost(64, 64, 0.45);
   const double c256x128 = cost(256, 128, 0.75);
@@ -689,13 +693,89 @@ inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
   const double c128x64 = cost(128, 64, kEffHalf);
   const double c64x128 = cost(64, 128, kEffHalf);
   const double best = std::min({c256, c128, c64, c256x128, c128x256, c128x64, c64x128});
-  if (c256 == best) return Tile::k256x256;
-  if (c256x128 == best) return Tile::k256x128;
-  if (c128x256 == best) return Tile::k128x256;
-  if (c128 == best) return Tile::k128x128;
-  if (c128x64 == best) return Tile::k128x64;
-  if (c64x128 == best) return Tile::k64x128;
-  return Tile::k64x64;
+  if (c256 == best) return {Tile::k256x256, best};
+  if (c256x128 == best) return {Tile::k256x128, best};
+  if (c128x256 == best) return {Tile::k128x256, best};
+  if (c128 == best) return {Tile::k128x128, best};
+  if (c128x64 == best) return {Tile::k128x64, best};
+  if (c64x128 == best) return {Tile::k64x128, best};
+  return {Tile::k64x64, best};
+}
+inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
+  return BestTile(args, num_cus, split_b).tile;
+}
+
+// The sub-problem of `args` whose destination is rows [m_begin, m_begin +
+// m_count) x columns [n_begin, n_begin + n_count) of the original one: operand,
+// destination and per-row / per-column parameter pointers advanced, nothing
+// else changed. Not for the plane-split operand.
+inline GemmArgs SubProblem(const GemmArgs& args, int m_begin, int m_count, int n_begin, int n_count) {
+  GemmArgs sub = args;
+  const uint32_t a_skip = uint32_t(m_begin) * uint32_t(args.lda);
+  const uint32_t b_skip = uint32_t(n_begin) * uint32_t(args.ldb);
+  sub.a = static_cast<const char*>(args.a) + a_skip;
+  sub.b = static_cast<const char*>(args.b) + b_skip;
+  sub.a_bytes = args.a_bytes > a_skip ? args.a_bytes - a_skip : 0;
+  sub.b_bytes = args.b_bytes > b_skip ? args.b_bytes - b_skip : 0;
+  sub.M = m_count;
+  sub.N = n_count;
+  sub.n_logical = n_count;
+  sub.dst.rows = m_count;
+  sub.dst.cols = n_count;
+  sub.dst.data = static_cast<char*>(args.dst.data) +
+                 (int64_t(m_begin) * args.dst.rs + int64_t(n_begin) * args.dst.cs) * args.dst_elt;
+  sub.dst_vector_ok = (reinterpret_cast<uintptr_t>(sub.dst.data) & 15) == 0 && (args.dst.cs * args.dst_elt) % 16 == 0;
+  if (args.ep.lhs_sums) sub.ep.lhs_sums = args.ep.lhs_sums + m_begin;
+  if (args.ep.rhs_sums) sub.ep.rhs_sums = args.ep.rhs_sums + n_begin;
+  const int channel_begin = args.ep.channel_is_col ? n_begin : m_begin;
+  if (args.ep.bias) sub.ep.bias = static_cast<const char*>(args.ep.bias) + int64_t(channel_begin) * 4;  // int32 or fp32
+  if (args.ep.mult_fixedpoint) sub.ep.mult_fixedpoint = args.ep.mult_fixedpoint + channel_begin;
+  if (args.ep.mult_exponent) sub.ep.mult_exponent = args.ep.mult_exponent + channel_begin;
+  return sub;
+}
+
+// A grid of 256x256 tiles whose last round of workgroups would leave most CUs
+// idle (576 tiles on 256 CUs: three rounds for 2.25 rounds of work) is cut in
+// two launches: whole tile columns (or rows) that fill their rounds, and the
+// rest of the destination on whichever tile suits that strip best. The second
+// launch starts when the first has drained, which costs a few microseconds,
+// expressed here in depth steps of the large tile (`gap_steps`). The model
+// overstates the gain (a last round on a quarter of the CUs runs at a higher
+// clock than a full one; measured gains were about a third of the modelled
+// ones), so the cut is taken only for grids of at least 8 x 8 tiles and a
+// modelled saving of 12 % or more: 4608^3 135 -> 127 us, 7168^3 420 -> 396 us.
+struct TailPlan {
+  bool use = false;
+  bool along_n = false;  // the cut runs between tile columns (else between tile rows)
+  int main_tiles = 0;    // tile columns (rows) in the first launch
+};
+inline TailPlan PlanTail(const GemmArgs& args, int num_cus, double gap_steps) {
+  TailPlan plan;
+  const int tiles_m = (args.M + 255) / 256, tiles_n = (args.N + 255) / 256;
+  const int total = tiles_m * tiles_n;
+  if (total <= num_cus || total % num_cus == 0 || tiles_m < 8 || tiles_n < 8) return plan;
+  const double round_cost = 256.0 * 256.0;
+  const double single = double((total + num_cus - 1) / num_cus) * round_cost;
+  const int k_steps = std::max(1, (args.k_bytes + 127) / 128);
+  const double gap = gap_steps * round_cost / k_steps;
+  double best = single * 0.88;
+  for (int along_n = 0; along_n < 2; ++along_n) {
+    const int across = along_n ? tiles_m : tiles_n;  // tiles per column (row) of tiles
+    const int count = along_n ? tiles_n : tiles_m;
+    for (int c = 1; c < count; ++c) {
+      const int main_rounds = (across * c + num_cus - 1) / num_cus;
+      GemmArgs tail = args;
+      (along_n ? tail.N : tail.M) -= c * 256;
+      const double cost = main_rounds * round_cost + BestTile(tail, num_cus, false).cost + gap;
+      if (cost < best) {
+        best = cost;
+        plan.use = true;
+        plan.along_n = along_n != 0;
+        plan.main_tiles = c;
+      }
+    }
+  }
+  return plan;
 }
 
 // Depth split for a launch of `args` (see GemmArgs::split_k). Only the
@@ -732,8 +812,8 @@ inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, bool split_b
 }
 
 template <typename Traits>
-hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
-  switch (PickTile(args, num_cus, Traits::kSplitB)) {
+hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile) {
+  switch (tile) {
     case Tile::k256x256:
       return Launch<Traits, 4, 4, 128, 2>(stream, args);
     case Tile::k128x128:
@@ -744,7 +824,7 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
       break;
   }
   if constexpr (!Traits::kSplitB) {
-    switch (PickTile(args, num_cus, false)) {
+    switch (tile) {
       case Tile::k256x128:
         return Launch<Traits, 4, 2, 128, 3>(stream, args);
       case Tile::k128x256:
@@ -756,6 +836,26 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
     }
   }
   return hipErrorInvalidValue;
+}
+
+template <typename Traits>
+hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
+  const Tile tile = PickTile(args, num_cus, Traits::kSplitB);
+  if constexpr (!Traits::kSplitB) {
+    if (tile == Tile::k256x256 && args.split_k == 1 && !args.fuse_sums) {
+      const TailPlan plan = PlanTail(args, num_cus, Traits::kLaunchGapInDepthSteps);
+      if (plan.use) {
+        const int cut = plan.main_tiles * 256;
+        const GemmArgs main = plan.along_n ? SubProblem(args, 0, args.M, 0, cut) : SubProblem(args, 0, cut, 0, args.N);
+        const GemmArgs tail = plan.along_n ? SubProblem(args, 0, args.M, cut, args.N - cut)
+                                           : SubProblem(args, cut, args.M - cut, 0, args.N);
+        const hipError_t first = Launch<Traits, 4, 4, 128, 2>(stream, main);
+        if (first != hipSuccess) return first;
+        return LaunchTile<Traits>(stream, tail, PickTile(tail, num_cus, false));
+      }
+    }
+  }
+  return LaunchTile<Traits>(stream, args, tile);
 }
 
 }  // namespace mfma_gemm

@@ -657,6 +657,59 @@ def test_deep_shapes_that_split_the_depth(device_ctx, tup):
                 compare(p, D.device_mul(device_ctx, p), want)
 
 
+def _boundary_sample(rng, n, step=256, random_count=40):
+    """Indices in [0, n): a random handful, both ends, and two either side of
+    every multiple of `step` (where tiles, and launches cut between tiles, meet)."""
+    picks = [rng.choice(n, min(random_count, n), replace=False), np.arange(0, min(4, n)), np.arange(max(n - 4, 0), n)]
+    for edge in range(step, n, step):
+        picks.append(np.arange(edge - 2, min(edge + 2, n)))
+    return np.unique(np.concatenate(picks))
+
+
+@pytest.mark.parametrize("shape,tup", [((4608, 4608, 4608), (S.I8, S.I8, S.I32, S.I8)),
+                                       ((4056, 4096, 8348), (S.U8, S.I8, S.I32, S.I16)),
+                                       ((7000, 4096, 3000), (S.I8, S.U8, S.I32, S.U8)),
+                                       ((4608, 1024, 4608), (S.F32, S.F32, S.F32, S.F32))],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v[0], int) and v[0] > 16 else cases.tuple_name(v))
+def test_grids_cut_into_two_launches(device_ctx, shape, tup):
+    """Destinations whose 256x256 tiles make a whole number of rounds of
+    workgroups plus a small rest (324, 528, 336 tiles on 256 CUs): the
+    tiled kernel runs as two launches, whole tile rows or columns first and the
+    remaining strip on a smaller tile, with the per-row / per-column parameters
+    and the sums advanced to the strip. Both cut directions, ragged edges,
+    row-major and column-major destinations, per-channel parameters as the
+    random problem draws them. Too large for the checker as a whole:
+    requantized results are compared on a sample of rows and columns that
+    includes both sides of every tile edge, and for the integer cases every
+    element of the raw int32 product enters a row/column checksum."""
+    import device_runner as D
+    M, K, N = shape
+    rng = np.random.default_rng(5150 + M)
+    for orders in (cases.RCC, (1, 0, 1)):
+        p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
+                             name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+        if tup[0] != S.F32:
+            if p.lhs.zero_point in (0, 128):
+                p.lhs.zero_point = 9 if tup[0] == S.I8 else 121
+            if p.rhs.zero_point in (0, 128):
+                p.rhs.zero_point = -5 if tup[1] == S.I8 else 131
+        announce(p.name)
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        rows, cols = _boundary_sample(rng, M), _boundary_sample(rng, N)
+        g, w = _sample_block(p, got, rows, cols)
+        if tup[0] == S.F32:
+            err = np.linalg.norm(g.astype(np.float64) - w) / np.linalg.norm(w)
+            assert err <= REL_FROBENIUS_TOL, err
+            continue
+        assert (g == w).all(), "%d mismatches in the sampled block" % (g != w).sum()
+        raw = W.Problem("raw", p.lhs, p.rhs, W.HostMatrix(S.I32, M, N, S.ORDER_COL_MAJOR), S.I32)
+        got = O.dense_of(raw, D.device_mul(device_ctx, raw, dst_fill=0)).astype(np.int64)
+        L = p.lhs.dense().astype(np.int64) - p.lhs.zero_point
+        R = p.rhs.dense().astype(np.int64) - p.rhs.zero_point
+        assert ((got.sum(axis=0) % 2**32) == (L.sum(axis=0) @ R) % 2**32).all()
+        assert ((got.sum(axis=1) % 2**32) == (L @ R.sum(axis=1)) % 2**32).all()
+
+
 def test_operand_of_more_than_2_gib(device_ctx):
     """A 2.18 GB int8 LHS (66560 x 32768): the tuned kernels address an
     operand through 32-bit offsets, so the library computes the destination in
