@@ -200,6 +200,17 @@ def test_empty_and_degenerate_shapes(device_ctx):
         p = W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, *shape, 1, 0, 0)
         got, want = run_both(device_ctx, p)
         compare(p, got, want)
+    # Depth 0 at sizes that reach the tiled and the skinny kernels: the result
+    # is bias, zero-point terms (none are left), requantization and clamp only.
+    for tup in [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I32), (S.I8, S.I16, S.I32, S.I16),
+                (S.F32, S.F32, S.F32, S.F32)]:
+        for shape in [(300, 0, 200), (5, 0, 300), (300, 0, 5), (1, 0, 70), (0, 0, 0), (0, 300, 300), (300, 300, 0)]:
+            for orders in (cases.RCC, (1, 0, 1)):
+                p = W.random_problem(rng, *tup, *shape, *orders,
+                                     name="%s %s %s" % (cases.tuple_name(tup), shape, orders))
+                announce(p.name)
+                got, want = run_both(device_ctx, p)
+                compare(p, got, want)
 
 
 def test_rejects_what_the_reference_forbids(device_ctx):
