@@ -21,27 +21,35 @@ def to_dev(arr):
 class DeviceProblem:
     """Device-resident copy of a Problem: tensors + the two descriptor structs."""
 
-    def __init__(self, problem, dst_fill=0x5A):
+    def __init__(self, problem, dst_fill=0x5A, misalign=0):
+        """`misalign`: every buffer starts that many elements into its
+        allocation, so that base addresses are not 16-byte aligned."""
         p = problem
         self.problem = p
-        self.lhs_t = to_dev(p.lhs.storage)
-        self.rhs_t = to_dev(p.rhs.storage)
+
+        def shifted(arr):
+            if not misalign:
+                return to_dev(arr)
+            return to_dev(np.concatenate([np.zeros(misalign, arr.dtype), arr]))[misalign:]
+
+        self.lhs_t = shifted(p.lhs.storage)
+        self.rhs_t = shifted(p.rhs.storage)
         d = p.dst
         # The destination sits between two guard zones that must come back
         # untouched (the idea of the reference's guard-page allocator,
         # ruy/test.h:395-445, for a device buffer).
-        self.guard = GUARD_ELEMENTS
+        self.guard = GUARD_ELEMENTS + misalign
         self.n_dst = max(d.n_storage, 1)
         fill = np.full(self.n_dst + 2 * self.guard, 0, dtype=d.storage.dtype)
         fill.view(np.uint8)[:] = dst_fill
         self.dst_fill = dst_fill
         self.dst_all = to_dev(fill)
         self.dst_t = self.dst_all[self.guard:self.guard + self.n_dst]
-        self.bias_t = to_dev(p.bias) if p.bias is not None else None
+        self.bias_t = shifted(p.bias) if p.bias is not None else None
         self.mf_t = self.me_t = None
         if p.multiplier_fixedpoint_perchannel is not None:
-            self.mf_t = to_dev(p.multiplier_fixedpoint_perchannel)
-            self.me_t = to_dev(p.multiplier_exponent_perchannel)
+            self.mf_t = shifted(p.multiplier_fixedpoint_perchannel)
+            self.me_t = shifted(p.multiplier_exponent_perchannel)
         self.lhs_s = p.lhs.struct(self.lhs_t.data_ptr())
         self.rhs_s = p.rhs.struct(self.rhs_t.data_ptr())
         self.dst_s = p.dst.struct(self.dst_t.data_ptr())
@@ -64,10 +72,10 @@ class DeviceProblem:
         return everything[self.guard:self.guard + self.n_dst].copy()
 
 
-def device_mul(ctx, problem, dst_fill=0x5A):
+def device_mul(ctx, problem, dst_fill=0x5A, misalign=0):
     """dst storage (numpy, same layout as problem.dst) computed on the GPU from
     device-resident operands; untouched elements keep the fill byte."""
-    dp = DeviceProblem(problem, dst_fill)
+    dp = DeviceProblem(problem, dst_fill, misalign)
     dp.run(ctx)
     return dp.result()
 

@@ -721,6 +721,25 @@ def test_grids_cut_into_two_launches(device_ctx, shape, tup):
         assert ((got.sum(axis=1) % 2**32) == (L @ R.sum(axis=1)) % 2**32).all()
 
 
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I16), (S.I8, S.I16, S.I32, S.I16),
+                                 (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
+def test_base_addresses_that_are_not_aligned(device_ctx, tup):
+    """Every buffer (operands, destination, bias, multipliers) starts 1 or 3
+    elements into its allocation: the kernels that read operands in place and
+    store 16 bytes at a time need aligned addresses, so these calls take the
+    packed route and the element-wise stores, on the tiled, the skinny and the
+    one-column kernels. The guard zones around the destination stay intact."""
+    import device_runner as D
+    rng = np.random.default_rng(31337)
+    for shape in [(200, 256, 300), (300, 1024, 7), (9, 512, 400), (500, 2048, 1), (64, 4096, 64), (130, 130, 130)]:
+        for misalign in (1, 3):
+            orders = cases.ALL_ORDERS[int(rng.integers(8))]
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=False,
+                                 name="%s %s %s +%d" % (cases.tuple_name(tup), shape, orders, misalign))
+            announce(p.name)
+            compare(p, D.device_mul(device_ctx, p, misalign=misalign), expected(p))
+
+
 def test_operand_of_more_than_2_gib(device_ctx):
     """A 2.18 GB int8 LHS (66560 x 32768): the tuned kernels address an
     operand through 32-bit offsets, so the library computes the destination in
