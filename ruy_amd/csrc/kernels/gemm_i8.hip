@@ -150,10 +150,10 @@ hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
     // Both exist for the smallest tile only; flipped bytes need a whole number of depth steps.
     if (!GemmI8CanFuseSums(args, num_cus) || (flip && args.k_bytes % 128 != 0)) return hipErrorInvalidValue;
     if (flip) {
-      return args.fuse_sums ? mfma_gemm::Launch<Int8Traits, 1, 1, 128, mfma_gemm::kSmallestTileStages, true, true>(stream, args)
-                            : mfma_gemm::Launch<Int8Traits, 1, 1, 128, mfma_gemm::kSmallestTileStages, false, true>(stream, args);
+      return args.fuse_sums ? mfma_gemm::LaunchSmallestTile<Int8Traits, true, true>(stream, args)
+                            : mfma_gemm::LaunchSmallestTile<Int8Traits, false, true>(stream, args);
     }
-    return mfma_gemm::Launch<Int8Traits, 1, 1, 128, mfma_gemm::kSmallestTileStages, true>(stream, args);
+    return mfma_gemm::LaunchSmallestTile<Int8Traits, true>(stream, args);
   }
   return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);
 }

@@ -20,7 +20,9 @@
 // buffer_load_dwordx4 ... lds (global memory straight into LDS, no registers),
 // a whole step or more ahead of the matrix instructions. Rows past the end of
 // a matrix and depth granules past K read as zero through the buffer
-// descriptor's bounds check. The 16-byte granules of an LDS row are
+// descriptor's bounds check. (The 64x64 tile has a schedule of its own,
+// with the depth dealt out to the waves instead of the tile's blocks: see
+// kDepthWaves in the kernel.) The 16-byte granules of an LDS row are
 // XOR-swizzled by the row number so that a ds_read_b128 of 16 consecutive rows
 // touches all 64 banks; since a direct-to-LDS load places lane l at
 // base + 16*l, the swizzle is applied to the global address each lane fetches.
@@ -57,7 +59,6 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 
 constexpr int kGranule = 16;            // bytes per lane per load
-constexpr int kSmallestTileStages = 4;  // ring depth of the 64x64 tile
 constexpr int kSplitCounters = 1024;    // tiles a depth-split launch may have (one counter each)
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records we accept
 
@@ -158,11 +159,14 @@ struct Cfg {
 // kFlip (same tile only): args.a_flip / args.b_flip are applied to every
 // fragment before use, which turns uint8 data used in place into the int8
 // values the arithmetic is defined on.
-template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false>
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
+          bool kDepthWaves = false>
 __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
                 "fused sums exist for the tiles with one block (one block per plane) per wave only");
   static_assert(!kFlip || WM * WN == 1, "in-place uint8 operands exist for the single-block tile only");
+  static_assert(!kDepthWaves || (WM * WN == 1 && BK == 128 && STAGES == 8 && !Traits::kSplitB),
+                "the depth-per-wave schedule exists for the 64x64 tile, with two ring slots of 16 KiB per wave");
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   constexpr int kBK = BK;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -399,35 +403,181 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // kt+1: wait until its loads have landed, barrier (after which every wave has
   // also finished reading step kt, so its ring slot is free), issue the loads
   // of step kt+kStages into that slot, then read fragments (kt+1, 0).
+  if constexpr (kDepthWaves) {
+    // ---- the 64x64 tile, one wave per part of the depth ----
+    // With one 32x32 block per wave a depth step is four dependent matrix
+    // instructions and some eighty others around them (loads, LDS reads,
+    // waits, a barrier), and a lone wave issues an instruction every four or
+    // five cycles: the step takes a thousand cycles however deep the ring is.
+    // Here every wave computes the whole 64x64 tile (2 x 2 independent blocks)
+    // for every fourth depth step, through a two-slot ring of its own and
+    // without any barrier: four times the matrix work per LDS read and per
+    // load, and nobody to wait for. The four partial tiles are added through
+    // LDS afterwards, which leaves wave (wave_m, wave_n) with its block as in
+    // the other schedule.
+    constexpr int kSlotBytes = C::kStageBytes;  // 64 A rows + 64 B rows, 128 bytes each
+    constexpr int kLoads = kSlotBytes / 1024;
+    static_assert(kLoads == 16 && C::kBM == 64 && C::kBN == 64, "");
+    char* ring = lds + wave * 2 * kSlotBytes;
+    const uint32_t ring_base = lds_base + wave * 2 * kSlotBytes;
+    // Load n of a step fills rows 8n .. 8n+7 of the slot (A rows first).
+    uint32_t goff[kLoads];
+    int gk[kLoads];
 #pragma unroll
-  for (int s = 0; s < C::kStages; ++s) issue(s);
-  WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
-  __syncthreads();
-  Frags f[2];
-  read_frags(0, 0, f[0]);
-  auto ring_step = [&](int kt, auto dma_is_full_step) {
+    for (int n = 0; n < kLoads; ++n) {
+      const int r = (n % 8) * 8 + lane / 8;  // row inside its operand's tile
+      const int g = (lane % 8) ^ Swizzle<BK>(r);
+      gk[n] = g * kGranule;
+      if (n < 8)
+        goff[n] = m0 + r < args.M ? uint32_t(m0 + r) * uint32_t(args.lda) + g * kGranule : kOutOfRange;
+      else
+        goff[n] = n0 + r < args.N ? uint32_t(n0 + r) * uint32_t(args.ldb) + g * kGranule : kOutOfRange;
+    }
+    auto issue_step = [&](int step, int slot) {
+      const int kbase = phys(step) * kBK;
+      const uint32_t dst = ring_base + slot * kSlotBytes;
+      if (kbase + kBK <= K) {
 #pragma unroll
-    for (int ks = 0; ks < C::kKSteps; ++ks) {
-      if (ks + 1 < C::kKSteps) {
-        sub_step(f[ks & 1], f[(ks + 1) & 1], kt, ks + 1, -1, dma_is_full_step);
+        for (int n = 0; n < kLoads; ++n) LoadToLds16(dst + n * 1024, goff[n], uint32_t(kbase), n < 8 ? a_rsrc : b_rsrc);
       } else {
-        WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
-        __syncthreads();
-        sub_step(f[ks & 1], f[0], kt + 1, 0, kt + C::kStages, dma_is_full_step);
+#pragma unroll
+        for (int n = 0; n < kLoads; ++n)
+          LoadToLds16(dst + n * 1024, kbase + gk[n] < K ? goff[n] + kbase : kOutOfRange, n < 8 ? a_rsrc : b_rsrc);
+      }
+    };
+    struct Frags4 {
+      v4i a[2];
+      v4i b[2];
+    };
+    auto read4 = [&](int slot, int ks, Frags4& f) {
+      const char* base = ring + slot * kSlotBytes;
+      const int off = LdsOffset<BK>(frag_row, ks * 2 + frag_half);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        f.a[i] = *reinterpret_cast<const v4i*>(base + off + i * 32 * kBK);
+        f.b[i] = *reinterpret_cast<const v4i*>(base + C::kBM * kBK + off + i * 32 * kBK);
+      }
+    };
+    typename Traits::Acc full[2][2], rows_sum[2], cols_sum[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        full[i][0][v] = 0;
+        full[i][1][v] = 0;
+        rows_sum[i][v] = 0;
+        cols_sum[i][v] = 0;
       }
     }
-  };
-  // While the step whose loads are being issued (kt + kStages) lies entirely
-  // inside the depth, the cheap form of the loads is used; the last few steps
-  // (a partial step and the ones past the end, which fetch zeros) take the
-  // bounds-tested form.
-  int kt = 0;
-  const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
-  for (; kt < full_end; ++kt) ring_step(kt, std::true_type());
-  for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type());
+    auto mma4 = [&](Frags4 f) {
+      if constexpr (kFlip) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          f.a[i] ^= static_cast<int>(args.a_flip);
+          f.b[i] ^= static_cast<int>(args.b_flip);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) Traits::Mma(f.a[i], f.b[j], full[i][j]);
+      if constexpr (kFusedSums) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          Traits::Mma(f.a[i], ones, rows_sum[i]);
+          Traits::Mma(ones, f.b[i], cols_sum[i]);
+        }
+      }
+    };
+    // This wave's steps: wave, wave + 4, ... of the workgroup's k_tiles steps.
+    const int my_steps = k_tiles > wave ? (k_tiles - wave + 3) / 4 : 0;
+    if (my_steps > 0) issue_step(wave, 0);
+    if (my_steps > 1) issue_step(wave + 4, 1);
+    Frags4 fr[2];
+    for (int i = 0; i < my_steps; ++i) {
+      if (i + 1 < my_steps)
+        WaitVmcnt<kLoads>();  // in-order completion: only the next step's loads may be outstanding
+      else
+        WaitVmcnt<0>();
+      const int slot = i & 1;
+      read4(slot, 0, fr[0]);
+#pragma unroll
+      for (int ks = 0; ks < C::kKSteps; ++ks) {
+        if (ks + 1 < C::kKSteps) read4(slot, ks + 1, fr[(ks + 1) & 1]);
+        mma4(fr[ks & 1]);
+      }
+      // Every LDS read of the slot has been consumed; refill it.
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      if (i + 2 < my_steps) issue_step(wave + 4 * (i + 2), slot);
+    }
+    if constexpr (kFusedSums) {
+      const uint32_t fa = static_cast<uint32_t>(args.fused_a_factor);
+      const uint32_t fb = static_cast<uint32_t>(args.fused_b_factor);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            full[i][j][v] = static_cast<int>(static_cast<uint32_t>(full[i][j][v]) -
+                                             fa * static_cast<uint32_t>(rows_sum[i][v]) -
+                                             fb * static_cast<uint32_t>(cols_sum[j][v]));
+    }
+    // Add the four partial tiles: [wave][block][quarter][lane] in LDS.
+    __syncthreads();  // every wave is done with its ring
+    v4i* parts = reinterpret_cast<v4i*>(lds);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          v4i w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = Traits::RawBits(full[i][j][4 * q + e]);
+          parts[((wave * 4 + i * 2 + j) * 4 + q) * 64 + lane] = w;
+        }
+    __syncthreads();
+    const int my_block = wave_m * 2 + wave_n;
+#pragma unroll
+    for (int w4 = 0; w4 < 4; ++w4)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4i w = parts[((w4 * 4 + my_block) * 4 + q) * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[0][0][4 * q + e] += Traits::FromRawBits(w[e]);
+      }
+  } else {
+#pragma unroll
+    for (int s = 0; s < C::kStages; ++s) issue(s);
+    WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
+    __syncthreads();
+    Frags f[2];
+    read_frags(0, 0, f[0]);
+    auto ring_step = [&](int kt, auto dma_is_full_step) {
+#pragma unroll
+      for (int ks = 0; ks < C::kKSteps; ++ks) {
+        if (ks + 1 < C::kKSteps) {
+          sub_step(f[ks & 1], f[(ks + 1) & 1], kt, ks + 1, -1, dma_is_full_step);
+        } else {
+          WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
+          __syncthreads();
+          sub_step(f[ks & 1], f[0], kt + 1, 0, kt + C::kStages, dma_is_full_step);
+        }
+      }
+    };
+    // While the step whose loads are being issued (kt + kStages) lies entirely
+    // inside the depth, the cheap form of the loads is used; the last few steps
+    // (a partial step and the ones past the end, which fetch zeros) take the
+    // bounds-tested form.
+    int kt = 0;
+    const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
+    for (; kt < full_end; ++kt) ring_step(kt, std::true_type());
+    for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type());
+  }
   WaitVmcnt<0>();
   __syncthreads();  // every wave is done with the operand ring
-  if constexpr (kFusedSums) {
+  if constexpr (kFusedSums && !kDepthWaves) {
     const uint32_t fa = static_cast<uint32_t>(args.fused_a_factor);
     const uint32_t fb = static_cast<uint32_t>(args.fused_b_factor);
     // Plane-split operand: the correction belongs to the low plane's block
@@ -627,7 +777,8 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   }
 }
 
-template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false>
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
+          bool kDepthWaves = false>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
@@ -635,7 +786,7 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int total = tiles_m * tiles_n;
   const int grid = ((total + 7) / 8) * 8;
   const size_t lds_bytes = C::kLdsBytes;
-  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip>;
+  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>;
   if (lds_bytes > 48 * 1024) {
     // Once per process; static initialisation is safe against concurrent callers.
     static const hipError_t attr = hipFuncSetAttribute(
@@ -782,17 +933,16 @@ inline TailPlan PlanTail(const GemmArgs& args, int num_cus, double gap_steps) {
 // smallest tile has it (64x64, or 64 rows x 128 plane columns for the
 // plane-split operand): adding up the parts costs time in proportion to the
 // tile's area, and with larger tiles that outweighed the gain at every shape
-// measured. One workgroup streams its operands at a rate that the CU's
-// outstanding-request capacity fixes (about 35 GB/s), whatever the depth of the
-// ring, so a problem with few tiles and a long depth only gets faster by
-// putting more workgroups on it. The split is taken when the tiles alone leave
-// CUs idle, aims at as many workgroups per CU as the ring's LDS lets run
-// together (two, one for the plane-split tile), and keeps at least
-// kMinStepsPerPart depth steps in every part so that filling the ring and
-// adding up the parts (about as long as one depth step per part) stay small
-// against the work shared out.
+// measured. One workgroup streams operands that are not in L2 at 80-100 GB/s
+// at best (what its ring keeps in flight over a round trip to memory), so a
+// problem with few tiles and a long depth only gets faster by putting more
+// workgroups on it. The split is taken when the tiles alone leave CUs idle,
+// aims at one workgroup per CU (the rings take most of a CU's LDS), and keeps
+// at least kMinStepsPerPart depth steps in every part (16 for the 64x64 tile:
+// four steps for each of its waves) so that filling the ring and adding up the
+// parts stay small against the work shared out.
 inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, bool split_b) {
-  constexpr int kMinStepsPerPart = 8;
+  const int kMinStepsPerPart = split_b ? 8 : 16;
   constexpr int kMaxParts = 32;
   const Tile tile = PickTile(args, num_cus, split_b);
   if (tile != (split_b ? Tile::k64x128 : Tile::k64x64)) return DepthSplit();
@@ -800,8 +950,7 @@ inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, bool split_b
   const int tiles = TileCount(args, bm, bn);
   const int k_tiles = (args.k_bytes + 127) / 128;
   if (tiles == 0 || tiles > kSplitCounters) return DepthSplit();
-  const int resident_per_cu = split_b ? 1 : 2;
-  int parts = std::min({resident_per_cu * num_cus / tiles, k_tiles / kMinStepsPerPart, kMaxParts});
+  int parts = std::min({num_cus / tiles, k_tiles / kMinStepsPerPart, kMaxParts});
   if (parts < 2) return DepthSplit();
   const int steps_per_part = (k_tiles + parts - 1) / parts;
   parts = (k_tiles + steps_per_part - 1) / steps_per_part;  // no empty part
@@ -809,6 +958,18 @@ inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, bool split_b
   split.parts = parts;
   split.partial_bytes = size_t(parts) * tiles * bm * bn * 4;
   return split;
+}
+
+// The 64x64 tile: the depth-per-wave schedule (its "8 stages" are the two
+// ring slots of each of the four waves), except for depths of at most three
+// steps per workgroup, which would leave waves without work: there the four
+// waves share every step (256^3 replayed from a graph: 5.3 against 5.6 us).
+template <typename Traits, bool kFusedSums = false, bool kFlip = false>
+hipError_t LaunchSmallestTile(hipStream_t stream, const GemmArgs& args) {
+  const int k_tiles = (args.k_bytes + 127) / 128;
+  const int parts = args.split_k > 1 ? args.split_k : 1;
+  if ((k_tiles + parts - 1) / parts <= 3) return Launch<Traits, 1, 1, 128, 4, kFusedSums, kFlip, false>(stream, args);
+  return Launch<Traits, 1, 1, 128, 8, kFusedSums, kFlip, true>(stream, args);
 }
 
 template <typename Traits>
@@ -832,7 +993,7 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile) {
       case Tile::k128x64:
         return Launch<Traits, 2, 1, 128, 4>(stream, args);
       default:
-        return Launch<Traits, 1, 1, 128, kSmallestTileStages>(stream, args);
+        return LaunchSmallestTile<Traits>(stream, args);
     }
   }
   return hipErrorInvalidValue;
