@@ -129,7 +129,7 @@ bool GemmI8I16CanFuseSums(const GemmArgs& args, int num_cus) {
 hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus) {
   if (args.fuse_sums) {
     if (!GemmI8I16CanFuseSums(args, num_cus)) return hipErrorInvalidValue;
-    return mfma_gemm::Launch<Int8SplitTraits, 1, 2, 128, 4, true>(stream, args);
+    return mfma_gemm::LaunchSmallestTile<Int8SplitTraits, true>(stream, args);
   }
   return mfma_gemm::LaunchBest<Int8SplitTraits>(stream, args, num_cus);
 }

@@ -165,8 +165,8 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
                 "fused sums exist for the tiles with one block (one block per plane) per wave only");
   static_assert(!kFlip || WM * WN == 1, "in-place uint8 operands exist for the single-block tile only");
-  static_assert(!kDepthWaves || (WM * WN == 1 && BK == 128 && STAGES == 8 && !Traits::kSplitB),
-                "the depth-per-wave schedule exists for the 64x64 tile, with two ring slots of 16 KiB per wave");
+  static_assert(!kDepthWaves || (WM == 1 && WN == (Traits::kSplitB ? 2 : 1) && BK == 128),
+                "the depth-per-wave schedule exists for the smallest tile of each kernel");
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
   constexpr int kBK = BK;
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -404,20 +404,27 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // also finished reading step kt, so its ring slot is free), issue the loads
   // of step kt+kStages into that slot, then read fragments (kt+1, 0).
   if constexpr (kDepthWaves) {
-    // ---- the 64x64 tile, one wave per part of the depth ----
+    // ---- the smallest tile, the depth dealt out to the waves ----
     // With one 32x32 block per wave a depth step is four dependent matrix
     // instructions and some eighty others around them (loads, LDS reads,
     // waits, a barrier), and a lone wave issues an instruction every four or
     // five cycles: the step takes a thousand cycles however deep the ring is.
-    // Here every wave computes the whole 64x64 tile (2 x 2 independent blocks)
-    // for every fourth depth step, through a two-slot ring of its own and
+    // Here every wave computes a whole 64x64 piece (2 x 2 independent blocks)
+    // for a share of the depth steps, through a two-slot ring of its own and
     // without any barrier: four times the matrix work per LDS read and per
-    // load, and nobody to wait for. The four partial tiles are added through
-    // LDS afterwards, which leaves wave (wave_m, wave_n) with its block as in
-    // the other schedule.
-    constexpr int kSlotBytes = C::kStageBytes;  // 64 A rows + 64 B rows, 128 bytes each
+    // load, and nobody to wait for. 64x64 tile: the piece is the tile and
+    // wave w takes steps w, w+4, ... Plane-split kernel (64 rows x 128 plane
+    // columns): wave (d, c) takes the 64 plane columns of half c at steps
+    // d, d+2, ... The partial pieces are added through LDS afterwards, which
+    // leaves wave (wave_m, wave_n) with its WM x WN blocks as in the other
+    // schedule.
+    constexpr int kColWays = Traits::kSplitB ? 2 : 1;
+    constexpr int kDepthWays = 4 / kColWays;
+    const int depth_way = wave / kColWays;
+    const int col_way = wave % kColWays;
+    constexpr int kSlotBytes = 128 * kBK;  // 64 A rows + 64 B rows, 128 bytes each
     constexpr int kLoads = kSlotBytes / 1024;
-    static_assert(kLoads == 16 && C::kBM == 64 && C::kBN == 64, "");
+    static_assert(kLoads == 16 && C::kBM == 64 && C::kBN == 64 * kColWays, "");
     char* ring = lds + wave * 2 * kSlotBytes;
     const uint32_t ring_base = lds_base + wave * 2 * kSlotBytes;
     // Load n of a step fills rows 8n .. 8n+7 of the slot (A rows first).
@@ -431,7 +438,9 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
       if (n < 8)
         goff[n] = m0 + r < args.M ? uint32_t(m0 + r) * uint32_t(args.lda) + g * kGranule : kOutOfRange;
       else
-        goff[n] = n0 + r < args.N ? uint32_t(n0 + r) * uint32_t(args.ldb) + g * kGranule : kOutOfRange;
+        goff[n] = n0 + col_way * 64 + r < args.N
+                      ? uint32_t(n0 + col_way * 64 + r) * uint32_t(args.ldb) + g * kGranule
+                      : kOutOfRange;
     }
     auto issue_step = [&](int step, int slot) {
       const int kbase = phys(step) * kBK;
@@ -455,7 +464,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         f.a[i] = *reinterpret_cast<const v4i*>(base + off + i * 32 * kBK);
-        f.b[i] = *reinterpret_cast<const v4i*>(base + C::kBM * kBK + off + i * 32 * kBK);
+        f.b[i] = *reinterpret_cast<const v4i*>(base + 64 * kBK + off + i * 32 * kBK);
       }
     };
     typename Traits::Acc full[2][2], rows_sum[2], cols_sum[2];
@@ -482,17 +491,19 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) Traits::Mma(f.a[i], f.b[j], full[i][j]);
       if constexpr (kFusedSums) {
+        // The plane-split operand has zero point 0 by definition, so its
+        // column sums are never needed.
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
           Traits::Mma(f.a[i], ones, rows_sum[i]);
-          Traits::Mma(ones, f.b[i], cols_sum[i]);
+          if constexpr (!Traits::kSplitB) Traits::Mma(ones, f.b[i], cols_sum[i]);
         }
       }
     };
-    // This wave's steps: wave, wave + 4, ... of the workgroup's k_tiles steps.
-    const int my_steps = k_tiles > wave ? (k_tiles - wave + 3) / 4 : 0;
-    if (my_steps > 0) issue_step(wave, 0);
-    if (my_steps > 1) issue_step(wave + 4, 1);
+    // This wave's steps: depth_way, depth_way + kDepthWays, ... of the workgroup's k_tiles steps.
+    const int my_steps = k_tiles > depth_way ? (k_tiles - depth_way + kDepthWays - 1) / kDepthWays : 0;
+    if (my_steps > 0) issue_step(depth_way, 0);
+    if (my_steps > 1) issue_step(depth_way + kDepthWays, 1);
     Frags4 fr[2];
     for (int i = 0; i < my_steps; ++i) {
       if (i + 1 < my_steps)
@@ -508,22 +519,24 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
       }
       // Every LDS read of the slot has been consumed; refill it.
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      if (i + 2 < my_steps) issue_step(wave + 4 * (i + 2), slot);
+      if (i + 2 < my_steps) issue_step(depth_way + kDepthWays * (i + 2), slot);
     }
     if constexpr (kFusedSums) {
       const uint32_t fa = static_cast<uint32_t>(args.fused_a_factor);
       const uint32_t fb = static_cast<uint32_t>(args.fused_b_factor);
+      // Plane-split operand: the correction belongs to the low plane's block
+      // (the odd one of a pair; the write-back combines 256 * high + low).
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = Traits::kSplitB ? 1 : 0; j < 2; ++j)
 #pragma unroll
           for (int v = 0; v < 16; ++v)
             full[i][j][v] = static_cast<int>(static_cast<uint32_t>(full[i][j][v]) -
                                              fa * static_cast<uint32_t>(rows_sum[i][v]) -
                                              fb * static_cast<uint32_t>(cols_sum[j][v]));
     }
-    // Add the four partial tiles: [wave][block][quarter][lane] in LDS.
+    // Add the partial pieces: [wave][block][quarter][lane] in LDS.
     __syncthreads();  // every wave is done with its ring
     v4i* parts = reinterpret_cast<v4i*>(lds);
 #pragma unroll
@@ -538,15 +551,22 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
           parts[((wave * 4 + i * 2 + j) * 4 + q) * 64 + lane] = w;
         }
     __syncthreads();
-    const int my_block = wave_m * 2 + wave_n;
+    // Wave (wave_m, wave_n) ends up with block row wave_m and, of the piece's
+    // two block columns, column wave_n (64x64 tile) or both (plane-split: the
+    // piece of column half wave_n).
 #pragma unroll
-    for (int w4 = 0; w4 < 4; ++w4)
+    for (int j = 0; j < WN; ++j) {
+      const int from_col_way = kColWays == 1 ? 0 : wave_n;
+      const int block = wave_m * 2 + (kColWays == 1 ? wave_n : j);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const v4i w = parts[((w4 * 4 + my_block) * 4 + q) * 64 + lane];
+      for (int d = 0; d < kDepthWays; ++d)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[0][0][4 * q + e] += Traits::FromRawBits(w[e]);
-      }
+        for (int q = 0; q < 4; ++q) {
+          const v4i w = parts[(((d * kColWays + from_col_way) * 4 + block) * 4 + q) * 64 + lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[0][j][4 * q + e] += Traits::FromRawBits(w[e]);
+        }
+    }
   } else {
 #pragma unroll
     for (int s = 0; s < C::kStages; ++s) issue(s);
@@ -785,7 +805,8 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int tiles_n = (args.N + C::kBN - 1) / C::kBN;
   const int total = tiles_m * tiles_n;
   const int grid = ((total + 7) / 8) * 8;
-  const size_t lds_bytes = C::kLdsBytes;
+  // The depth-per-wave schedule: two ring slots of 16 KiB for each of four waves.
+  const size_t lds_bytes = kDepthWaves ? size_t(4 * 2 * 128 * BK) : size_t(C::kLdsBytes);
   auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>;
   if (lds_bytes > 48 * 1024) {
     // Once per process; static initialisation is safe against concurrent callers.
@@ -960,16 +981,19 @@ inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, bool split_b
   return split;
 }
 
-// The 64x64 tile: the depth-per-wave schedule (its "8 stages" are the two
-// ring slots of each of the four waves), except for depths of at most three
-// steps per workgroup, which would leave waves without work: there the four
-// waves share every step (256^3 replayed from a graph: 5.3 against 5.6 us).
+// The smallest tile of a kernel (64x64; 64 rows x 128 plane columns for the
+// plane-split operand): the depth-per-wave schedule, except for depths so
+// short that waves would be left without a step: there the four waves share
+// every step (256^3 replayed from a graph: 5.3 against 5.6 us).
 template <typename Traits, bool kFusedSums = false, bool kFlip = false>
 hipError_t LaunchSmallestTile(hipStream_t stream, const GemmArgs& args) {
+  constexpr int kWN = Traits::kSplitB ? 2 : 1;
+  constexpr int kDepthWays = 4 / kWN;
   const int k_tiles = (args.k_bytes + 127) / 128;
   const int parts = args.split_k > 1 ? args.split_k : 1;
-  if ((k_tiles + parts - 1) / parts <= 3) return Launch<Traits, 1, 1, 128, 4, kFusedSums, kFlip, false>(stream, args);
-  return Launch<Traits, 1, 1, 128, 8, kFusedSums, kFlip, true>(stream, args);
+  if ((k_tiles + parts - 1) / parts < kDepthWays)
+    return Launch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, false>(stream, args);
+  return Launch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, true>(stream, args);
 }
 
 template <typename Traits>
@@ -980,6 +1004,7 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile) {
     case Tile::k128x128:
       return Launch<Traits, 2, 2, 128, 4>(stream, args);
     case Tile::k64x128:
+      if constexpr (Traits::kSplitB) return LaunchSmallestTile<Traits>(stream, args);
       return Launch<Traits, 1, 2, 128, 4>(stream, args);
     default:
       break;
