@@ -841,29 +841,48 @@ enum class Tile { k256x256, k256x128, k128x256, k128x128, k128x64, k64x128, k64x
 // rate). Large tiles win when there are many rounds, small tiles when the last
 // (or only) round would leave most CUs idle. `split_b`: the plane-split form
 // of the int16 kernel, which has the two square large tiles and a 64x128 one.
+//
+// The 128x128, 128x64 and 64x128 tiles come with two ring depths. Four stages
+// when every tile has a CU to itself (a lone workgroup needs the deep prefetch:
+// 1280x1280 with K = 4096 runs in 24 us on 128x64 with four stages, 28 us with
+// two). Two stages when there are more tiles than CUs: two (three) workgroups
+// then fit a CU's LDS together, and a second wave on each SIMD fills the issue
+// slots and barrier waits of the first (4096x4096 with K = 2048 on 128x128:
+// 81 -> 58 us; 2560^3: 45 -> 34 us). The cost model knows the case of up to
+// two tiles per CU, where both run side by side as one shared round with a
+// measured efficiency of 0.85 (128x128) and 0.65 (128x64, 64x128); with more
+// tiles than that the large tiles win anyway and the rounds are counted as
+// before.
 constexpr double kEffHalf = 0.55;
 struct TileChoice {
   Tile tile;
   double cost;  // rounds x tile area / efficiency
 };
+inline bool ShallowRing(const GemmArgs& args, int num_cus, int bm, int bn) {
+  return TileCount(args, bm, bn) > num_cus;
+}
 inline TileChoice BestTile(const GemmArgs& args, int num_cus, bool split_b) {
-  auto cost = [&](int bm, int bn, double efficiency) {
-    const int rounds = (TileCount(args, bm, bn) + num_cus - 1) / num_cus;
+  auto cost = [&](int bm, int bn, double efficiency, double efficiency_shared = 0) {
+    const int tiles = TileCount(args, bm, bn);
+    if (efficiency_shared > 0 && tiles > num_cus && tiles <= 2 * num_cus)
+      return 2 * double(bm) * double(bn) / efficiency_shared;
+    const int rounds = (tiles + num_cus - 1) / num_cus;
     return rounds * double(bm) * double(bn) / efficiency;
   };
   const double c256 = cost(256, 256, 1.0);
-  const double c128 = cost(128, 128, 0.65);
   if (split_b) {
     // Plane-split operand: the smallest tile is 64 rows x 128 plane columns (64 destination columns).
+    const double c128 = cost(128, 128, 0.65);
     const double c64x128 = cost(64, 128, 0.5);
     if (c256 <= c128 && c256 <= c64x128) return {Tile::k256x256, c256};
     return c128 <= c64x128 ? TileChoice{Tile::k128x128, c128} : TileChoice{Tile::k64x128, c64x128};
   }
+  const double c128 = cost(128, 128, 0.65, 0.85);
   const double c64 = cost(64, 64, 0.45);
   const double c256x128 = cost(256, 128, 0.75);
   const double c128x256 = cost(128, 256, 0.75);
-  const double c128x64 = cost(128, 64, kEffHalf);
-  const double c64x128 = cost(64, 128, kEffHalf);
+  const double c128x64 = cost(128, 64, kEffHalf, 0.65);
+  const double c64x128 = cost(64, 128, kEffHalf, 0.65);
   const double best = std::min({c256, c128, c64, c256x128, c128x256, c128x64, c64x128});
   if (c256 == best) return {Tile::k256x256, best};
   if (c256x128 == best) return {Tile::k256x128, best};
@@ -997,14 +1016,16 @@ hipError_t LaunchSmallestTile(hipStream_t stream, const GemmArgs& args) {
 }
 
 template <typename Traits>
-hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile) {
+hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int num_cus) {
   switch (tile) {
     case Tile::k256x256:
       return Launch<Traits, 4, 4, 128, 2>(stream, args);
     case Tile::k128x128:
+      if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128)) return Launch<Traits, 2, 2, 128, 2>(stream, args);
       return Launch<Traits, 2, 2, 128, 4>(stream, args);
     case Tile::k64x128:
       if constexpr (Traits::kSplitB) return LaunchSmallestTile<Traits>(stream, args);
+      if (ShallowRing(args, num_cus, 64, 128)) return Launch<Traits, 1, 2, 128, 2>(stream, args);
       return Launch<Traits, 1, 2, 128, 4>(stream, args);
     default:
       break;
@@ -1016,6 +1037,7 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile) {
       case Tile::k128x256:
         return Launch<Traits, 2, 4, 128, 3>(stream, args);
       case Tile::k128x64:
+        if (ShallowRing(args, num_cus, 128, 64)) return Launch<Traits, 2, 1, 128, 2>(stream, args);
         return Launch<Traits, 2, 1, 128, 4>(stream, args);
       default:
         return LaunchSmallestTile<Traits>(stream, args);
@@ -1037,11 +1059,11 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
                                            : SubProblem(args, cut, args.M - cut, 0, args.N);
         const hipError_t first = Launch<Traits, 4, 4, 128, 2>(stream, main);
         if (first != hipSuccess) return first;
-        return LaunchTile<Traits>(stream, tail, PickTile(tail, num_cus, false));
+        return LaunchTile<Traits>(stream, tail, PickTile(tail, num_cus, false), num_cus);
       }
     }
   }
-  return LaunchTile<Traits>(stream, args, tile);
+  return LaunchTile<Traits>(stream, args, tile, num_cus);
 }
 
 }  // namespace mfma_gemm
