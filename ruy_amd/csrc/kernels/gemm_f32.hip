@@ -24,6 +24,7 @@ struct F32Traits {
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[e]), __int_as_float(b[e]), acc, 0, 0, 0);
   }
   static constexpr bool kSplitB = false;
+  static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kF32;
   // Time between two dependent launches (about 5 us) in depth steps of the
   // 256x256 tile (32 floats deep, 7.8 us each).
   static constexpr double kLaunchGapInDepthSteps = 0.65;

@@ -25,6 +25,7 @@ struct Int8Traits {
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
   }
   static constexpr bool kSplitB = false;
+  static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kInt8;
   // Time between two dependent launches (about 5 us) in depth steps of the
   // 256x256 tile (1.9 us each on int8).
   static constexpr double kLaunchGapInDepthSteps = 2.6;
@@ -115,6 +116,7 @@ struct Int8Traits {
 // which the dispatcher sets. Everything is exact modulo 2^32.
 struct Int8SplitTraits : Int8Traits {
   static constexpr bool kSplitB = true;
+  static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kInt8PlaneSplit;
   static __device__ __forceinline__ int Bits(int hi, int lo) {
     return static_cast<int>(static_cast<uint32_t>(hi) * 256u + static_cast<uint32_t>(lo));
   }
@@ -123,7 +125,7 @@ struct Int8SplitTraits : Int8Traits {
 }  // namespace
 
 bool GemmI8I16CanFuseSums(const GemmArgs& args, int num_cus) {
-  return mfma_gemm::PickTile(args, num_cus, true) == mfma_gemm::Tile::k64x128;
+  return mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8PlaneSplit) == mfma_gemm::Tile::k64x128;
 }
 
 hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus) {
@@ -135,13 +137,16 @@ hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus
 }
 
 DepthSplit GemmDepthSplit(const GemmArgs& args, int num_cus, GemmKind kind) {
-  return mfma_gemm::PlanDepthSplit(args, num_cus, kind == GemmKind::kInt8Int16);
+  const mfma_gemm::Model model = kind == GemmKind::kInt8Int16 ? mfma_gemm::Model::kInt8PlaneSplit
+                                 : kind == GemmKind::kF32     ? mfma_gemm::Model::kF32
+                                                              : mfma_gemm::Model::kInt8;
+  return mfma_gemm::PlanDepthSplit(args, num_cus, model);
 }
 
 int GemmDepthSplitCounters() { return mfma_gemm::kSplitCounters; }
 
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
-  return mfma_gemm::PickTile(args, num_cus, false) == mfma_gemm::Tile::k64x64;
+  return mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k64x64;
 }
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {

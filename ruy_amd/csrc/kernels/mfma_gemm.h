@@ -839,7 +839,7 @@ enum class Tile { k256x256, k256x128, k128x256, k128x128, k128x64, k64x128, k64x
 // 128x128 tile about 0.65 and the 64x64 tile, whose waves read one LDS
 // fragment pair per matrix instruction, about 0.45 of the 256x256 tile's
 // rate). Large tiles win when there are many rounds, small tiles when the last
-// (or only) round would leave most CUs idle. `split_b`: the plane-split form
+// (or only) round would leave most CUs idle. Model::kInt8PlaneSplit: the plane-split form
 // of the int16 kernel, which has the two square large tiles and a 64x128 one.
 //
 // The 128x128, 128x64 and 64x128 tiles come with two ring depths. Four stages
@@ -853,7 +853,20 @@ enum class Tile { k256x256, k256x128, k128x256, k128x128, k128x64, k64x128, k64x
 // measured efficiency of 0.85 (128x128) and 0.65 (128x64, 64x128); with more
 // tiles than that the large tiles win anyway and the rounds are counted as
 // before.
-constexpr double kEffHalf = 0.55;
+//
+// fp32 is bound by its matrix instructions at every tile size (64 cycles of
+// matrix pipe per 32 bytes of fragment pair, eight times the int8 ratio), so
+// the small tiles lose little there and filling the CUs evenly matters more:
+// measured against the 256x256 tile, 256x128, 128x128 and 128x64 sustain
+// about 0.85 (0.9 in a shared round) and 64x64 0.75, which moves e.g.
+// 3072^3 from 256x256 (144 tiles, 723 us) to 128x64 (556 us) and 1536^3 from
+// 128x128 to 64x64 (114 -> 97 us).
+enum class Model { kInt8, kInt8PlaneSplit, kF32 };
+struct Efficiencies {
+  double t256x128, t128x128, t128x128_shared, t128x64, t128x64_shared, t64x64;
+};
+constexpr Efficiencies kInt8Efficiencies = {0.75, 0.65, 0.85, 0.55, 0.65, 0.45};
+constexpr Efficiencies kF32Efficiencies = {0.85, 0.85, 0.9, 0.85, 0.9, 0.75};
 struct TileChoice {
   Tile tile;
   double cost;  // rounds x tile area / efficiency
@@ -861,7 +874,9 @@ struct TileChoice {
 inline bool ShallowRing(const GemmArgs& args, int num_cus, int bm, int bn) {
   return TileCount(args, bm, bn) > num_cus;
 }
-inline TileChoice BestTile(const GemmArgs& args, int num_cus, bool split_b) {
+inline TileChoice BestTile(const GemmArgs& args, int num_cus, Model model) {
+  const bool split_b = model == Model::kInt8PlaneSplit;
+  const Efficiencies& eff = model == Model::kF32 ? kF32Efficiencies : kInt8Efficiencies;
   auto cost = [&](int bm, int bn, double efficiency, double efficiency_shared = 0) {
     const int tiles = TileCount(args, bm, bn);
     if (efficiency_shared > 0 && tiles > num_cus && tiles <= 2 * num_cus)
@@ -877,12 +892,12 @@ inline TileChoice BestTile(const GemmArgs& args, int num_cus, bool split_b) {
     if (c256 <= c128 && c256 <= c64x128) return {Tile::k256x256, c256};
     return c128 <= c64x128 ? TileChoice{Tile::k128x128, c128} : TileChoice{Tile::k64x128, c64x128};
   }
-  const double c128 = cost(128, 128, 0.65, 0.85);
-  const double c64 = cost(64, 64, 0.45);
-  const double c256x128 = cost(256, 128, 0.75);
-  const double c128x256 = cost(128, 256, 0.75);
-  const double c128x64 = cost(128, 64, kEffHalf, 0.65);
-  const double c64x128 = cost(64, 128, kEffHalf, 0.65);
+  const double c128 = cost(128, 128, eff.t128x128, eff.t128x128_shared);
+  const double c64 = cost(64, 64, eff.t64x64);
+  const double c256x128 = cost(256, 128, eff.t256x128);
+  const double c128x256 = cost(128, 256, eff.t256x128);
+  const double c128x64 = cost(128, 64, eff.t128x64, eff.t128x64_shared);
+  const double c64x128 = cost(64, 128, eff.t128x64, eff.t128x64_shared);
   const double best = std::min({c256, c128, c64, c256x128, c128x256, c128x64, c64x128});
   if (c256 == best) return {Tile::k256x256, best};
   if (c256x128 == best) return {Tile::k256x128, best};
@@ -892,8 +907,8 @@ inline TileChoice BestTile(const GemmArgs& args, int num_cus, bool split_b) {
   if (c64x128 == best) return {Tile::k64x128, best};
   return {Tile::k64x64, best};
 }
-inline Tile PickTile(const GemmArgs& args, int num_cus, bool split_b) {
-  return BestTile(args, num_cus, split_b).tile;
+inline Tile PickTile(const GemmArgs& args, int num_cus, Model model) {
+  return BestTile(args, num_cus, model).tile;
 }
 
 // The sub-problem of `args` whose destination is rows [m_begin, m_begin +
@@ -940,7 +955,7 @@ struct TailPlan {
   bool along_n = false;  // the cut runs between tile columns (else between tile rows)
   int main_tiles = 0;    // tile columns (rows) in the first launch
 };
-inline TailPlan PlanTail(const GemmArgs& args, int num_cus, double gap_steps) {
+inline TailPlan PlanTail(const GemmArgs& args, int num_cus, double gap_steps, Model model) {
   TailPlan plan;
   const int tiles_m = (args.M + 255) / 256, tiles_n = (args.N + 255) / 256;
   const int total = tiles_m * tiles_n;
@@ -957,7 +972,7 @@ inline TailPlan PlanTail(const GemmArgs& args, int num_cus, double gap_steps) {
       const int main_rounds = (across * c + num_cus - 1) / num_cus;
       GemmArgs tail = args;
       (along_n ? tail.N : tail.M) -= c * 256;
-      const double cost = main_rounds * round_cost + BestTile(tail, num_cus, false).cost + gap;
+      const double cost = main_rounds * round_cost + BestTile(tail, num_cus, model).cost + gap;
       if (cost < best) {
         best = cost;
         plan.use = true;
@@ -981,10 +996,11 @@ inline TailPlan PlanTail(const GemmArgs& args, int num_cus, double gap_steps) {
 // at least kMinStepsPerPart depth steps in every part (16 for the 64x64 tile:
 // four steps for each of its waves) so that filling the ring and adding up the
 // parts stay small against the work shared out.
-inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, bool split_b) {
+inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, Model model) {
+  const bool split_b = model == Model::kInt8PlaneSplit;
   const int kMinStepsPerPart = split_b ? 8 : 16;
   constexpr int kMaxParts = 32;
-  const Tile tile = PickTile(args, num_cus, split_b);
+  const Tile tile = PickTile(args, num_cus, model);
   if (tile != (split_b ? Tile::k64x128 : Tile::k64x64)) return DepthSplit();
   const int bm = 64, bn = split_b ? 128 : 64;
   const int tiles = TileCount(args, bm, bn);
@@ -1048,10 +1064,10 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
 
 template <typename Traits>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
-  const Tile tile = PickTile(args, num_cus, Traits::kSplitB);
+  const Tile tile = PickTile(args, num_cus, Traits::kModel);
   if constexpr (!Traits::kSplitB) {
     if (tile == Tile::k256x256 && args.split_k == 1 && !args.fuse_sums) {
-      const TailPlan plan = PlanTail(args, num_cus, Traits::kLaunchGapInDepthSteps);
+      const TailPlan plan = PlanTail(args, num_cus, Traits::kLaunchGapInDepthSteps, Traits::kModel);
       if (plan.use) {
         const int cut = plan.main_tiles * 256;
         const GemmArgs main = plan.along_n ? SubProblem(args, 0, args.M, 0, cut) : SubProblem(args, 0, cut, 0, args.N);
@@ -1059,7 +1075,7 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
                                            : SubProblem(args, cut, args.M - cut, 0, args.N);
         const hipError_t first = Launch<Traits, 4, 4, 128, 2>(stream, main);
         if (first != hipSuccess) return first;
-        return LaunchTile<Traits>(stream, tail, PickTile(tail, num_cus, false), num_cus);
+        return LaunchTile<Traits>(stream, tail, PickTile(tail, num_cus, Traits::kModel), num_cus);
       }
     }
   }
