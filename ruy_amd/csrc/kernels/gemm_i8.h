@@ -168,6 +168,13 @@ hipError_t LaunchPackI16Split(hipStream_t stream, const PackSource& src, int8_t*
 // fp32 counterpart: vector c as floats at dst + c*ld (ld in elements, a
 // multiple of 4), zero-filled from K up to ld. `src.dtype` is fp32.
 hipError_t LaunchPackF32(hipStream_t stream, const PackSource& src, float* dst, int32_t ld);
+// Both operands of a small multiplication packed by one launch (same results
+// as two LaunchPackI8 / LaunchPackF32 calls).
+hipError_t LaunchPackI8Pair(hipStream_t stream, const PackSource& src_a, int8_t* dst_a, int32_t ld_a,
+                            int32_t* sums_a, const PackSource& src_b, int8_t* dst_b, int32_t ld_b,
+                            int32_t* sums_b);
+hipError_t LaunchPackF32Pair(hipStream_t stream, const PackSource& src_a, float* dst_a, int32_t ld_a,
+                             const PackSource& src_b, float* dst_b, int32_t ld_b);
 
 // dst(i, j) = src(i, j): same shape and element size, any two storage orders
 // (strides in elements).

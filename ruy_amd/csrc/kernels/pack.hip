@@ -35,12 +35,12 @@ __global__ void ZeroI32Kernel(int32_t* p, int n) {
 // Block = 256 threads = one 64-vector x (k_span) slab, walked 64 depth bytes at
 // a time through LDS so that both the read (along the source's contiguous
 // dimension) and the write (along depth) are coalesced.
-__global__ __launch_bounds__(256) void PackI8Kernel(PackSource src, int8_t* dst, int32_t ld,
-                                                   int32_t* sums, int k_span) {
-  __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kPitch];
+// (`bx`, `by` of `ny`: which slab of vectors and which depth span.)
+__device__ __forceinline__ void PackI8Block(const PackSource& src, int8_t* dst, int32_t ld, int32_t* sums,
+                                            int k_span, int bx, int by, int ny, uint8_t* tile) {
   const int tid = threadIdx.x;
-  const int c0 = blockIdx.x * kTileC;
-  const int k_begin = blockIdx.y * k_span;
+  const int c0 = bx * kTileC;
+  const int k_begin = by * k_span;
   const int k_end = min(k_begin + k_span, ld);  // includes the zero-filled padding
   const uint8_t* s = static_cast<const uint8_t*>(src.data);
   const uint32_t flip = src.dtype == RUYAMD_DTYPE_U8 ? 0x80808080u : 0u;
@@ -101,13 +101,20 @@ __global__ __launch_bounds__(256) void PackI8Kernel(PackSource src, int8_t* dst,
     sum += __shfl_xor(sum, 2, 64);
     const int c = c0 + wc;
     if (wg == 0 && c < src.count) {
-      if (gridDim.y == 1)
+      if (ny == 1)
         sums[c] = sum;
       else
         atomicAdd(&sums[c], sum);
     }
   }
 }
+
+__global__ __launch_bounds__(256) void PackI8Kernel(PackSource src, int8_t* dst, int32_t ld,
+                                                   int32_t* sums, int k_span) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kPitch];
+  PackI8Block(src, dst, ld, sums, k_span, blockIdx.x, blockIdx.y, gridDim.y, tile);
+}
+
 
 // Depth-contiguous source (any alignment, any depth): one wave per vector (or
 // per part of a vector when there are few vectors) streams it 1024 bytes at a
@@ -116,15 +123,15 @@ __global__ __launch_bounds__(256) void PackI8Kernel(PackSource src, int8_t* dst,
 // v_alignbyte_b32, so no byte loads are needed for unaligned rows. A dword
 // may reach up to three bytes before or past the row, always inside an
 // aligned dword that also holds a byte of the row.
-__global__ __launch_bounds__(256) void PackI8RowsKernel(PackSource src, int8_t* dst, int32_t ld,
-                                                       int32_t* sums, int k_span) {
+__device__ __forceinline__ void PackI8RowsBlock(const PackSource& src, int8_t* dst, int32_t ld, int32_t* sums,
+                                                int k_span, int bx, int by, int ny) {
   const int lane = threadIdx.x & 63;
-  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int c = bx * 4 + (threadIdx.x >> 6);
   if (c >= src.count) return;
   const uint8_t* row = static_cast<const uint8_t*>(src.data) + int64_t(c) * src.stride_c;
   const uint32_t flip = src.dtype == RUYAMD_DTYPE_U8 ? 0x80808080u : 0u;
   const int K = src.K;
-  const int k_begin = blockIdx.y * k_span;
+  const int k_begin = by * k_span;
   const int k_end = min(k_begin + k_span, ld);
   int8_t* out_row = dst + int64_t(c) * ld;
   int32_t sum = 0;
@@ -155,11 +162,41 @@ __global__ __launch_bounds__(256) void PackI8RowsKernel(PackSource src, int8_t* 
   if (sums) {
     const int32_t total = WaveSum(sum);
     if (lane == 0) {
-      if (gridDim.y == 1)
+      if (ny == 1)
         sums[c] = total;
       else
         atomicAdd(&sums[c], total);
     }
+  }
+}
+
+__global__ __launch_bounds__(256) void PackI8RowsKernel(PackSource src, int8_t* dst, int32_t ld,
+                                                       int32_t* sums, int k_span) {
+  PackI8RowsBlock(src, dst, ld, sums, k_span, blockIdx.x, blockIdx.y, gridDim.y);
+}
+
+// Both operands of a small multiplication in one launch (blockIdx.z says which
+// one): the second launch would cost more than the packing itself. Each side
+// is packed over its whole depth by the depth-contiguous scheme above or by
+// the generic one.
+struct PackPairI8 {
+  PackSource src[2];
+  int8_t* dst[2];
+  int32_t ld[2];
+  int32_t* sums[2];
+};
+__global__ __launch_bounds__(256) void PackI8PairKernel(PackPairI8 pair) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[kTileC * kPitch];
+  const int side = blockIdx.z;
+  const PackSource& src = pair.src[side];
+  if (src.stride_k == 1) {
+    if (static_cast<int>(blockIdx.x) * 4 >= src.count) return;
+    const int whole_depth = (pair.ld[side] + 1023) / 1024 * 1024;
+    PackI8RowsBlock(src, pair.dst[side], pair.ld[side], pair.sums[side], whole_depth, blockIdx.x, 0, 1);
+  } else {
+    if (static_cast<int>(blockIdx.x) * kTileC >= src.count) return;
+    const int whole_depth = (pair.ld[side] + kTileK - 1) / kTileK * kTileK;
+    PackI8Block(src, pair.dst[side], pair.ld[side], pair.sums[side], whole_depth, blockIdx.x, 0, 1, tile);
   }
 }
 
@@ -271,14 +308,14 @@ __global__ __launch_bounds__(256) void SumsI8Kernel(const int8_t* data, int32_t 
 // reads follow the source's contiguous dimension and writes follow depth.
 // There are no sums and no conversion for floating point
 // (ruy/pack_common.h:100-133).
-__global__ __launch_bounds__(256) void PackF32Kernel(PackSource src, float* dst, int32_t ld) {
-  __shared__ float tile[32][33];
+__device__ __forceinline__ void PackF32Block(const PackSource& src, float* dst, int32_t ld, int bx, int by,
+                                             int ny, float (*tile)[33]) {
   const int tx = threadIdx.x & 31;
   const int ty = threadIdx.x >> 5;  // 0..7
-  const int c0 = blockIdx.x * 32;
+  const int c0 = bx * 32;
   const float* s = static_cast<const float*>(src.data);
   const bool depth_contiguous = src.stride_k == 1;
-  for (int k0 = blockIdx.y * 32; k0 < ld; k0 += gridDim.y * 32) {
+  for (int k0 = by * 32; k0 < ld; k0 += ny * 32) {
 #pragma unroll
     for (int t = ty; t < 32; t += 8) {
       // (c, k) read so that tx runs along the contiguous source dimension
@@ -300,6 +337,23 @@ __global__ __launch_bounds__(256) void PackF32Kernel(PackSource src, float* dst,
     }
     __syncthreads();
   }
+}
+
+__global__ __launch_bounds__(256) void PackF32Kernel(PackSource src, float* dst, int32_t ld) {
+  __shared__ float tile[32][33];
+  PackF32Block(src, dst, ld, blockIdx.x, blockIdx.y, gridDim.y, tile);
+}
+
+struct PackPairF32 {
+  PackSource src[2];
+  float* dst[2];
+  int32_t ld[2];
+};
+__global__ __launch_bounds__(256) void PackF32PairKernel(PackPairF32 pair) {
+  __shared__ float tile[32][33];
+  const int side = blockIdx.z;
+  if (static_cast<int>(blockIdx.x) * 32 >= pair.src[side].count) return;
+  PackF32Block(pair.src[side], pair.dst[side], pair.ld[side], blockIdx.x, blockIdx.y, gridDim.y, tile);
 }
 
 // int16 -> two int8 planes. Block = 32 vectors (one group) x a depth span; the
@@ -503,6 +557,44 @@ hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, 
     hipLaunchKernelGGL(PackI8Kernel, dim3(blocks_c, k_split), dim3(256), 0, stream, src, dst, ld, sums,
                        k_span);
   }
+  return hipGetLastError();
+}
+
+hipError_t LaunchPackI8Pair(hipStream_t stream, const PackSource& src_a, int8_t* dst_a, int32_t ld_a,
+                            int32_t* sums_a, const PackSource& src_b, int8_t* dst_b, int32_t ld_b,
+                            int32_t* sums_b) {
+  PackPairI8 pair;
+  pair.src[0] = src_a;
+  pair.src[1] = src_b;
+  pair.dst[0] = dst_a;
+  pair.dst[1] = dst_b;
+  pair.ld[0] = ld_a;
+  pair.ld[1] = ld_b;
+  pair.sums[0] = sums_a;
+  pair.sums[1] = sums_b;
+  auto blocks_of = [](const PackSource& src) {
+    return src.stride_k == 1 ? (src.count + 3) / 4 : (src.count + kTileC - 1) / kTileC;
+  };
+  const int blocks = std::max(blocks_of(src_a), blocks_of(src_b));
+  if (blocks == 0) return hipSuccess;
+  hipLaunchKernelGGL(PackI8PairKernel, dim3(blocks, 1, 2), dim3(256), 0, stream, pair);
+  return hipGetLastError();
+}
+
+hipError_t LaunchPackF32Pair(hipStream_t stream, const PackSource& src_a, float* dst_a, int32_t ld_a,
+                             const PackSource& src_b, float* dst_b, int32_t ld_b) {
+  PackPairF32 pair;
+  pair.src[0] = src_a;
+  pair.src[1] = src_b;
+  pair.dst[0] = dst_a;
+  pair.dst[1] = dst_b;
+  pair.ld[0] = ld_a;
+  pair.ld[1] = ld_b;
+  const int blocks_c = (std::max(src_a.count, src_b.count) + 31) / 32;
+  if (blocks_c == 0) return hipSuccess;
+  int blocks_k = (std::max(ld_a, ld_b) + 31) / 32;
+  if (blocks_k > 16) blocks_k = 16;
+  hipLaunchKernelGGL(PackF32PairKernel, dim3(blocks_c, blocks_k, 2), dim3(256), 0, stream, pair);
   return hipGetLastError();
 }
 

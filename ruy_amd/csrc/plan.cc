@@ -78,13 +78,44 @@ const char kCaptureCacheMiss[] =
     "the stream is capturing and an operand with a cache policy is not in the prepacked cache yet: "
     "run the same call once before the capture";
 
-// Prepares one side: from the cache, in place, or packed into the workspace.
+// A pack into the workspace that has been set up but not launched yet: when
+// both sides of a small multiplication need one, a single launch does both.
+struct PendingPack8 {
+  bool pending = false;
+  PackSource src;
+  int8_t* dst = nullptr;
+  int32_t ld = 0;
+  int32_t* sums = nullptr;
+  uint64_t bytes = 0;
+};
+// Packed operands up to this size are worth pairing (the launch saved costs
+// more than the slower generic pack kernel loses on them).
+constexpr uint64_t kPairedPackLimit = 256 * 1024;
+
+int LaunchPendingPacks8(ruyamd_ctx* ctx, PendingPack8* a, PendingPack8* b, std::string* err) {
+  hipError_t status = hipSuccess;
+  if (a->pending && b->pending && a->bytes <= kPairedPackLimit && b->bytes <= kPairedPackLimit) {
+    status = LaunchPackI8Pair(ctx->stream, a->src, a->dst, a->ld, a->sums, b->src, b->dst, b->ld, b->sums);
+  } else {
+    if (a->pending) status = LaunchPackI8(ctx->stream, a->src, a->dst, a->ld, a->sums);
+    if (status == hipSuccess && b->pending) status = LaunchPackI8(ctx->stream, b->src, b->dst, b->ld, b->sums);
+  }
+  a->pending = b->pending = false;
+  if (status != hipSuccess) {
+    *err = "pack kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  return RUYAMD_OK;
+}
+
+// Prepares one side: from the cache, in place, or packed into the workspace
+// (with `defer`, that pack is only set up, for LaunchPendingPacks8).
 // `src` views the side as `count` depth vectors (LHS rows / RHS columns).
 // `u8_depth_step`: uint8 data may be used in place (the kernel flips the top
 // bit of every byte) if the depth is a multiple of this; 0 = never.
 int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point, bool need_sums,
                     int cache_policy, const void* src_key, int other_width, int u8_depth_step,
-                    Operand8* out, std::string* err) {
+                    Operand8* out, std::string* err, PendingPack8* defer = nullptr) {
   // View of the side as `count` depth vectors; its data pointer is only valid
   // on the device after EnsureOnDevice.
   auto view = [&]() {
@@ -164,7 +195,14 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
     *err = "workspace allocation failed";
     return RUYAMD_E_HIP;
   }
-  if (LaunchPackI8(ctx->stream, src, packed, ld, sums) != hipSuccess) {
+  if (defer) {
+    defer->pending = true;
+    defer->src = src;
+    defer->dst = packed;
+    defer->ld = ld;
+    defer->sums = sums;
+    defer->bytes = packed_bytes;
+  } else if (LaunchPackI8(ctx->stream, src, packed, ld, sums) != hipSuccess) {
     *err = "pack kernel launch failed";
     return RUYAMD_E_HIP;
   }
@@ -211,12 +249,14 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   }
   // Row sums of one side are needed iff the other side's zero point is not 0
   // (ruy/kernel.h:219-232).
+  PendingPack8 pack_a, pack_b;
   if (int rc = PrepareOperand8(ctx, call, 0, lhs.zero_point, rzp != 0, call->lhs_cache_policy,
-                               call->lhs_src_key, N, u8_depth_step, &a, err))
+                               call->lhs_src_key, N, u8_depth_step, &a, err, &pack_a))
     return rc;
   if (int rc = PrepareOperand8(ctx, call, 1, rhs.zero_point, lzp != 0, call->rhs_cache_policy,
-                               call->rhs_src_key, M, u8_depth_step, &b, err))
+                               call->rhs_src_key, M, u8_depth_step, &b, err, &pack_b))
     return rc;
+  if (int rc = LaunchPendingPacks8(ctx, &pack_a, &pack_b, err)) return rc;
   const int32_t zp_product_depth =
       static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
   if (skinny) {
@@ -321,8 +361,33 @@ struct OperandF32 {
   uint32_t bytes = 0;
 };
 
+struct PendingPackF32 {
+  bool pending = false;
+  PackSource src;
+  float* dst = nullptr;
+  int32_t ld = 0;
+  uint64_t bytes = 0;
+};
+
+int LaunchPendingPacksF32(ruyamd_ctx* ctx, PendingPackF32* a, PendingPackF32* b, std::string* err) {
+  hipError_t status = hipSuccess;
+  if (a->pending && b->pending && a->bytes <= kPairedPackLimit && b->bytes <= kPairedPackLimit) {
+    status = LaunchPackF32Pair(ctx->stream, a->src, a->dst, a->ld, b->src, b->dst, b->ld);
+  } else {
+    if (a->pending) status = LaunchPackF32(ctx->stream, a->src, a->dst, a->ld);
+    if (status == hipSuccess && b->pending) status = LaunchPackF32(ctx->stream, b->src, b->dst, b->ld);
+  }
+  a->pending = b->pending = false;
+  if (status != hipSuccess) {
+    *err = "pack kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  return RUYAMD_OK;
+}
+
 int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy,
-                      const void* src_key, int other_width, OperandF32* out, std::string* err) {
+                      const void* src_key, int other_width, OperandF32* out, std::string* err,
+                      PendingPackF32* defer = nullptr) {
   auto view = [&]() {
     const DevMat& m = side == 0 ? call->lhs : call->rhs;
     return side == 0 ? PackSource{m.data, m.rs, m.cs, m.rows, m.cols, m.dtype}
@@ -384,7 +449,13 @@ int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy
     *err = "workspace allocation failed";
     return RUYAMD_E_HIP;
   }
-  if (LaunchPackF32(ctx->stream, src, packed, ld) != hipSuccess) {
+  if (defer) {
+    defer->pending = true;
+    defer->src = src;
+    defer->dst = packed;
+    defer->ld = ld;
+    defer->bytes = packed_bytes;
+  } else if (LaunchPackF32(ctx->stream, src, packed, ld) != hipSuccess) {
     *err = "pack kernel launch failed";
     return RUYAMD_E_HIP;
   }
@@ -420,8 +491,12 @@ bool SetupDestination(const MulCall& call, GemmArgs* args) {
 int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
   OperandF32 a, b;
-  if (int rc = PrepareOperandF32(ctx, call, 0, call->lhs_cache_policy, call->lhs_src_key, N, &a, err)) return rc;
-  if (int rc = PrepareOperandF32(ctx, call, 1, call->rhs_cache_policy, call->rhs_src_key, M, &b, err)) return rc;
+  PendingPackF32 pack_a, pack_b;
+  if (int rc = PrepareOperandF32(ctx, call, 0, call->lhs_cache_policy, call->lhs_src_key, N, &a, err, &pack_a))
+    return rc;
+  if (int rc = PrepareOperandF32(ctx, call, 1, call->rhs_cache_policy, call->rhs_src_key, M, &b, err, &pack_b))
+    return rc;
+  if (int rc = LaunchPendingPacksF32(ctx, &pack_a, &pack_b, err)) return rc;
   if (N <= kSkinnyKernelWidth || M <= kSkinnyKernelWidth) {
     // Bandwidth-bound shapes: stream the wide side exactly once.
     GemvI8Args g;
