@@ -29,6 +29,9 @@ def _problems():
         W.config_int8_gemv(2048, N=1),                                        # cached LHS
         W.config_int8_gemv(1024, N=4, requant=True),
         W.random_problem(rng, S.I8, S.I8, S.I32, S.I32, 300, 260, 7, R, C, C, name="skinny_raw"),
+        # few tiles and a long depth: several workgroups per tile, arrival counters reused by every replay
+        W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, 64, 4096, 100, R, C, C, name="deep_i8"),
+        W.random_problem(rng, S.F32, S.F32, S.F32, S.F32, 64, 2048, 96, R, C, C, name="deep_f32"),
     ]
     return probs
 
