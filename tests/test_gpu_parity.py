@@ -615,6 +615,28 @@ def test_seeded_random_shapes(device_ctx, seed):
         device_ctx.clear_prepacked_cache()
 
 
+@pytest.mark.parametrize("seed", [100, 101])
+def test_seeded_random_deep_shapes(device_ctx, seed):
+    """The same kind of walk over small destinations with long depths (2048 to
+    16384, on and just off the step edges): the products that split the depth
+    over workgroups and over the waves of a workgroup, every type tuple but
+    the fp64 ones, random orders, strides, zero points and parameters. 40
+    problems per seed."""
+    rng = np.random.default_rng(seed)
+    tuples = [t for t in cases.TYPE_TUPLES if S.F64 not in t]
+    for i in range(40):
+        tup = tuples[int(rng.integers(len(tuples)))]
+        M, N = int(rng.integers(1, 330)), int(rng.integers(1, 330))
+        K = int(rng.choice([2048, 4096, 4100, 6144, 8192, 9000, 3000, 16384])) + \
+            int(rng.integers(-3, 4)) * int(rng.integers(2))
+        orders = cases.ALL_ORDERS[int(rng.integers(8))]
+        p = W.random_problem(rng, *tup, M, K, N, *orders, strided=bool(rng.integers(2)),
+                             name="deep seed %d #%d %s %dx%dx%d %s" % (seed, i, cases.tuple_name(tup), M, K, N, orders))
+        announce(p.name)
+        got, want = run_both(device_ctx, p)
+        compare(p, got, want)
+
+
 @pytest.mark.parametrize("tup", [(S.U8, S.U8, S.I32, S.U8), (S.I8, S.U8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I32),
                                  (S.U8, S.U8, S.I32, S.I16)], ids=cases.tuple_name)
 def test_uint8_operands_used_in_place(device_ctx, tup):
