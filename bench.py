@@ -42,7 +42,10 @@ def parse_args():
     # default warm-up is long enough to time the sustained rate.
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="all", choices=["all", "gemm", "gemv"])
+    ap.add_argument("--workload", default="all", choices=["all", "gemm", "gemv", "shape"])
+    ap.add_argument("--shape", default="256,8192,256",
+                    help="M,K,N of --workload shape: the int8 GEMM configuration at another shape "
+                         "(for profiles of the smaller tiles; not part of the default run)")
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the int8 GEMM")
     ap.add_argument("--gemv-size", type=int, default=16384, help="M=K of the int8 GEMV")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -184,6 +187,18 @@ def bench_gemm(ctx, args):
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_gemm(problem, min(n, 512))
     return problem, out
+
+
+def bench_shape(ctx, args):
+    """One int8 product of the GEMM configuration at --shape, timed like the others."""
+    from ruy_amd import workloads as W
+    M, K, N = (int(x) for x in args.shape.split(","))
+    problem = W.config_int8_gemm_shape(M, K, N)
+    dp = device_problem(problem)
+    dp.run(ctx)
+    step_s, kernel_ms, _ = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx)
+    return {"shape": [M, K, N], "kernel": ctx.last_kernel_name(), "us_per_step": step_s * 1e6,
+            "kernel_us": kernel_ms * 1e3 if kernel_ms else None, "Top/s": problem.ops() / step_s / 1e12}
 
 
 def bench_gemm_host_buffers(ctx, problem, steps=3):
@@ -391,6 +406,13 @@ def main():
         "dtype": "int8",
         "data": "synthetic (SplitMix64-seeded uniform int8, random int32 bias)",
     }
+    if args.workload == "shape":
+        line["shape"] = bench_shape(ctx, args)
+        line["value"] = line["shape"]["Top/s"]
+        line["ms_per_step"] = line["shape"]["us_per_step"] / 1e3
+        line["config"] = {"workload": "int8xint8->int8 GEMM configuration at M,K,N = %s" % args.shape}
+        print(json.dumps(line))
+        return
     if args.workload in ("all", "gemm"):
         problem, g = bench_gemm(ctx, args)
         line.update({"value": g["value"], "ms_per_step": g["ms_per_step"],

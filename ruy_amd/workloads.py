@@ -196,6 +196,18 @@ def _filled(dtype, rows, cols, order, seed, lo, hi, **kw):
     return m
 
 
+def config_int8_gemm_shape(M, K, N, config_id=7):
+    """The int8 GEMM configuration at a rectangular shape (same layouts, zero
+    points, bias range, multiplier and clamp as config_int8_gemm)."""
+    lhs = _filled(S.I8, M, K, S.ORDER_ROW_MAJOR, _seed(config_id, 0), -127, 127)
+    rhs = _filled(S.I8, K, N, S.ORDER_COL_MAJOR, _seed(config_id, 1), -128, 127, zero_point=-3)
+    dst = HostMatrix(S.I8, M, N, S.ORDER_COL_MAJOR, zero_point=5)
+    bias = uniform_int(_seed(config_id, 2), M, -1000, 1000, np.int32)
+    return Problem("int8_gemm_%dx%dx%d" % (M, K, N), lhs, rhs, dst, S.I32, bias=bias,
+                   multiplier_fixedpoint=1395864371, multiplier_exponent=-8,
+                   clamp_min=-128, clamp_max=127)
+
+
 def config_int8_gemm(size=256, config_id=1, name=None):
     """int8 x int8 -> int8, M=N=K=size: LHS row-major U[-127,127] zp 0, RHS
     col-major U[-128,127] zp -3, dst col-major zp 5, int32 bias
