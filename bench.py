@@ -42,7 +42,7 @@ def parse_args():
     # default warm-up is long enough to time the sustained rate.
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="all", choices=["all", "gemm", "gemv", "shape"])
+    ap.add_argument("--workload", default="all", choices=["all", "gemm", "gemv", "shape", "mfma-ceiling"])
     ap.add_argument("--shape", default="256,8192,256",
                     help="M,K,N of --workload shape: the int8 GEMM configuration at another shape "
                          "(for profiles of the smaller tiles; not part of the default run)")
@@ -199,6 +199,23 @@ def bench_shape(ctx, args):
     step_s, kernel_ms, _ = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx)
     return {"shape": [M, K, N], "kernel": ctx.last_kernel_name(), "us_per_step": step_s * 1e6,
             "kernel_us": kernel_ms * 1e3 if kernel_ms else None, "Top/s": problem.ops() / step_s / 1e12}
+
+
+def bench_mfma_ceiling(ctx, settle_ms=150.0):
+    """What the bare int8 matrix-instruction loop sustains on this card
+    (ruyamd_diag_mfma_ceiling): both instruction shapes, fragments kept in
+    registers or re-read from LDS, all-zero or uniformly random operands."""
+    out = []
+    for instruction, name in ((0, "v_mfma_i32_32x32x32_i8"), (1, "v_mfma_i32_16x16x64_i8")):
+        for from_lds in (0, 1):
+            for random_operands in (0, 1):
+                tops, ms = ctx.mfma_ceiling(instruction, from_lds, random_operands, settle_ms)
+                out.append({"instruction": name,
+                            "fragments": "lds + barrier" if from_lds else "registers",
+                            "operands": "random bytes" if random_operands else "zero",
+                            "TOP/s": tops, "frac_of_peak": tops / INT8_MFMA_PEAK_TOPS,
+                            "ms_per_launch": ms})
+    return out
 
 
 def bench_gemm_host_buffers(ctx, problem, steps=3):
@@ -406,6 +423,16 @@ def main():
         "dtype": "int8",
         "data": "synthetic (SplitMix64-seeded uniform int8, random int32 bias)",
     }
+    if args.workload == "mfma-ceiling":
+        rows = bench_mfma_ceiling(ctx)
+        best_random = max(r["TOP/s"] for r in rows if r["operands"] == "random bytes")
+        line.update({"metric": "bare int8 matrix-instruction loop, best form on random bytes", "value": best_random,
+                     "ms_per_step": None, "mfma_ceiling": rows,
+                     "config": {"workload": "register/LDS-only matrix-instruction loops, one wave per SIMD, "
+                                            "128x128 accumulator tile per wave, no global memory traffic"}})
+        ctx.close()
+        print(json.dumps(line))
+        return
     if args.workload == "shape":
         line["shape"] = bench_shape(ctx, args)
         line["value"] = line["shape"]["Top/s"]

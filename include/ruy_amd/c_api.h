@@ -238,6 +238,24 @@ RUYAMD_API int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x,
                                        const int32_t* m, const int32_t* e,
                                        int32_t* out, int64_t n);
 
+/* What the int8 matrix instructions sustain on this card when nothing else
+ * runs: one wave per SIMD, each with the 128 x 128 accumulator tile of the
+ * large GEMM tile, issuing `instruction` 0 = v_mfma_i32_32x32x32_i8 or
+ * 1 = v_mfma_i32_16x16x64_i8 back to back on fragments held in registers
+ * (`operands_from_lds` = 0) or re-read from LDS with one workgroup barrier per
+ * 128 bytes of depth (1); operands all zero (`random_operands` = 0) or
+ * uniformly random bytes (1). The card is first kept under this load for
+ * `settle_ms` so that its clock has settled, then 16 launches are timed with
+ * HIP events. This is the ceiling the inner loop that replaces
+ * ruy/kernel_avx512.cc:251-317 can reach here; on random bytes the power
+ * limit sets it well below the published peak. No counterpart in the
+ * reference. */
+RUYAMD_API int ruyamd_diag_mfma_ceiling(ruyamd_ctx* ctx, int instruction,
+                                        int operands_from_lds,
+                                        int random_operands, double settle_ms,
+                                        double* tera_ops_per_second,
+                                        double* ms_per_launch);
+
 /* Library version string. */
 RUYAMD_API const char* ruyamd_version(void);
 

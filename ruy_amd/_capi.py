@@ -59,6 +59,8 @@ PROTOTYPES = {
                                           C.c_void_p, C.c_int64]),
     "ruyamd_ctx_set_kernel_timing": (C.c_int, [_ctx, C.c_int]),
     "ruyamd_ctx_kernel_timing": (C.c_int, [_ctx, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
+    "ruyamd_diag_mfma_ceiling": (C.c_int, [_ctx, C.c_int, C.c_int, C.c_int, C.c_double,
+                                           C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "ruyamd_version": (C.c_char_p, []),
 }
 

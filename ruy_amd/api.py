@@ -329,6 +329,14 @@ class Context:
         self._check(lib.ruyamd_ctx_kernel_timing(self._h, C.byref(ms), C.byref(n)))
         return ms.value, n.value
 
+    def mfma_ceiling(self, instruction, operands_from_lds, random_operands, settle_ms=100.0):
+        """(TOP/s, ms per launch) of the bare int8 matrix-instruction loop."""
+        tops, ms = C.c_double(0), C.c_double(0)
+        self._check(lib.ruyamd_diag_mfma_ceiling(self._h, instruction, int(operands_from_lds),
+                                                 int(random_operands), float(settle_ms),
+                                                 C.byref(tops), C.byref(ms)))
+        return tops.value, ms.value
+
     def apply_multiplier(self, x, m, e, out, n):
         self._check(lib.ruyamd_apply_multiplier(
             self._h, _address(x), _address(m), _address(e), _address(out), n))

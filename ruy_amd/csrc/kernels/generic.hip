@@ -13,6 +13,7 @@
 
 #include "../epilogue.h"
 #include "../internal.h"
+#include "launch_geometry.h"
 
 // Keep every floating-point multiply and add separate in this file: the
 // reference's scalar loop rounds after each of them.
@@ -21,7 +22,7 @@
 namespace ruyamd {
 namespace {
 
-constexpr int kTile = 16;
+constexpr int kTile = kGenericTile;
 
 __device__ __forceinline__ int32_t LoadInt(const void* p, int dtype, int64_t off) {
   switch (dtype) {
@@ -45,21 +46,26 @@ __global__ __launch_bounds__(kTile * kTile) void GenericIntKernel(DevMat lhs, De
   // Lanes run along the destination's contiguous dimension.
   const bool dst_col_major = dst.rs == 1;
   const int fast = blockIdx.x * kTile + threadIdx.x;
-  const int slow = blockIdx.y * kTile + threadIdx.y;
-  const int i = dst_col_major ? fast : slow;
-  const int j = dst_col_major ? slow : fast;
-  if (i >= dst.rows || j >= dst.cols) return;
-  const int depth = lhs.cols;
-  uint32_t acc = 0;
-  const int64_t lbase = int64_t(i) * lhs.rs;
-  const int64_t rbase = int64_t(j) * rhs.cs;
-  for (int k = 0; k < depth; ++k) {
-    const int32_t l = LoadInt(lhs.data, lhs.dtype, lbase + k * lhs.cs) - lhs.zero_point;
-    const int32_t r = LoadInt(rhs.data, rhs.dtype, rbase + k * rhs.rs) - rhs.zero_point;
-    acc += static_cast<uint32_t>(l * r);
+  const int slow_extent = dst_col_major ? dst.cols : dst.rows;
+  // grid.y is capped (65535 tile rows): walk the rest with a stride.
+  for (int64_t slow64 = int64_t(blockIdx.y) * kTile + threadIdx.y; slow64 < slow_extent;
+       slow64 += int64_t(gridDim.y) * kTile) {
+    const int slow = static_cast<int>(slow64);
+    const int i = dst_col_major ? fast : slow;
+    const int j = dst_col_major ? slow : fast;
+    if (i >= dst.rows || j >= dst.cols) return;
+    const int depth = lhs.cols;
+    uint32_t acc = 0;
+    const int64_t lbase = int64_t(i) * lhs.rs;
+    const int64_t rbase = int64_t(j) * rhs.cs;
+    for (int k = 0; k < depth; ++k) {
+      const int32_t l = LoadInt(lhs.data, lhs.dtype, lbase + k * lhs.cs) - lhs.zero_point;
+      const int32_t r = LoadInt(rhs.data, rhs.dtype, rbase + k * rhs.rs) - rhs.zero_point;
+      acc += static_cast<uint32_t>(l * r);
+    }
+    const int32_t v = FinishInt<false>(static_cast<int32_t>(acc), i, j, ep);
+    StoreInt(dst.data, dst.dtype, int64_t(i) * dst.rs + int64_t(j) * dst.cs, v);
   }
-  const int32_t v = FinishInt<false>(static_cast<int32_t>(acc), i, j, ep);
-  StoreInt(dst.data, dst.dtype, int64_t(i) * dst.rs + int64_t(j) * dst.cs, v);
 }
 
 template <typename Acc>
@@ -67,36 +73,41 @@ __global__ __launch_bounds__(kTile * kTile) void GenericFpKernel(DevMat lhs, Dev
                                                                 Epilogue ep, DevMat dst) {
   const bool dst_col_major = dst.rs == 1;
   const int fast = blockIdx.x * kTile + threadIdx.x;
-  const int slow = blockIdx.y * kTile + threadIdx.y;
-  const int i = dst_col_major ? fast : slow;
-  const int j = dst_col_major ? slow : fast;
-  if (i >= dst.rows || j >= dst.cols) return;
-  const int depth = lhs.cols;
-  Acc acc = 0;
-  const int64_t lbase = int64_t(i) * lhs.rs;
-  const int64_t rbase = int64_t(j) * rhs.cs;
-  for (int k = 0; k < depth; ++k) {
-    const Acc l = LoadFp<Acc>(lhs.data, lhs.dtype, lbase + k * lhs.cs);
-    const Acc r = LoadFp<Acc>(rhs.data, rhs.dtype, rbase + k * rhs.rs);
-    const Acc prod = l * r;  // rounded on its own: contraction is off in this file
-    acc = acc + prod;
-  }
-  const int64_t off = int64_t(i) * dst.rs + int64_t(j) * dst.cs;
-  if constexpr (sizeof(Acc) == 4) {
-    static_cast<float*>(dst.data)[off] = FinishF32(acc, i, j, ep);
-  } else {
-    const double v = FinishF64(acc, i, j, ep);
-    if (dst.dtype == RUYAMD_DTYPE_F32)
-      static_cast<float*>(dst.data)[off] = static_cast<float>(v);
-    else
-      static_cast<double*>(dst.data)[off] = v;
+  const int slow_extent = dst_col_major ? dst.cols : dst.rows;
+  for (int64_t slow64 = int64_t(blockIdx.y) * kTile + threadIdx.y; slow64 < slow_extent;
+       slow64 += int64_t(gridDim.y) * kTile) {
+    const int slow = static_cast<int>(slow64);
+    const int i = dst_col_major ? fast : slow;
+    const int j = dst_col_major ? slow : fast;
+    if (i >= dst.rows || j >= dst.cols) return;
+    const int depth = lhs.cols;
+    Acc acc = 0;
+    const int64_t lbase = int64_t(i) * lhs.rs;
+    const int64_t rbase = int64_t(j) * rhs.cs;
+    for (int k = 0; k < depth; ++k) {
+      const Acc l = LoadFp<Acc>(lhs.data, lhs.dtype, lbase + k * lhs.cs);
+      const Acc r = LoadFp<Acc>(rhs.data, rhs.dtype, rbase + k * rhs.rs);
+      const Acc prod = l * r;  // rounded on its own: contraction is off in this file
+      acc = acc + prod;
+    }
+    const int64_t off = int64_t(i) * dst.rs + int64_t(j) * dst.cs;
+    if constexpr (sizeof(Acc) == 4) {
+      static_cast<float*>(dst.data)[off] = FinishF32(acc, i, j, ep);
+    } else {
+      const double v = FinishF64(acc, i, j, ep);
+      if (dst.dtype == RUYAMD_DTYPE_F32)
+        static_cast<float*>(dst.data)[off] = static_cast<float>(v);
+      else
+        static_cast<double*>(dst.data)[off] = v;
+    }
   }
 }
 
 __global__ void ApplyMultiplierKernel(const int32_t* x, const int32_t* m, const int32_t* e,
                                       int32_t* out, int64_t n) {
-  const int64_t idx = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx < n) out[idx] = MultiplyByQuantizedMultiplier(x[idx], m[idx], e[idx]);
+  for (int64_t idx = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; idx < n;
+       idx += int64_t(gridDim.x) * blockDim.x)
+    out[idx] = MultiplyByQuantizedMultiplier(x[idx], m[idx], e[idx]);
 }
 
 }  // namespace
@@ -108,7 +119,8 @@ hipError_t LaunchGeneric(hipStream_t stream, const DevMat& lhs, const DevMat& rh
   const int fast = dst_col_major ? dst.rows : dst.cols;
   const int slow = dst_col_major ? dst.cols : dst.rows;
   dim3 block(kTile, kTile);
-  dim3 grid((fast + kTile - 1) / kTile, (slow + kTile - 1) / kTile);
+  const Grid2D geometry = GenericGrid(fast, slow);
+  dim3 grid(geometry.x, geometry.y);
   if (accum_dtype == RUYAMD_DTYPE_I32) {
     hipLaunchKernelGGL(GenericIntKernel, grid, block, 0, stream, lhs, rhs, ep, dst);
   } else if (accum_dtype == RUYAMD_DTYPE_F32) {
@@ -123,7 +135,7 @@ hipError_t LaunchApplyMultiplier(hipStream_t stream, const int32_t* x, const int
                                  const int32_t* e, int32_t* out, int64_t n) {
   if (n == 0) return hipSuccess;
   const int threads = 256;
-  const unsigned blocks = static_cast<unsigned>((n + threads - 1) / threads);
+  const unsigned blocks = ElementwiseBlocks(n, threads);
   hipLaunchKernelGGL(ApplyMultiplierKernel, dim3(blocks), dim3(threads), 0, stream, x, m, e, out, n);
   return hipGetLastError();
 }

@@ -156,9 +156,15 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
       return RUYAMD_E_HIP;
     }
     if (action == PrepackedCache::Action::kInsertedNewEntry) {
-      if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
+      // The entry exists from here on; if it cannot be filled it must not stay,
+      // or the next call would hit buffers that were never packed.
+      if (int rc = EnsureOnDevice(ctx, call, side, err)) {
+        ctx->cache->Erase(src_key, pm);
+        return rc;
+      }
       src = view();
       if (LaunchPackI8(ctx->stream, src, static_cast<int8_t*>(pm.data), ld, pm.sums) != hipSuccess) {
+        ctx->cache->Erase(src_key, pm);
         *err = "pack kernel launch failed";
         return RUYAMD_E_HIP;
       }
@@ -420,9 +426,13 @@ int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy
       return RUYAMD_E_HIP;
     }
     if (action == PrepackedCache::Action::kInsertedNewEntry) {
-      if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
+      if (int rc = EnsureOnDevice(ctx, call, side, err)) {
+        ctx->cache->Erase(src_key, pm);
+        return rc;
+      }
       src = view();
       if (LaunchPackF32(ctx->stream, src, static_cast<float*>(pm.data), ld) != hipSuccess) {
+        ctx->cache->Erase(src_key, pm);
         *err = "pack kernel launch failed";
         return RUYAMD_E_HIP;
       }

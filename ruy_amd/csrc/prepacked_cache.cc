@@ -23,7 +23,7 @@ PrepackedCache::Action PrepackedCache::Get(const void* src_data, PackedMatrix* p
     *packed_matrix = it->second.packed;
     return Action::kGotExistingEntry;
   }
-  if (mode == Mode::kPinExisting) {
+  if (mode != Mode::kInsertOnMiss) {
     packed_matrix->data = nullptr;
     packed_matrix->sums = nullptr;
     return Action::kMissing;
@@ -46,6 +46,17 @@ PrepackedCache::Action PrepackedCache::Get(const void* src_data, PackedMatrix* p
   cache_.emplace(key, Entry{*packed_matrix, timestamp_++});
   buffers_bytes_ += new_bytes;
   return Action::kInsertedNewEntry;
+}
+
+bool PrepackedCache::Erase(const void* src_data, const PackedMatrix& packed_matrix) {
+  auto it = cache_.find(Key{src_data, packed_matrix.layout, packed_matrix.zero_point});
+  if (it == cache_.end()) return false;
+  const PackedMatrix& pm = it->second.packed;
+  buffers_bytes_ -= pm.DataBytes() + pm.SumsBytes();
+  free_(pm.data);
+  if (pm.sums) free_(pm.sums);
+  cache_.erase(it);
+  return true;
 }
 
 void PrepackedCache::EjectUntilRoomFor(std::ptrdiff_t new_bytes) {

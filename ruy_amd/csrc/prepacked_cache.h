@@ -55,8 +55,10 @@ class PrepackedCache final {
   enum class Action { kGotExistingEntry, kInsertedNewEntry, kMissing };
   // kPinExisting never allocates or frees: a hit is marked so that ejection
   // passes it over from then on (its buffers may be referenced by work that
-  // was recorded for later replay), a miss returns kMissing.
-  enum class Mode { kInsertOnMiss, kPinExisting };
+  // was recorded for later replay), a miss returns kMissing. kLookupOnly is
+  // the same without the mark (for callers that may not allocate but whose
+  // work has run by the time anything could be ejected).
+  enum class Mode { kInsertOnMiss, kPinExisting, kLookupOnly };
   using AllocFn = std::function<void*(std::size_t)>;
   using FreeFn = std::function<void(void*)>;
 
@@ -77,6 +79,12 @@ class PrepackedCache final {
   // is still kept), and inserts it; the caller must then pack into the buffers.
   // Returns kInsertedNewEntry with null data if allocation failed.
   Action Get(const void* src_data, PackedMatrix* packed_matrix, Mode mode = Mode::kInsertOnMiss);
+
+  // Removes the entry with this key, if any, and releases its buffers: for a
+  // caller that was handed a new entry and then failed to fill it, so that no
+  // later Get finds buffers that were never packed. Returns whether an entry
+  // was removed. (No counterpart in the reference, whose pack cannot fail.)
+  bool Erase(const void* src_data, const PackedMatrix& packed_matrix);
 
   std::ptrdiff_t BuffersBytes() const { return buffers_bytes_; }
   int MatrixCount() const { return static_cast<int>(cache_.size()); }

@@ -182,7 +182,44 @@ static void TestDistinguishSubtlyDifferentMatrices() {
   EXPECT(cache.MatrixCount() == 0 && cache.BuffersBytes() == 0);
 }
 
+// A caller that got a new entry and then could not fill it (staging or the
+// pack launch failed) erases it: the next Get for the same key must insert
+// again instead of returning buffers that were never packed, and the byte and
+// allocation accounting must be as if the entry had never existed.
+static void TestEraseAfterFailedPack() {
+  const int live_before = g_live_allocations;
+  {
+    PrepackedCache cache(CountingAlloc, CountingFree, 1000);
+    std::vector<std::uint8_t> d1(200), d2(15);
+    PackedMatrix m1 = Dummy(false, 10, 20), m2 = Dummy(false, 5, 3);
+    EXPECT(cache.Get(d1.data(), &m1) == kInserted);
+    EXPECT(cache.Get(d2.data(), &m2) == kInserted);
+    EXPECT(cache.BuffersBytes() == 307 && cache.MatrixCount() == 2);
+    EXPECT(cache.Erase(d1.data(), m1));
+    EXPECT(cache.BuffersBytes() == 27 && cache.MatrixCount() == 1);
+    EXPECT(g_live_allocations == live_before + 2);  // only m2's data and sums are left
+    EXPECT(!cache.Erase(d1.data(), m1));            // already gone
+    PackedMatrix again = Dummy(false, 10, 20);
+    EXPECT(cache.Get(d1.data(), &again) == kInserted);  // not a hit on stale buffers
+    EXPECT(cache.BuffersBytes() == 307 && cache.MatrixCount() == 2);
+    // A key that differs only in the zero point is a different entry.
+    PackedMatrix other = Dummy(false, 5, 3);
+    other.zero_point = 1;
+    EXPECT(!cache.Erase(d2.data(), other));
+    EXPECT(cache.MatrixCount() == 2);
+    // Lookup-only mode: a hit without the ejection mark, a miss without an insert.
+    PackedMatrix probe = Dummy(false, 5, 3);
+    EXPECT(cache.Get(d2.data(), &probe, PrepackedCache::Mode::kLookupOnly) == kExisting);
+    EXPECT(probe.data == m2.data);
+    PackedMatrix absent = Dummy(false, 7, 7);
+    EXPECT(cache.Get(d2.data(), &absent, PrepackedCache::Mode::kLookupOnly) == PrepackedCache::Action::kMissing);
+    EXPECT(absent.data == nullptr && cache.MatrixCount() == 2);
+  }
+  EXPECT(g_live_allocations == live_before);
+}
+
 int main() {
+  TestEraseAfterFailedPack();
   TestBasic();
   TestBasicFloat();
   TestEjection();

@@ -77,6 +77,15 @@ def test_prepacked_cache_known_answers():
     assert "all passed" in out
 
 
+def test_host_launch_arithmetic():
+    """Grid shapes stay inside HIP's limits and still cover every element."""
+    exe = os.path.join(ROOT, "tests", "cpp", "host_logic_test")
+    subprocess.check_call(["g++", "-std=c++17", "-pthread", "-I" + os.path.join(ROOT, "ruy_amd", "csrc"),
+                           exe + ".cc", "-o", exe])
+    out = subprocess.check_output([exe]).decode()
+    assert "all passed" in out
+
+
 @pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "example")),
                     reason="reference tree not present")
 @pytest.mark.parametrize("std", ["c++14", "c++17"])
