@@ -58,9 +58,8 @@ def parse_args():
 
 
 def device_problem(problem):
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import device_runner
-    return device_runner.DeviceProblem(problem, dst_fill=0)
+    from ruy_amd import device_problem as D
+    return D.DeviceProblem(problem, dst_fill=0)
 
 
 def time_steps(run, steps, warmup, ctx):

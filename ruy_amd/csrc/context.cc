@@ -9,7 +9,14 @@
 namespace ruyamd {
 
 Workspace::~Workspace() {
+  if (fixed_) return;
   for (auto& b : blocks_) (void)hipFree(b.base);
+}
+
+void Workspace::UseFixed(void* base, std::size_t size) {
+  fixed_ = true;
+  growth_allowed_ = false;
+  blocks_.assign(1, Block{static_cast<char*>(base), size, 0});
 }
 
 std::size_t Workspace::capacity() const {
@@ -27,11 +34,15 @@ void* Workspace::Alloc(std::size_t bytes) {
       return p;
     }
   }
-  if (!growth_allowed_) return nullptr;
+  if (!growth_allowed_ || fixed_) {
+    exhausted_ = true;
+    return nullptr;
+  }
   std::size_t size = need < (std::size_t(1) << 20) ? (std::size_t(1) << 20) : need;
   void* p = nullptr;
   if (hipMalloc(&p, size) != hipSuccess) {
     (void)hipGetLastError();
+    exhausted_ = true;
     return nullptr;
   }
   blocks_.push_back(Block{static_cast<char*>(p), size, need});
@@ -39,7 +50,8 @@ void* Workspace::Alloc(std::size_t bytes) {
 }
 
 void Workspace::Reset() {
-  if (blocks_.size() > 1 && !pinned_ && growth_allowed_) {
+  exhausted_ = false;
+  if (blocks_.size() > 1 && !pinned_ && growth_allowed_ && !fixed_) {
     // Coalesce: one block as large as everything the last call needed.
     std::size_t total = 0;
     for (auto& b : blocks_) {
@@ -211,7 +223,7 @@ void HostStaging::Reset() {
 using ruyamd::PrepackedCache;
 
 bool ruyamd_ctx::TimingBegin() {
-  if (!kernel_timing || capturing) return false;
+  if (!kernel_timing || capturing || no_alloc) return false;  // creating events allocates
   std::pair<hipEvent_t, hipEvent_t> ev;
   if (!timing_pool.empty()) {
     ev = timing_pool.back();

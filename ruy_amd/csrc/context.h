@@ -36,6 +36,11 @@ class Workspace {
   std::size_t capacity() const;
   void Pin() { pinned_ = true; }
   void set_growth_allowed(bool allowed) { growth_allowed_ = allowed; }
+  // Makes this a workspace over memory it does not own: one block that is
+  // never released, replaced or added to. For a workspace that owns nothing.
+  void UseFixed(void* base, std::size_t size);
+  // Whether an Alloc has failed since the last Reset.
+  bool exhausted() const { return exhausted_; }
 
  private:
   struct Block {
@@ -46,6 +51,8 @@ class Workspace {
   std::vector<Block> blocks_;
   bool pinned_ = false;
   bool growth_allowed_ = true;
+  bool fixed_ = false;
+  bool exhausted_ = false;
 };
 
 // Moves pageable host memory to and from the device through a small ring of
@@ -92,6 +99,9 @@ struct ruyamd_ctx {
   hipStream_t stream = nullptr;
   bool synchronous = true;
   bool capturing = false;  // this call's stream is recording a graph
+  // This call may not allocate device memory (ruyamd_mul_no_alloc): scratch
+  // comes from the GPU's static area, the prepacked cache is only looked up.
+  bool no_alloc = false;
   int last_used_path = RUYAMD_PATH_NONE;
   int runtime_enabled_paths = RUYAMD_PATH_NONE;  // kNone = not decided yet
   int max_num_threads = 1;
@@ -101,13 +111,17 @@ struct ruyamd_ctx {
   int last_kernel = RUYAMD_KERNEL_NONE;
   bool force_generic = false;
   std::string last_error;
-  ruyamd::Workspace workspace;
+  ruyamd::Workspace workspace;         // grows on demand (hipMalloc)
+  ruyamd::Workspace static_workspace;  // over this GPU's static scratch area
+  ruyamd::Workspace* ws = &workspace;  // the one the current call draws from
   ruyamd::HostStaging staging;
   std::unique_ptr<ruyamd::PrepackedCache> cache;
   int multiprocessor_count = 0;
   // Arrival counters of the depth-split matrix-core kernels: zero between
   // launches (the kernels leave them so), allocated with the context.
   uint32_t* split_counters = nullptr;
+  // The same in this GPU's static scratch area, for calls that may not allocate.
+  uint32_t* static_split_counters = nullptr;
   // Optional timing of the dominant kernel of each call.
   bool kernel_timing = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pending;

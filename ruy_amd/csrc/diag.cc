@@ -24,10 +24,10 @@ extern "C" int ruyamd_diag_mfma_ceiling(ruyamd_ctx* ctx, int instruction, int op
   if (hipStreamIsCapturing(ctx->stream, &status) == hipSuccess && status == hipStreamCaptureStatusActive)
     return fail(RUYAMD_E_UNSUPPORTED, "the stream is capturing");
   if (hipStreamSynchronize(ctx->stream) != hipSuccess) return fail(RUYAMD_E_HIP, "stream synchronisation failed");
-  ctx->workspace.Reset();
+  ctx->ws->Reset();
   const int workgroups = ctx->multiprocessor_count;  // one workgroup of four waves per CU
-  void* operands = ctx->workspace.Alloc(kMfmaCeilingOperandBytes);
-  int* sink = static_cast<int*>(ctx->workspace.Alloc(std::size_t(workgroups) * 256 * sizeof(int)));
+  void* operands = ctx->ws->Alloc(kMfmaCeilingOperandBytes);
+  int* sink = static_cast<int*>(ctx->ws->Alloc(std::size_t(workgroups) * 256 * sizeof(int)));
   if (!operands || !sink) return fail(RUYAMD_E_HIP, "workspace allocation failed");
   std::vector<uint64_t> host(kMfmaCeilingOperandBytes / 8, 0);
   if (random_operands) {

@@ -96,10 +96,14 @@ __global__ __launch_bounds__(256) void MfmaCeilingKernel(const v4i* operands, in
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
-          for (int j = 0; j < 8; ++j) c[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], c[i][j], 0, 0, 0);
+          for (int j = 0; j < 8; ++j)
+            // Accumulator tied to itself: with the builtin the compiler moves these
+            // small accumulators between registers inside the loop.
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[i][j]) : "v"(a[i]), "v"(b[j]));
       }
       if constexpr (kFromLds) __syncthreads();
     }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last instructions finish before their results are read
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll

@@ -23,6 +23,9 @@ struct F32Traits {
     for (int e = 0; e < 4; ++e)
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[e]), __int_as_float(b[e]), acc, 0, 0, 0);
   }
+  static __device__ __forceinline__ void DrainMma() {}
+  static constexpr int kBlock = 32;
+  using LargeTile = F32Traits;
   static constexpr bool kSplitB = false;
   static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kF32;
   // Time between two dependent launches (about 5 us) in depth steps of the

@@ -19,11 +19,17 @@ __device__ __forceinline__ int32_t RequantHigh(int32_t x, int32_t m, int s) {
   return (__mulhi(x, m) + (1 << (s - 1))) >> s;
 }
 
+struct Int8Traits16;
+
 struct Int8Traits {
   using Acc = v16i;
   static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
   }
+  static __device__ __forceinline__ void DrainMma() {}
+  static constexpr int kBlock = 32;
+  // The 256x256 tile runs on 16x16 blocks (below).
+  using LargeTile = Int8Traits16;
   static constexpr bool kSplitB = false;
   static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kInt8;
   // Time between two dependent launches (about 5 us) in depth steps of the
@@ -107,6 +113,31 @@ struct Int8Traits {
   }
 };
 
+// The same arithmetic on v_mfma_i32_16x16x64_i8: a quarter of the accumulator
+// registers read and written per instruction for half the operations, which on
+// random operand bytes, where the card runs into its power limit, costs about
+// a tenth less energy per operation than the 32x32x32 form; the fragment bytes
+// read from LDS per operation are the same. Used for the largest tile, whose
+// grids run long enough for the power limit to decide the clock.
+//
+// The instruction is written as inline assembly with the accumulator tied to
+// itself: given the builtin, the compiler's register allocator moves dozens of
+// these small accumulators between registers on every trip round the loop.
+// The compiler's hazard checks do not look inside inline assembly; the kernel
+// keeps what they would have ensured: consecutive instructions never share an
+// accumulator, an accumulator is next touched 63 instructions later, and
+// DrainMma() stands between the last instruction and the first ordinary read
+// of an accumulator.
+struct Int8Traits16 : Int8Traits {
+  using Acc = v4i;
+  static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void DrainMma() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+  static constexpr int kBlock = 16;
+  using LargeTile = Int8Traits16;
+};
+
 // int8 x int16 (ruy/kernel_avx512.cc:55-626 instantiated for a 16-bit RHS,
 // ruy/kernel_x86.h:62-90): the int16 operand arrives split into a high and a
 // low int8 plane, v = 256*hi + (lo + 128), and each plane is multiplied on
@@ -115,6 +146,7 @@ struct Int8Traits {
 // row" is the ordinary zero-point correction with an RHS zero point of -128,
 // which the dispatcher sets. Everything is exact modulo 2^32.
 struct Int8SplitTraits : Int8Traits {
+  using LargeTile = Int8SplitTraits;
   static constexpr bool kSplitB = true;
   static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kInt8PlaneSplit;
   static __device__ __forceinline__ int Bits(int hi, int lo) {

@@ -27,8 +27,11 @@
 // touches all 64 banks; since a direct-to-LDS load places lane l at
 // base + 16*l, the swizzle is applied to the global address each lane fetches.
 //
-// A Traits type supplies: Acc (16-element accumulator vector), Mma(a, b, acc)
-// for one 16-byte fragment pair, kSplitB (the B operand holds, for every 32
+// A Traits type supplies: kBlock (32: one matrix instruction per 32x32 block
+// and 32 bytes of depth; 16: per 16x16 block and 64 bytes of depth), Acc (the
+// accumulator vector of one block: 16 or 4 elements), Mma(a, b, acc)
+// for one 16-byte fragment pair, DrainMma() (called once after the last Mma),
+// LargeTile (the Traits the 256x256 tile runs with), kSplitB (the B operand holds, for every 32
 // destination columns, 32 high-plane rows followed by 32 low-plane rows whose
 // accumulators are combined), Bits(x, x2) (accumulator element - or combined
 // pair - as raw 32 bits), RawBits(x) / FromRawBits(w) (one accumulator element
@@ -120,14 +123,16 @@ __device__ __forceinline__ int LdsOffset(int r, int g) {
   return r * BK + ((g ^ Swizzle<BK>(r)) << 4);
 }
 
-template <int WM, int WN, int BK, int STAGES, bool SPLIT_B = false>
+template <int WM, int WN, int BK, int STAGES, bool SPLIT_B = false, int BLOCK = 32>
 struct Cfg {
   static constexpr int kBM = 2 * WM * 32;
   static constexpr int kBN = 2 * WN * 32;
   static constexpr int kBK = BK;
   static constexpr int kThreads = 256;
   static constexpr int kStages = STAGES;
-  static constexpr int kKSteps = BK / 32;           // matrix-instruction depth steps per stage
+  // Matrix-instruction depth steps per stage: a 32x32 block instruction takes
+  // 32 bytes of depth, a 16x16 block instruction 64.
+  static constexpr int kKSteps = BK / (BLOCK == 16 ? 64 : 32);
   static constexpr int kGranulesPerRow = BK / kGranule;
   static constexpr int kRowsPerLoad = 64 / kGranulesPerRow;  // tile rows one wave-level load covers
   static constexpr int kALoads = kBM / kRowsPerLoad / 4;     // per wave per stage
@@ -167,7 +172,21 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   static_assert(!kFlip || WM * WN == 1, "in-place uint8 operands exist for the single-block tile only");
   static_assert(!kDepthWaves || (WM == 1 && WN == (Traits::kSplitB ? 2 : 1) && BK == 128),
                 "the depth-per-wave schedule exists for the smallest tile of each kernel");
-  using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
+  // Accumulator blocks: Traits::kBlock = 32 (one matrix instruction covers a
+  // 32x32 block and 32 bytes of depth: lane l supplies 16 depth bytes of row
+  // l%32 at depth granule l/32) or 16 (16x16 block, 64 bytes of depth: row
+  // l%16, depth granule l/16). WM and WN always count 32-row units; with 16x16
+  // blocks a wave holds kNB*WM x kNB*WN blocks of a quarter of the size.
+  constexpr int kB = Traits::kBlock;
+  static_assert(kB == 32 || kB == 16, "");
+  static_assert(kB == 32 || (!kFusedSums && !kFlip && !kDepthWaves && !Traits::kSplitB),
+                "the 16x16 block form exists for the plain schedule only");
+  constexpr int kNB = 32 / kB;
+  constexpr int kAB = WM * kNB;  // blocks of A rows per wave
+  constexpr int kBB = WN * kNB;  // blocks of B rows (destination columns) per wave
+  constexpr int kAccElems = kB * kB / 64;
+  constexpr int kGranulesPerMma = 64 / kB;  // 16-byte depth granules of a row that one instruction consumes
+  using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB, kB>;
   constexpr int kBK = BK;
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -244,7 +263,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // steps only; their accumulators are added up before the write-back (below).
   // k_tiles, kt_first: the steps this workgroup walks.
   const int k_tiles_all = (K + kBK - 1) / kBK;
-  constexpr bool kCanSplitDepth = WM * WN <= 2;
+  constexpr bool kCanSplitDepth = WM * WN <= 2 && kB == 32;
   const int split = kCanSplitDepth ? args.split_k : 1;
   const int split_index = kCanSplitDepth ? blockIdx.y : 0;
   const int k_tiles_per_split = (k_tiles_all + split - 1) / split;
@@ -288,50 +307,55 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   };
 
   // ---- LDS -> MFMA fragments ----
-  // Fragment of 32x32 block b, depth sub-step ks: lane reads tile row
-  // b*32 + lane%32, granule ks*2 + lane/32.
-  const int frag_row = lane & 31;
-  const int frag_half = lane >> 5;
+  // Fragment of block b (kB rows), depth sub-step ks: lane reads tile row
+  // b*kB + lane%kB, granule ks*kGranulesPerMma + lane/kB.
+  const int frag_row = lane & (kB - 1);
+  const int frag_half = lane / kB;
   int a_foff[C::kKSteps], b_foff[C::kKSteps];  // byte offsets inside a stage, block 0 of this wave
 #pragma unroll
   for (int ks = 0; ks < C::kKSteps; ++ks) {
-    // Blocks are 32 rows apart, which leaves the swizzle term unchanged.
-    a_foff[ks] = LdsOffset<BK>(wave_m * WM * 32 + frag_row, ks * 2 + frag_half);
-    b_foff[ks] = C::kBM * kBK + LdsOffset<BK>(wave_n * WN * 32 + frag_row, ks * 2 + frag_half);
+    // Blocks are 32 (16) rows apart, which leaves the swizzle term unchanged.
+    a_foff[ks] = LdsOffset<BK>(wave_m * WM * 32 + frag_row, ks * kGranulesPerMma + frag_half);
+    b_foff[ks] = C::kBM * kBK + LdsOffset<BK>(wave_n * WN * 32 + frag_row, ks * kGranulesPerMma + frag_half);
   }
   struct Frags {
-    v4i a[WM];
-    v4i b[WN];
+    v4i a[kAB];
+    v4i b[kBB];
   };
   auto read_frags = [&](int kt, int ks, Frags& f) {
     const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
 #pragma unroll
-    for (int i = 0; i < WM; ++i)
-      f.a[i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * 32 * kBK);
+    for (int i = 0; i < kAB; ++i)
+      f.a[i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * kB * kBK);
 #pragma unroll
-    for (int j = 0; j < WN; ++j)
-      f.b[j] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * 32 * kBK);
+    for (int j = 0; j < kBB; ++j)
+      f.b[j] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * kB * kBK);
   };
-  // Fragment number r (0 .. WM+WN-1: the A fragments, then the B fragments).
+  // Fragment number r. 32x32 blocks: the A fragments, then the B fragments.
+  // 16x16 blocks: the B fragments first, because the matrix instructions of a
+  // sub-step walk the blocks row by row and so need every B fragment, but only
+  // the first A fragment, right at its start.
   auto read_one = [&](int kt, int ks, int r, Frags& f) {
     const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
-    if (r < WM)
-      f.a[r] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + r * 32 * kBK);
+    const bool is_a = kB == 32 ? r < kAB : r >= kBB;
+    const int idx = kB == 32 ? (r < kAB ? r : r - kAB) : (r < kBB ? r : r - kBB);
+    if (is_a)
+      f.a[idx] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + idx * kB * kBK);
     else
-      f.b[r - WM] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + (r - WM) * 32 * kBK);
+      f.b[idx] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + idx * kB * kBK);
   };
 
-  typename Traits::Acc acc[WM][WN];
+  typename Traits::Acc acc[kAB][kBB];
 #pragma unroll
-  for (int i = 0; i < WM; ++i)
+  for (int i = 0; i < kAB; ++i)
 #pragma unroll
-    for (int j = 0; j < WN; ++j)
+    for (int j = 0; j < kBB; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+      for (int v = 0; v < kAccElems; ++v) acc[i][j][v] = 0;
 
   typename Traits::Acc sum_a, sum_b;  // kFusedSums: row sums of a / column sums of b, in every column / row
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
+  for (int v = 0; v < kAccElems; ++v) {
     sum_a[v] = 0;
     sum_b[v] = 0;
   }
@@ -343,11 +367,15 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // one at a time between them. A matrix instruction occupies its pipe for 32
   // cycles but issues in a few, so whatever is issued right behind it is free;
   // a block of loads issued back to back instead would stall the pipe.
-  constexpr int kMmas = WM * WN;
-  constexpr int kFrags = WM + WN;
+  constexpr int kMmas = kAB * kBB;
+  constexpr int kFrags = kAB + kBB;
   // The fragment reads go behind the first matrix instructions of the
   // sub-step, so that they have landed well before the next sub-step starts.
-  constexpr int kReadSlots = kMmas < kFrags ? kMmas : kFrags;
+  // (16x16 blocks: four times as many, shorter instructions per fragment; the
+  // reads are spread over the first half of the sub-step, one behind every
+  // second instruction, so that the barrier at the end of a ring step, which
+  // waits for every LDS read, finds them done.)
+  constexpr int kReadSlots = kB == 16 ? kMmas / 2 : (kMmas < kFrags ? kMmas : kFrags);
   auto sub_step = [&](const Frags& cur_raw, Frags& next, int kt_next, int ks_next, int kt_dma,
                       auto dma_is_full_step) {
     Frags flipped;
@@ -368,7 +396,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 #pragma unroll
     for (int n = 0; n < kMmas; ++n) {
       __builtin_amdgcn_sched_barrier(0);
-      Traits::Mma(cur.a[n / WN], cur.b[n % WN], acc[n / WN][n % WN]);
+      Traits::Mma(cur.a[n / kBB], cur.b[n % kBB], acc[n / kBB][n % kBB]);
       if constexpr (kFusedSums) {
         // Once per sub-step. The plane-split operand has zero point 0 by
         // definition, so its column sums are never needed.
@@ -595,6 +623,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
     for (; kt < full_end; ++kt) ring_step(kt, std::true_type());
     for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type());
   }
+  Traits::DrainMma();  // (matrix instructions the compiler does not see: let the last ones finish)
   WaitVmcnt<0>();
   __syncthreads();  // every wave is done with the operand ring
   if constexpr (kFusedSums && !kDepthWaves) {
@@ -715,21 +744,40 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   for (int half = 0; half < C::kLogicalWN / C::kEpilogueBlockCols; ++half) {
 #pragma unroll
     for (int bjj = 0; bjj < C::kEpilogueBlockCols; ++bjj) {
+      const int lb = half * C::kEpilogueBlockCols + bjj;  // logical block column (32 destination columns)
+      if constexpr (kB == 32) {
 #pragma unroll
-      for (int bi = 0; bi < WM; ++bi) {
+        for (int bi = 0; bi < WM; ++bi) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          constexpr int kPhys = Traits::kSplitB ? 2 : 1;
-          const int lb = half * C::kEpilogueBlockCols + bjj;  // logical block column
-          const typename Traits::Acc& a = acc[bi][kPhys * lb];
-          const typename Traits::Acc& a2 = acc[bi][kPhys * lb + kPhys - 1];
-          v4i w;
-          w[0] = Traits::Bits(a[4 * q + 0], a2[4 * q + 0]);
-          w[1] = Traits::Bits(a[4 * q + 1], a2[4 * q + 1]);
-          w[2] = Traits::Bits(a[4 * q + 2], a2[4 * q + 2]);
-          w[3] = Traits::Bits(a[4 * q + 3], a2[4 * q + 3]);
-          const int r = bi * 32 + 8 * q + 4 * frag_half;
-          *reinterpret_cast<v4i*>(region + (bjj * 32 + frag_row) * kPitch + r) = w;
+          for (int q = 0; q < 4; ++q) {
+            constexpr int kPhys = Traits::kSplitB ? 2 : 1;
+            const typename Traits::Acc& a = acc[bi][kPhys * lb];
+            const typename Traits::Acc& a2 = acc[bi][kPhys * lb + kPhys - 1];
+            v4i w;
+            w[0] = Traits::Bits(a[4 * q + 0], a2[4 * q + 0]);
+            w[1] = Traits::Bits(a[4 * q + 1], a2[4 * q + 1]);
+            w[2] = Traits::Bits(a[4 * q + 2], a2[4 * q + 2]);
+            w[3] = Traits::Bits(a[4 * q + 3], a2[4 * q + 3]);
+            const int r = bi * 32 + 8 * q + 4 * frag_half;
+            *reinterpret_cast<v4i*>(region + (bjj * 32 + frag_row) * kPitch + r) = w;
+          }
+        }
+      } else {
+        // 16x16 block: lane l holds column l%16 and the four consecutive rows
+        // 4*(l/16) .. 4*(l/16)+3, which is one 16-byte LDS write.
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj) {
+#pragma unroll
+          for (int bi = 0; bi < kAB; ++bi) {
+            const typename Traits::Acc& a = acc[bi][2 * lb + bj];
+            v4i w;
+            w[0] = Traits::Bits(a[0], a[0]);
+            w[1] = Traits::Bits(a[1], a[1]);
+            w[2] = Traits::Bits(a[2], a[2]);
+            w[3] = Traits::Bits(a[3], a[3]);
+            const int r = bi * 16 + 4 * frag_half;
+            *reinterpret_cast<v4i*>(region + (bjj * 32 + bj * 16 + frag_row) * kPitch + r) = w;
+          }
         }
       }
     }
@@ -800,7 +848,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
-  using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB>;
+  using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB, Traits::kBlock>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
   const int tiles_n = (args.N + C::kBN - 1) / C::kBN;
   const int total = tiles_m * tiles_n;
@@ -819,7 +867,7 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int split = args.split_k;
   if (split != 1) {
     const int k_tiles = (args.k_bytes + BK - 1) / BK;
-    if (WM * WN > 2 || split < 1 || !args.split_partials || !args.split_counters || total > kSplitCounters ||
+    if (WM * WN > 2 || Traits::kBlock != 32 || split < 1 || !args.split_partials || !args.split_counters || total > kSplitCounters ||
         (split - 1) * ((k_tiles + split - 1) / split) >= k_tiles)
       return hipErrorInvalidValue;
   }
@@ -1035,7 +1083,7 @@ template <typename Traits>
 hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int num_cus) {
   switch (tile) {
     case Tile::k256x256:
-      return Launch<Traits, 4, 4, 128, 2>(stream, args);
+      return Launch<typename Traits::LargeTile, 4, 4, 128, 2>(stream, args);
     case Tile::k128x128:
       if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128)) return Launch<Traits, 2, 2, 128, 2>(stream, args);
       return Launch<Traits, 2, 2, 128, 4>(stream, args);
@@ -1073,7 +1121,7 @@ hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
         const GemmArgs main = plan.along_n ? SubProblem(args, 0, args.M, 0, cut) : SubProblem(args, 0, cut, 0, args.N);
         const GemmArgs tail = plan.along_n ? SubProblem(args, 0, args.M, cut, args.N - cut)
                                            : SubProblem(args, cut, args.M - cut, 0, args.N);
-        const hipError_t first = Launch<Traits, 4, 4, 128, 2>(stream, main);
+        const hipError_t first = Launch<typename Traits::LargeTile, 4, 4, 128, 2>(stream, main);
         if (first != hipSuccess) return first;
         return LaunchTile<Traits>(stream, tail, PickTile(tail, num_cus, Traits::kModel), num_cus);
       }

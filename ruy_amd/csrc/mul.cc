@@ -108,10 +108,11 @@ int64_t StorageElements(const ruyamd_mat& m) {
   return (outer - 1) * m.stride + inner;
 }
 
-// Makes `bytes` of possibly-host memory readable on the device.
-const void* StageIn(ruyamd_ctx* ctx, const void* p, std::size_t bytes, bool* staged_any, bool* ok) {
-  if (!p || bytes == 0 || IsDevicePointer(p)) return p;
-  void* d = ctx->workspace.Alloc(bytes);
+// Makes `bytes` of host memory readable on the device (`on_device`: it already is).
+const void* StageIn(ruyamd_ctx* ctx, const void* p, bool on_device, std::size_t bytes, bool* staged_any,
+                    bool* ok) {
+  if (!p || bytes == 0 || on_device) return p;
+  void* d = ctx->ws->Alloc(bytes);
   if (!d || !ctx->staging.ToDevice(d, p, bytes, ctx->stream)) {
     *ok = false;
     return nullptr;
@@ -131,10 +132,14 @@ class CaptureScope {
       status = hipStreamCaptureStatusNone;
     }
     ctx->capturing = status == hipStreamCaptureStatusActive;
-    if (ctx->capturing) {
-      ctx->workspace.Pin();
-      ctx->workspace.set_growth_allowed(false);
-    }
+    if (ctx->capturing) ctx->workspace.set_growth_allowed(false);
+  }
+  // The call has recorded its kernels: the scratch memory they refer to must
+  // stay where it is from now on. (A call that failed has recorded nothing that
+  // will be replayed by a caller who checks the return code, and leaves the
+  // workspace free to coalesce.)
+  void Recorded() {
+    if (ctx_->capturing && !ctx_->no_alloc) ctx_->workspace.Pin();
   }
   ~CaptureScope() {
     ctx_->capturing = false;
@@ -168,10 +173,29 @@ int32_t ClampToInt32(double v) {
 }  // namespace
 }  // namespace ruyamd
 
-using namespace ruyamd;
+namespace ruyamd {
+namespace {
 
-extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
-                          const ruyamd_mul_params* p, const ruyamd_mat* dst) {
+// Restores the context's per-call mode when a call that may not allocate ends.
+class NoAllocScope {
+ public:
+  NoAllocScope(ruyamd_ctx* ctx, bool no_alloc) : ctx_(ctx) {
+    ctx->no_alloc = no_alloc;
+    ctx->ws = no_alloc ? &ctx->static_workspace : &ctx->workspace;
+  }
+  ~NoAllocScope() {
+    ctx_->no_alloc = false;
+    ctx_->ws = &ctx_->workspace;
+  }
+  NoAllocScope(const NoAllocScope&) = delete;
+  NoAllocScope& operator=(const NoAllocScope&) = delete;
+
+ private:
+  ruyamd_ctx* ctx_;
+};
+
+int MulImpl(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs, const ruyamd_mul_params* p,
+            const ruyamd_mat* dst, bool no_alloc) {
   if (!ctx) return RUYAMD_E_INVALID;
   ctx->performance_advisories = 0;  // ruy/frontend.h:86 clears them per call
   if (int rc = Validate(ctx, lhs, rhs, p, dst)) return rc;
@@ -187,56 +211,61 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
   ctx->last_used_path = RUYAMD_PATH_GFX950;
   ctx->last_kernel = RUYAMD_KERNEL_NONE;
 
-  if (hipSetDevice(ctx->device) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "hipSetDevice failed");
+  int current_device = -1;
+  if (hipGetDevice(&current_device) != hipSuccess || current_device != ctx->device) {
+    if (hipSetDevice(ctx->device) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "hipSetDevice failed");
+  }
   if (dst->rows == 0 || dst->cols == 0) return RUYAMD_OK;
 
+  NoAllocScope no_alloc_scope(ctx, no_alloc);
   // A stream that is recording a graph takes kernel launches only: nothing
   // below may allocate, free, copy from or to the host, or wait. Scratch
   // memory and cache entries that recorded kernels refer to stay where they
   // are until the context is destroyed (cache entries: or cleared).
   CaptureScope capture_scope(ctx);
-  if (ctx->capturing) {
-    const void* pointers[] = {lhs->data, rhs->data, dst->data, p->bias, p->multiplier_fixedpoint_perchannel,
-                              p->multiplier_exponent_perchannel};
-    for (const void* ptr : pointers) {
-      if (ptr && !IsDevicePointer(ptr))
-        return Fail(ctx, RUYAMD_E_UNSUPPORTED, "the stream is capturing: every buffer must be device memory");
-    }
-  }
+
+  // Every buffer of the call is classified once.
+  const bool lhs_dev = !lhs->data || IsDevicePointer(lhs->data);
+  const bool rhs_dev = !rhs->data || IsDevicePointer(rhs->data);
+  const bool dst_on_device = IsDevicePointer(dst->data);
+  const bool bias_dev = !p->bias || IsDevicePointer(p->bias);
+  const bool mf_dev = !p->multiplier_fixedpoint_perchannel || IsDevicePointer(p->multiplier_fixedpoint_perchannel);
+  const bool me_dev = !p->multiplier_exponent_perchannel || IsDevicePointer(p->multiplier_exponent_perchannel);
+  if ((ctx->capturing || no_alloc) && !(lhs_dev && rhs_dev && dst_on_device && bias_dev && mf_dev && me_dev))
+    return Fail(ctx, RUYAMD_E_UNSUPPORTED,
+                no_alloc ? "ruyamd_mul_no_alloc: every buffer must be device memory (staging host memory allocates)"
+                         : "the stream is capturing: every buffer must be device memory");
 
   // Scratch of the previous call is reused. If that call was asynchronous its
   // kernels may not have run yet, but everything that touches the scratch -
   // theirs and ours - is enqueued on ctx->stream, so stream order keeps the
   // uses apart.
-  ctx->workspace.Reset();
+  ctx->ws->Reset();
 
   bool staged = false, ok = true;
   const int channels = p->channel_dimension == RUYAMD_CHANNEL_ROW ? dst->rows : dst->cols;
   // The two source matrices are staged lazily by the dispatcher (a cache hit
   // needs no copy); the small per-channel vectors are staged now.
-  const void* bias_d = StageIn(ctx, p->bias, std::size_t(channels) * DtypeSize(p->accum_dtype), &staged, &ok);
-  const void* mf_d = StageIn(ctx, p->multiplier_fixedpoint_perchannel, std::size_t(channels) * 4, &staged, &ok);
-  const void* me_d = StageIn(ctx, p->multiplier_exponent_perchannel, std::size_t(channels) * 4, &staged, &ok);
+  const void* bias_d = StageIn(ctx, p->bias, bias_dev, std::size_t(channels) * DtypeSize(p->accum_dtype), &staged, &ok);
+  const void* mf_d = StageIn(ctx, p->multiplier_fixedpoint_perchannel, mf_dev, std::size_t(channels) * 4, &staged, &ok);
+  const void* me_d = StageIn(ctx, p->multiplier_exponent_perchannel, me_dev, std::size_t(channels) * 4, &staged, &ok);
   if (!ok) return Fail(ctx, RUYAMD_E_HIP, "staging host operands to the device failed");
 
   // Destination: device memory is written in place; host memory gets a device
   // image with the same stride of which only the rows (columns) themselves are
   // copied back, so the padding between them is never touched.
-  const bool dst_on_device = IsDevicePointer(dst->data);
   void* dst_d = dst->data;
   const std::size_t dst_elt = DtypeSize(dst->dtype);
   if (!dst_on_device) {
-    dst_d = ctx->workspace.Alloc(StorageElements(*dst) * dst_elt);
+    dst_d = ctx->ws->Alloc(StorageElements(*dst) * dst_elt);
     if (!dst_d) return Fail(ctx, RUYAMD_E_HIP, "device allocation for the destination failed");
   }
 
   MulCall call;
   call.lhs = ToDevMat(*lhs, lhs->data);
   call.rhs = ToDevMat(*rhs, rhs->data);
-  if (lhs->data && !IsDevicePointer(lhs->data))
-    call.lhs_host_bytes = StorageElements(*lhs) * DtypeSize(lhs->dtype);
-  if (rhs->data && !IsDevicePointer(rhs->data))
-    call.rhs_host_bytes = StorageElements(*rhs) * DtypeSize(rhs->dtype);
+  if (!lhs_dev) call.lhs_host_bytes = StorageElements(*lhs) * DtypeSize(lhs->dtype);
+  if (!rhs_dev) call.rhs_host_bytes = StorageElements(*rhs) * DtypeSize(rhs->dtype);
   call.dst = ToDevMat(*dst, dst_d);
   call.lhs_src_key = lhs->data;
   call.rhs_src_key = rhs->data;
@@ -274,6 +303,7 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
       err += " (the stream is capturing, so no memory can be allocated: run the same call once before the capture)";
     return Fail(ctx, rc, err);
   }
+  capture_scope.Recorded();
   staged = staged || call.staged_any;
 
   if (!dst_on_device) {
@@ -296,6 +326,16 @@ extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_m
   return RUYAMD_OK;
 }
 
+}  // namespace
+}  // namespace ruyamd
+
+using namespace ruyamd;
+
+extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
+                          const ruyamd_mul_params* p, const ruyamd_mat* dst) {
+  return MulImpl(ctx, lhs, rhs, p, dst, /*no_alloc=*/false);
+}
+
 extern "C" int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x, const int32_t* m,
                                        const int32_t* e, int32_t* out, int64_t n) {
   if (!ctx || n < 0) return RUYAMD_E_INVALID;
@@ -305,9 +345,9 @@ extern "C" int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x, const 
   ctx->workspace.Reset();
   bool staged = false, ok = true;
   const std::size_t bytes = std::size_t(n) * 4;
-  const int32_t* xd = static_cast<const int32_t*>(StageIn(ctx, x, bytes, &staged, &ok));
-  const int32_t* md = static_cast<const int32_t*>(StageIn(ctx, m, bytes, &staged, &ok));
-  const int32_t* ed = static_cast<const int32_t*>(StageIn(ctx, e, bytes, &staged, &ok));
+  const int32_t* xd = static_cast<const int32_t*>(StageIn(ctx, x, IsDevicePointer(x), bytes, &staged, &ok));
+  const int32_t* md = static_cast<const int32_t*>(StageIn(ctx, m, IsDevicePointer(m), bytes, &staged, &ok));
+  const int32_t* ed = static_cast<const int32_t*>(StageIn(ctx, e, IsDevicePointer(e), bytes, &staged, &ok));
   if (!ok) return Fail(ctx, RUYAMD_E_HIP, "staging failed");
   const bool out_dev = IsDevicePointer(out);
   int32_t* od = out_dev ? out : static_cast<int32_t*>(ctx->workspace.Alloc(bytes));

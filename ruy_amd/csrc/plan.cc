@@ -54,7 +54,7 @@ struct Operand8 {
 
 int MaterializeSums(ruyamd_ctx* ctx, Operand8* op, int32_t K, std::string* err) {
   if (!op->sums_pending) return RUYAMD_OK;
-  int32_t* sums = static_cast<int32_t*>(ctx->workspace.Alloc(std::size_t(op->count) * 4));
+  int32_t* sums = static_cast<int32_t*>(ctx->ws->Alloc(std::size_t(op->count) * 4));
   if (!sums) {
     *err = "workspace allocation failed";
     return RUYAMD_E_HIP;
@@ -71,8 +71,12 @@ int MaterializeSums(ruyamd_ctx* ctx, Operand8* op, int32_t K, std::string* err) 
 // While the stream records a graph the cache may neither allocate nor eject:
 // a hit is pinned (the recorded kernels keep reading its buffers on every
 // replay), a miss is an error.
+// A call that may not allocate only looks the entry up (and pins it when its
+// kernels are being recorded too); a miss there is no error: the operand is
+// then prepared in scratch memory for this call alone.
 PrepackedCache::Mode CacheMode(const ruyamd_ctx* ctx) {
-  return ctx->capturing ? PrepackedCache::Mode::kPinExisting : PrepackedCache::Mode::kInsertOnMiss;
+  if (ctx->capturing) return PrepackedCache::Mode::kPinExisting;
+  return ctx->no_alloc ? PrepackedCache::Mode::kLookupOnly : PrepackedCache::Mode::kInsertOnMiss;
 }
 const char kCaptureCacheMiss[] =
     "the stream is capturing and an operand with a cache policy is not in the prepacked cache yet: "
@@ -147,11 +151,11 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
     pm.layout.kernel_cols = 1;
     pm.zero_point = out->zero_point;
     const auto action = ctx->cache->Get(src_key, &pm, CacheMode(ctx));
-    if (action == PrepackedCache::Action::kMissing) {
+    if (action == PrepackedCache::Action::kMissing && !ctx->no_alloc) {
       *err = kCaptureCacheMiss;
       return RUYAMD_E_UNSUPPORTED;
     }
-    if (!pm.data) {
+    if (action != PrepackedCache::Action::kMissing && !pm.data) {
       *err = "device allocation for a cached packed matrix failed";
       return RUYAMD_E_HIP;
     }
@@ -169,11 +173,13 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
         return RUYAMD_E_HIP;
       }
     }
-    out->data = static_cast<const int8_t*>(pm.data);
-    out->ld = ld;
-    out->sums = pm.sums;
-    out->bytes = static_cast<uint32_t>(packed_bytes);
-    return RUYAMD_OK;
+    if (action != PrepackedCache::Action::kMissing) {
+      out->data = static_cast<const int8_t*>(pm.data);
+      out->ld = ld;
+      out->sums = pm.sums;
+      out->bytes = static_cast<uint32_t>(packed_bytes);
+      return RUYAMD_OK;
+    }
   }
 
   if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
@@ -195,8 +201,8 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
     return RUYAMD_OK;
   }
 
-  int8_t* packed = static_cast<int8_t*>(ctx->workspace.Alloc(packed_bytes ? packed_bytes : 16));
-  int32_t* sums = need_sums ? static_cast<int32_t*>(ctx->workspace.Alloc(std::size_t(src.count) * 4)) : nullptr;
+  int8_t* packed = static_cast<int8_t*>(ctx->ws->Alloc(packed_bytes ? packed_bytes : 16));
+  int32_t* sums = need_sums ? static_cast<int32_t*>(ctx->ws->Alloc(std::size_t(src.count) * 4)) : nullptr;
   if (!packed || (need_sums && !sums)) {
     *err = "workspace allocation failed";
     return RUYAMD_E_HIP;
@@ -225,11 +231,12 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
 void PlanDepthSplit(ruyamd_ctx* ctx, GemmKind kind, GemmArgs* args) {
   const DepthSplit split = GemmDepthSplit(*args, ctx->multiprocessor_count, kind);
   if (split.parts < 2) return;
-  void* partials = ctx->workspace.Alloc(split.partial_bytes);
+  void* partials = ctx->ws->Alloc(split.partial_bytes);
   if (!partials) return;
+  uint32_t* counters = ctx->split_counters;
   args->split_k = split.parts;
   args->split_partials = partials;
-  args->split_counters = ctx->split_counters;
+  args->split_counters = counters;
 }
 
 int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
@@ -417,11 +424,11 @@ int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy
     pm.layout.kernel_rows = 4;
     pm.layout.kernel_cols = 1;
     const auto action = ctx->cache->Get(src_key, &pm, CacheMode(ctx));
-    if (action == PrepackedCache::Action::kMissing) {
+    if (action == PrepackedCache::Action::kMissing && !ctx->no_alloc) {
       *err = kCaptureCacheMiss;
       return RUYAMD_E_UNSUPPORTED;
     }
-    if (!pm.data) {
+    if (action != PrepackedCache::Action::kMissing && !pm.data) {
       *err = "device allocation for a cached packed matrix failed";
       return RUYAMD_E_HIP;
     }
@@ -437,10 +444,12 @@ int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy
         return RUYAMD_E_HIP;
       }
     }
-    out->data = static_cast<const float*>(pm.data);
-    out->ld = ld;
-    out->bytes = static_cast<uint32_t>(packed_bytes);
-    return RUYAMD_OK;
+    if (action != PrepackedCache::Action::kMissing) {
+      out->data = static_cast<const float*>(pm.data);
+      out->ld = ld;
+      out->bytes = static_cast<uint32_t>(packed_bytes);
+      return RUYAMD_OK;
+    }
   }
   if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
   src = view();
@@ -454,7 +463,7 @@ int PrepareOperandF32(ruyamd_ctx* ctx, MulCall* call, int side, int cache_policy
     out->bytes = static_cast<uint32_t>(extent);
     return RUYAMD_OK;
   }
-  float* packed = static_cast<float*>(ctx->workspace.Alloc(packed_bytes ? packed_bytes : 16));
+  float* packed = static_cast<float*>(ctx->ws->Alloc(packed_bytes ? packed_bytes : 16));
   if (!packed) {
     *err = "workspace allocation failed";
     return RUYAMD_E_HIP;
@@ -585,7 +594,7 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     *err = "int16 operand too large for the matrix-core kernel";
     return RUYAMD_E_UNSUPPORTED;
   }
-  int8_t* planes = static_cast<int8_t*>(ctx->workspace.Alloc(packed_bytes));
+  int8_t* planes = static_cast<int8_t*>(ctx->ws->Alloc(packed_bytes));
   if (!planes) {
     *err = "workspace allocation failed";
     return RUYAMD_E_HIP;
@@ -635,7 +644,7 @@ int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
   DevMat& m = side == 0 ? call->lhs : call->rhs;
   std::size_t& bytes = side == 0 ? call->lhs_host_bytes : call->rhs_host_bytes;
   if (bytes == 0) return RUYAMD_OK;
-  void* d = ctx->workspace.Alloc(bytes);
+  void* d = ctx->ws->Alloc(bytes);
   if (!d || !ctx->staging.ToDevice(d, m.data, bytes, ctx->stream)) {
     *err = "staging a host operand to the device failed";
     return RUYAMD_E_HIP;
@@ -702,7 +711,7 @@ int RunTuned(ruyamd_ctx* ctx, MulCall* call, TunedPath path, std::string* err) {
       if (dst_col_major && call->dst.cols == 1) return RunGeneric(ctx, call, err);
       MulCall flipped = *call;
       DevMat& t = flipped.dst;
-      t.data = ctx->workspace.Alloc(std::size_t(t.rows) * t.cols * DtypeSize(t.dtype));
+      t.data = ctx->ws->Alloc(std::size_t(t.rows) * t.cols * DtypeSize(t.dtype));
       if (!t.data) {
         *err = "workspace allocation failed";
         return RUYAMD_E_HIP;
