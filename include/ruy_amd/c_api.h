@@ -148,6 +148,33 @@ RUYAMD_API int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs,
                           const ruyamd_mul_params* params,
                           const ruyamd_mat* dst);
 
+/* ruyamd_mul for callers that cannot allocate device memory: code whose
+ * stream is being captured into a graph, tight serving loops, harnesses that
+ * forbid hipMalloc. It has no counterpart in the reference. Same arguments,
+ * arithmetic and results as ruyamd_mul, with these differences:
+ *  - it calls no hipMalloc / hipFree / hipHostMalloc / event creation and no
+ *    other allocating routine. All scratch memory its kernels need (packed
+ *    operands, operand sums, the partial accumulators and arrival counters of
+ *    depth-split launches) comes from one static device array of
+ *    RUYAMD_NO_ALLOC_SCRATCH_BYTES that every GPU the library runs on holds
+ *    until the process ends;
+ *  - a call that needs more scratch than that fails with RUYAMD_E_UNSUPPORTED
+ *    and a message that says so (operands that are used in place - device
+ *    memory, depth-contiguous, 16-byte aligned, as in every benchmark
+ *    configuration - need none, whatever their size);
+ *  - every buffer must be device memory (RUYAMD_E_UNSUPPORTED otherwise);
+ *  - an operand with a cache policy is taken from the prepacked cache if it is
+ *    there and is otherwise prepared in the scratch area for this call only:
+ *    the cache is never inserted into; kernel timing skips these calls.
+ * All calls on one GPU, from any context, share that GPU's array: calls that
+ * overlap in time on one GPU race, so order them on one stream (or otherwise
+ * serialise them). The call may itself be recorded into a graph. */
+#define RUYAMD_NO_ALLOC_SCRATCH_BYTES (16u << 20)
+RUYAMD_API int ruyamd_mul_no_alloc(ruyamd_ctx* ctx, const ruyamd_mat* lhs,
+                                   const ruyamd_mat* rhs,
+                                   const ruyamd_mul_params* params,
+                                   const ruyamd_mat* dst);
+
 /* Stream control. By default a context owns a stream and every ruyamd_mul
  * synchronises it before returning, which is ruy::Mul's contract
  * (ruy/thread_pool.cc:239 waits for all workers). `ruyamd_ctx_set_stream`

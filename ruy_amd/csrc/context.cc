@@ -5,6 +5,7 @@
 #include <cstring>
 
 #include "kernels/gemm_i8.h"
+#include "kernels/static_scratch.h"
 
 namespace ruyamd {
 
@@ -296,6 +297,20 @@ int ruyamd_ctx_create(ruyamd_ctx** out) {
     delete ctx;
     return RUYAMD_E_HIP;
   }
+  // This GPU's static scratch area: the address is looked up here, with the
+  // device current, and kept; the array's name is never used as an address.
+  void* static_scratch = nullptr;
+  if (ruyamd::StaticScratchOfCurrentDevice(&static_scratch) != hipSuccess) {
+    (void)hipGetLastError();
+    DeviceFree(ctx->split_counters);
+    (void)hipStreamDestroy(ctx->own_stream);
+    delete ctx;
+    return RUYAMD_E_HIP;
+  }
+  static_assert(ruyamd::kStaticScratchCounterBytes >= 1024 * sizeof(uint32_t), "");
+  ctx->static_split_counters = static_cast<uint32_t*>(static_scratch);
+  ctx->static_workspace.UseFixed(static_cast<char*>(static_scratch) + ruyamd::kStaticScratchCounterBytes,
+                                 ruyamd::kStaticScratchBytes - ruyamd::kStaticScratchCounterBytes);
   ctx->cache = MakeCache(PrepackedCache::kDefaultMaxBuffersBytes);
   *out = ctx;
   return RUYAMD_OK;

@@ -13,6 +13,7 @@
 #include "context.h"
 #include "internal.h"
 #include "plan.h"
+#include "kernels/static_scratch.h"
 
 namespace ruyamd {
 namespace {
@@ -299,6 +300,14 @@ int MulImpl(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs, const
   std::string err;
   const int rc = RunMul(ctx, &call, &err);
   if (rc != RUYAMD_OK) {
+    if (no_alloc && ctx->ws->exhausted()) {
+      char msg[192];
+      std::snprintf(msg, sizeof(msg),
+                    "ruyamd_mul_no_alloc: this call needs more scratch memory than the %zu bytes of the "
+                    "static scratch area (packed operands, sums or partial accumulators); use ruyamd_mul",
+                    static_cast<std::size_t>(RUYAMD_NO_ALLOC_SCRATCH_BYTES));
+      return Fail(ctx, RUYAMD_E_UNSUPPORTED, msg);
+    }
     if (ctx->capturing && rc == RUYAMD_E_HIP)
       err += " (the stream is capturing, so no memory can be allocated: run the same call once before the capture)";
     return Fail(ctx, rc, err);
@@ -334,6 +343,11 @@ using namespace ruyamd;
 extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
                           const ruyamd_mul_params* p, const ruyamd_mat* dst) {
   return MulImpl(ctx, lhs, rhs, p, dst, /*no_alloc=*/false);
+}
+
+extern "C" int ruyamd_mul_no_alloc(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
+                                   const ruyamd_mul_params* p, const ruyamd_mat* dst) {
+  return MulImpl(ctx, lhs, rhs, p, dst, /*no_alloc=*/true);
 }
 
 extern "C" int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x, const int32_t* m,

@@ -4,6 +4,7 @@
 #include <cstdint>
 
 #include "kernels/gemm_i8.h"
+#include "kernels/static_scratch.h"
 
 namespace ruyamd {
 namespace {
@@ -234,6 +235,13 @@ void PlanDepthSplit(ruyamd_ctx* ctx, GemmKind kind, GemmArgs* args) {
   void* partials = ctx->ws->Alloc(split.partial_bytes);
   if (!partials) return;
   uint32_t* counters = ctx->split_counters;
+  if (ctx->no_alloc) {
+    // The static area is shared by every context on this GPU and keeps what the
+    // last call left there: the counters start from zero by a fill kernel of
+    // this call (the kernels leave them at zero too, unless a launch failed).
+    counters = ctx->static_split_counters;
+    if (LaunchFillZero(ctx->stream, counters, static_cast<uint32_t>(GemmDepthSplitCounters())) != hipSuccess) return;
+  }
   args->split_k = split.parts;
   args->split_partials = partials;
   args->split_counters = counters;
