@@ -7,47 +7,65 @@ A step is one ruyamd_mul call (through the C ABI) on seeded synthetic operands
 that are already resident in HBM. The headline workload is the int8 GEMM
 M=N=K=8192 with the full fused epilogue (zero points, int32 bias, fixed-point
 requantization to int8, clamp); the same run also measures the int8 GEMV
-M=K=16384, N=1 (prepacked-cache LHS, raw int32 destination) and reports it in
-the "gemv" object. One JSON line is printed:
+M=K=16384 (prepacked-cache LHS) and the remaining benchmark configurations.
+One JSON line is printed:
 
-  value     = 2*M*N*K / step time (the reference's own operation count,
-              ruy/benchmark.cc:199-200), wall clock around K steps
+  value     = 2*M*N*K / mean step time (the reference's own operation count,
+              ruy/benchmark.cc:199-200), wall clock around exactly K steps;
+              ms_per_step_min / _median come from HIP events between the steps
+              (the reference reports the minimum latency over repeats,
+              ruy/test.h:2082-2136)
+  settle_ms = after the W warm-up steps the same step keeps running until the
+              card's clock has settled under the load (at least 100 ms of
+              back-to-back steps, then until two windows of steps agree within
+              1 %); this many milliseconds of untimed steps preceded the K
+              timed ones
   roofline  = the dominant kernel against MI355X's published dense int8 MFMA
               peak (GEMM) or HBM peak (GEMV); its duration is measured with HIP
-              events around each launch on the launch stream
+              events around each launch on the launch stream.
+              frac_of_measured_ceiling relates the same rate to what a loop of
+              nothing but matrix instructions sustains on this card on random
+              operand bytes (ruyamd_diag_mfma_ceiling, measured in this run)
   cpu_baseline = the stock reference library (built from its own sources into
-              oracle/_ref) timed on this machine's host cores on a bounded
-              slice of the same workload; falls back to the C restatement
-              ("port") when that build is not present.
+              oracle/_ref) timed on this machine's host cores with the
+              reference's own method (minimum latency over repeats); falls
+              back to the C restatement ("port") when that build is absent.
+
+Every entry of `other_configs` (and `gemv`) carries its own roofline and
+cpu_baseline objects.
 """
 import argparse
 import ctypes as C
 import json
 import os
+import statistics
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X published dense int8 matrix peak, TOP/s
-HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E peak, GB/s
+INT8_MFMA_PEAK_TOPS = 5000.0   # MI355X published dense int8 matrix peak, TOP/s
+F32_MFMA_PEAK_TFLOPS = 157.3   # MI355X published dense fp32 matrix peak, TFLOP/s
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak, GB/s
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # The card's clock takes about 50 ms of load to settle after an idle period
-    # (the 8192^3 step measures 5 % slower in the first tens of steps), so the
-    # default warm-up is long enough to time the sustained rate.
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all", choices=["all", "gemm", "gemv", "shape", "mfma-ceiling"])
     ap.add_argument("--shape", default="256,8192,256",
                     help="M,K,N of --workload shape: the int8 GEMM configuration at another shape "
                          "(for profiles of the smaller tiles; not part of the default run)")
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the int8 GEMM")
     ap.add_argument("--gemv-size", type=int, default=16384, help="M=K of the int8 GEMV")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="diagnostic for --workload gemm / shape: all-zero operand values, on which the card "
+                         "does not run into its power limit (not a valid benchmark figure)")
+    ap.add_argument("--no-settle", action="store_true",
+                    help="time the K steps right after the W warm-up steps (no settling period)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the HIP-graph replay timing of the small configurations")
@@ -62,29 +80,64 @@ def device_problem(problem):
     return D.DeviceProblem(problem, dst_fill=0)
 
 
-def time_steps(run, steps, warmup, ctx):
+SETTLE_MIN_MS = 100.0
+SETTLE_MAX_MS = 1500.0
+
+
+def time_steps(run, steps, warmup, ctx, settle=True, events_every=1):
+    """W warm-up steps, a settling period, then exactly `steps` timed steps.
+
+    Returns a dict: step_s (mean, wall clock between two synchronisations),
+    step_min_s / step_median_s (from HIP events recorded on the launch stream
+    every `events_every` steps), kernel_ms (mean per launch, from the library's
+    per-launch events; None if kernel timing is off), region_ms (events around
+    all timed steps, per step) and settle_ms."""
     import torch
     for _ in range(warmup):
         run()
     torch.cuda.synchronize()
-    ctx.kernel_timing()  # drop the warm-up launches
+    settle_ms = 0.0
+    if settle:
+        # Windows of back-to-back steps, each timed with one event pair.
+        window = max(10, min(steps, 50))
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        previous = None
+        while settle_ms < SETTLE_MAX_MS:
+            e0.record()
+            for _ in range(window):
+                run()
+            e1.record()
+            e1.synchronize()
+            ms = e0.elapsed_time(e1)
+            settle_ms += ms
+            agree = previous is not None and abs(ms - previous) <= 0.01 * previous
+            previous = ms
+            if settle_ms >= SETTLE_MIN_MS and agree:
+                break
+    ctx.kernel_timing()  # drop the warm-up and settling launches
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
+    events_every = max(1, min(events_every, steps))
+    n_marks = steps // events_every + 1
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(n_marks)]
     t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
+    marks[0].record()
+    for i in range(steps):
         run()
-    e1.record()
+        if (i + 1) % events_every == 0:
+            marks[(i + 1) // events_every].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    region_ms = e0.elapsed_time(e1) / steps  # events on the launch stream around all K steps
+    per = [marks[i].elapsed_time(marks[i + 1]) / events_every for i in range(n_marks - 1)]
+    region_ms = marks[0].elapsed_time(marks[n_marks - 1]) / ((n_marks - 1) * events_every)
     kernel_ms, launches = ctx.kernel_timing()
-    return wall / steps, (kernel_ms / launches if launches else None), region_ms
+    return {"step_s": wall / steps, "step_min_s": min(per) * 1e-3, "step_median_s": statistics.median(per) * 1e-3,
+            "kernel_ms": kernel_ms / launches if launches else None, "region_ms": region_ms,
+            "settle_ms": settle_ms}
 
 
 def load_traffic(name):
-    """Measured HBM bytes per launch, recorded from rocprofv3 --pmc runs."""
+    """Measured HBM bytes per launch, recorded from rocprofv3 --pmc runs (profiles/traffic.json)."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
@@ -93,71 +146,116 @@ def load_traffic(name):
         return None
 
 
-def cpu_baseline_gemm(problem, n_slice):
-    """Stock ruy on the host cores over the first n_slice RHS columns."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import oracle_lib as O
-    from ruy_amd import workloads as W
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
-    sub = W.Problem(problem.name, problem.lhs,
-                    W.HostMatrix(problem.rhs.dtype, problem.K, n_slice, problem.rhs.order,
-                                 stride=problem.rhs.stride, zero_point=problem.rhs.zero_point,
-                                 storage=problem.rhs.storage),
-                    W.HostMatrix(problem.dst.dtype, problem.M, n_slice, problem.dst.order,
-                                 zero_point=problem.dst.zero_point),
-                    problem.accum_dtype, bias=problem.bias,
-                    multiplier_fixedpoint=problem.multiplier_fixedpoint,
-                    multiplier_exponent=problem.multiplier_exponent,
-                    clamp_min=problem.clamp_min, clamp_max=problem.clamp_max)
-    ops = 2.0 * sub.M * sub.N * sub.K
-    sample = "first %d of %d rhs columns (M=%d, K=%d)" % (n_slice, problem.N, sub.M, sub.K)
-    if O.stock is not None:
-        l, r, d = sub.lhs.struct(), sub.rhs.struct(), sub.dst.struct()
-        p = sub.params_struct()
-        lat, used = C.c_double(0), C.c_int(0)
-        rc = O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, cores,
-                                         2.0, 2, C.byref(lat), C.byref(used))
-        if rc == 0 and lat.value > 0:
-            out = {"value": ops / lat.value / 1e12, "unit": "TOP/s", "cores": cores,
-                   "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
-            # ruy never picks a thread count itself (ruy/context.h:68-73): also one thread.
-            lat1 = C.c_double(0)
-            if O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, 1,
-                                           1.0, 1, C.byref(lat1), C.byref(used)) == 0 and lat1.value > 0:
-                out["value_1_thread"] = ops / lat1.value / 1e12
-            return out
-    t0 = time.perf_counter()
-    O.oracle_mul(sub)
-    dt = time.perf_counter() - t0
-    return {"value": ops / dt / 1e12, "unit": "TOP/s", "cores": cores, "kind": "port",
-            "sample": sample + ", C restatement with OpenMP"}
+# --------------------------------------------------------------------------
+# Host-CPU baseline: stock ruy, timed the reference's way.
+# --------------------------------------------------------------------------
+
+def host_threads():
+    """Threads for the multi-threaded baseline: the physical cores this process
+    may use. ruy never picks a thread count itself (ruy/context.h:68-73), so
+    the count is stated with every figure."""
+    physical = set()
+    try:
+        pkg = core = None
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("physical id"):
+                    pkg = line.split(":")[1].strip()
+                elif line.startswith("core id"):
+                    core = line.split(":")[1].strip()
+                elif not line.strip():
+                    if core is not None:
+                        physical.add((pkg, core))
+                    pkg = core = None
+    except OSError:
+        pass
+    detected = len(physical) or (os.cpu_count() or 1)
+    try:
+        affinity = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        affinity = os.cpu_count() or 1
+    # The share of the machine this job was given, where the environment says so.
+    share = None
+    try:
+        share = int(os.environ.get("OMP_NUM_THREADS", "")) or None
+    except ValueError:
+        pass
+    used = min(x for x in (detected, affinity, share) if x)
+    return {"threads": used, "detected_physical_cores": detected, "affinity_cpus": affinity,
+            "job_cpu_share": share}
 
 
-def cpu_baseline_gemv(problem):
+def _oracle():
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib as O
-    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
-    nbytes = problem.algorithmic_bytes()
-    sample = "full %dx%d weight, N=%d, LHS kAlwaysCache (warm)" % (problem.M, problem.K, problem.N)
+    return O
+
+
+def cpu_baseline(problem, work, unit, sample, min_secs=0.5, repeats=2):
+    """Stock ruy on `problem` (host memory): `work` / latency in `unit`
+    (work is operations for "TOP/s" / "TFLOP/s", bytes for "GB/s")."""
+    O = _oracle()
+    scale = 1e9 if unit == "GB/s" else 1e12
+    host = host_threads()
+    threads = host["threads"]
     if O.stock is not None:
         l, r, d = problem.lhs.struct(), problem.rhs.struct(), problem.dst.struct()
         p = problem.params_struct()
         lat, used = C.c_double(0), C.c_int(0)
-        rc = O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, cores,
-                                         1.0, 3, C.byref(lat), C.byref(used))
+        rc = O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, threads,
+                                         min_secs, repeats, C.byref(lat), C.byref(used))
         if rc == 0 and lat.value > 0:
-            out = {"value": nbytes / lat.value / 1e9, "unit": "GB/s", "cores": cores,
-                   "kind": "reference", "sample": sample + ", stock ruy path 0x%x" % used.value}
+            out = {"value": work / lat.value / scale, "unit": unit, "cores": threads, "kind": "reference",
+                   "sample": sample + "; stock ruy path 0x%x, min latency over %d x %.1f s of calls "
+                             "(ruy/test.h:2082-2136)" % (used.value, repeats, min_secs),
+                   "ms_per_call": lat.value * 1e3}
             lat1 = C.c_double(0)
             if O.stock.stock_ruy_benchmark(C.byref(l), C.byref(r), C.byref(p), C.byref(d), 0, 1,
-                                           1.0, 1, C.byref(lat1), C.byref(used)) == 0 and lat1.value > 0:
-                out["value_1_thread"] = nbytes / lat1.value / 1e9
+                                           min_secs, 1, C.byref(lat1), C.byref(used)) == 0 and lat1.value > 0:
+                out["value_1_thread"] = work / lat1.value / scale
             return out
     t0 = time.perf_counter()
     O.oracle_mul(problem)
     dt = time.perf_counter() - t0
-    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": sample + ", C restatement with OpenMP"}
+    return {"value": work / dt / scale, "unit": unit, "cores": threads, "kind": "port",
+            "sample": sample + "; C restatement with OpenMP, one call"}
+
+
+def gemm_slice(problem, n_slice):
+    """The first n_slice RHS (and destination) columns of `problem`: a bounded
+    sample of a GEMM that is too long for a CPU baseline at full size."""
+    from ruy_amd import workloads as W
+    return W.Problem(problem.name, problem.lhs,
+                     W.HostMatrix(problem.rhs.dtype, problem.K, n_slice, problem.rhs.order,
+                                  stride=problem.rhs.stride, zero_point=problem.rhs.zero_point,
+                                  storage=problem.rhs.storage),
+                     W.HostMatrix(problem.dst.dtype, problem.M, n_slice, problem.dst.order,
+                                  zero_point=problem.dst.zero_point),
+                     problem.accum_dtype, bias=problem.bias,
+                     multiplier_fixedpoint=problem.multiplier_fixedpoint,
+                     multiplier_exponent=problem.multiplier_exponent,
+                     clamp_min=problem.clamp_min, clamp_max=problem.clamp_max)
+
+
+# --------------------------------------------------------------------------
+# Workloads
+# --------------------------------------------------------------------------
+
+def bench_mfma_ceiling(ctx, settle_ms=150.0, only_best=False):
+    """What the bare int8 matrix-instruction loop sustains on this card
+    (ruyamd_diag_mfma_ceiling): both instruction shapes, fragments kept in
+    registers or re-read from LDS, all-zero or uniformly random operands."""
+    out = []
+    combos = [(1, 0, 1)] if only_best else [(i, l, r) for i in (0, 1) for l in (0, 1) for r in (0, 1)]
+    names = ("v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8")
+    for instruction, from_lds, random_operands in combos:
+        tops, ms = ctx.mfma_ceiling(instruction, from_lds, random_operands, settle_ms)
+        out.append({"instruction": names[instruction],
+                    "fragments": "lds + barrier" if from_lds else "registers",
+                    "operands": "random bytes" if random_operands else "zero",
+                    "TOP/s": tops, "frac_of_peak": tops / INT8_MFMA_PEAK_TOPS,
+                    "ms_per_launch": ms})
+    return out
 
 
 def bench_gemm(ctx, args):
@@ -165,26 +263,43 @@ def bench_gemm(ctx, args):
     n = args.size
     problem = W.config_int8_gemm(n, config_id=6, name="int8_gemm_%d" % n)
     dp = device_problem(problem)
+    if args.zero_operands:
+        dp.lhs_t.zero_()
+        dp.rhs_t.zero_()
     dp.run(ctx)
     kernel = ctx.last_kernel_name()
-    step_s, kernel_ms, _ = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx)
+    t = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx, settle=not args.no_settle)
     ops = float(problem.ops())
+    kernel_ms = t["kernel_ms"]
+    achieved = ops / (kernel_ms * 1e-3) / 1e12 if kernel_ms else None
+    ceiling = bench_mfma_ceiling(ctx, only_best=True)[0]
     out = {
-        "value": ops / step_s / 1e12,
-        "ms_per_step": step_s * 1e3,
+        "value": ops / t["step_s"] / 1e12,
+        "ms_per_step": t["step_s"] * 1e3,
+        "ms_per_step_min": t["step_min_s"] * 1e3,
+        "ms_per_step_median": t["step_median_s"] * 1e3,
+        "settle_ms": t["settle_ms"],
         "kernel": kernel,
         "roofline": {
             "bound": "mfma",
-            "achieved": ops / (kernel_ms * 1e-3) / 1e12 if kernel_ms else None,
+            "achieved": achieved,
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TOP/s",
-            "frac": ops / (kernel_ms * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS if kernel_ms else None,
+            "frac": achieved / INT8_MFMA_PEAK_TOPS if achieved else None,
             "traffic": load_traffic("int8_gemm_%d" % n),
             "kernel_ms": kernel_ms,
+            "measured_ceiling": {"TOP/s": ceiling["TOP/s"],
+                                 "what": "%s on fragments held in registers, random operand bytes, no memory "
+                                         "traffic, measured in this run" % ceiling["instruction"]},
+            "frac_of_measured_ceiling": achieved / ceiling["TOP/s"] if achieved else None,
         },
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_gemm(problem, min(n, 512))
+        n_slice = min(n, 512)
+        sub = gemm_slice(problem, n_slice)
+        out["cpu_baseline"] = cpu_baseline(
+            sub, 2.0 * sub.M * sub.N * sub.K, "TOP/s",
+            "first %d of %d rhs columns (M=%d, K=%d)" % (n_slice, problem.N, sub.M, sub.K), min_secs=2.0)
     return problem, out
 
 
@@ -194,27 +309,15 @@ def bench_shape(ctx, args):
     M, K, N = (int(x) for x in args.shape.split(","))
     problem = W.config_int8_gemm_shape(M, K, N)
     dp = device_problem(problem)
+    if args.zero_operands:
+        dp.lhs_t.zero_()
+        dp.rhs_t.zero_()
     dp.run(ctx)
-    step_s, kernel_ms, _ = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx)
-    return {"shape": [M, K, N], "kernel": ctx.last_kernel_name(), "us_per_step": step_s * 1e6,
-            "kernel_us": kernel_ms * 1e3 if kernel_ms else None, "Top/s": problem.ops() / step_s / 1e12}
-
-
-def bench_mfma_ceiling(ctx, settle_ms=150.0):
-    """What the bare int8 matrix-instruction loop sustains on this card
-    (ruyamd_diag_mfma_ceiling): both instruction shapes, fragments kept in
-    registers or re-read from LDS, all-zero or uniformly random operands."""
-    out = []
-    for instruction, name in ((0, "v_mfma_i32_32x32x32_i8"), (1, "v_mfma_i32_16x16x64_i8")):
-        for from_lds in (0, 1):
-            for random_operands in (0, 1):
-                tops, ms = ctx.mfma_ceiling(instruction, from_lds, random_operands, settle_ms)
-                out.append({"instruction": name,
-                            "fragments": "lds + barrier" if from_lds else "registers",
-                            "operands": "random bytes" if random_operands else "zero",
-                            "TOP/s": tops, "frac_of_peak": tops / INT8_MFMA_PEAK_TOPS,
-                            "ms_per_launch": ms})
-    return out
+    t = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx, settle=not args.no_settle)
+    return {"shape": [M, K, N], "kernel": ctx.last_kernel_name(), "us_per_step": t["step_s"] * 1e6,
+            "us_per_step_min": t["step_min_s"] * 1e6,
+            "kernel_us": t["kernel_ms"] * 1e3 if t["kernel_ms"] else None,
+            "Top/s": problem.ops() / t["step_s"] / 1e12}
 
 
 def bench_gemm_host_buffers(ctx, problem, steps=3):
@@ -257,6 +360,12 @@ def api_lib():
     return api.lib
 
 
+def hbm_roofline(nbytes, kernel_ms, traffic):
+    rate = nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None
+    return {"bound": "hbm", "achieved": rate, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": rate / HBM_PEAK_GBS if rate else None, "traffic": traffic, "kernel_ms": kernel_ms}
+
+
 def bench_gemv(ctx, args):
     """int8 GEMV with a prepacked-cache LHS. The 256 MiB weight is about the
     size of the 256 MB Infinity Cache, so the step rotates over four distinct
@@ -281,34 +390,35 @@ def bench_gemv(ctx, args):
     # and that kernel is short enough for a per-launch event pair to add ~10 %
     # to it; so per-launch events are switched off and its duration is taken
     # from one event pair around all launches of the timed region.
+    settle = not args.no_settle
     ctx.set_kernel_timing(False)
-    step_s, _, kernel_ms = time_steps(run, args.steps * 4, args.warmup * 4, ctx)
-    ctx.set_kernel_timing(True)
+    t = time_steps(run, args.steps * 4, args.warmup * 4, ctx, settle=settle, events_every=4)
     nbytes = float(problems[0].algorithmic_bytes())
     out = {
         "metric": "int8 GEMV M=K=%d N=1 algorithmic HBM GB/s" % n,
-        "value": nbytes / step_s / 1e9,
+        "value": nbytes / t["step_s"] / 1e9,
         "unit": "GB/s",
-        "ms_per_step": step_s * 1e3,
+        "ms_per_step": t["step_s"] * 1e3,
+        "ms_per_step_min": t["step_min_s"] * 1e3,
+        "ms_per_step_median": t["step_median_s"] * 1e3,
+        "settle_ms": t["settle_ms"],
         "kernel": kernel,
         "algorithmic_bytes": nbytes,
-        "roofline": {
-            "bound": "hbm",
-            "achieved": nbytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms else None,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": nbytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if kernel_ms else None,
-            "traffic": load_traffic("int8_gemv_%d_n1" % n),
-            "kernel_ms": kernel_ms,
-        },
+        "roofline": hbm_roofline(nbytes, t["region_ms"], load_traffic("int8_gemv_%d_n1" % n)),
     }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(
+            problems[0], nbytes, "GB/s",
+            "full %dx%d weight, N=1, LHS kAlwaysCache (warm)" % (n, n), min_secs=1.0)
     # The same weights against 4 and 8 activation vectors (the skinny kernel on
-    # the matrix cores), reusing the cache entries made above.
-    out["more_columns"] = []
-    for cols in (4, 8):
+    # the matrix cores) and the requantized N=1 run, reusing the cache entries.
+    out["more_runs"] = []
+    variants = [("N=4, raw int32 dst", dict(N=4)), ("N=8, raw int32 dst", dict(N=8)),
+                ("N=1, int8 dst (multiplier 2^30 * 2^-10)", dict(N=1, requant=True))]
+    for label, kw in variants:
         wider = []
         for base_problem, base_dp in zip(problems, dps):
-            p = W.config_int8_gemv(n, cols, lhs=base_problem.lhs)
+            p = W.config_int8_gemv(n, lhs=base_problem.lhs, **kw)
             dp = device_problem(p)
             dp.lhs_t = base_dp.lhs_t  # same device weights, hence the same cache entry
             dp.lhs_s = p.lhs.struct(base_dp.lhs_t.data_ptr())
@@ -321,43 +431,69 @@ def bench_gemv(ctx, args):
 
         run_wider()
         kernel_wider = ctx.last_kernel_name()
-        ctx.set_kernel_timing(False)
-        step_w, _, kernel_ms_w = time_steps(run_wider, args.steps * 4, args.warmup * 4, ctx)
-        ctx.set_kernel_timing(True)
+        tw = time_steps(run_wider, args.steps * 4, args.warmup * 4, ctx, settle=False, events_every=4)
         nbytes_w = float(wider[0].problem.algorithmic_bytes())
-        out["more_columns"].append({
-            "N": cols, "kernel": kernel_wider, "ms_per_step": step_w * 1e3, "kernel_ms": kernel_ms_w,
-            "algorithmic_bytes": nbytes_w, "GB/s": nbytes_w / (kernel_ms_w * 1e-3) / 1e9,
-            "frac": nbytes_w / (kernel_ms_w * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "traffic": load_traffic("int8_gemv_%d_n%d" % (n, cols))})
+        cols = kw["N"]
+        entry = {"run": label, "N": cols, "kernel": kernel_wider, "ms_per_step": tw["step_s"] * 1e3,
+                 "ms_per_step_min": tw["step_min_s"] * 1e3, "algorithmic_bytes": nbytes_w,
+                 "roofline": hbm_roofline(nbytes_w, tw["region_ms"],
+                                          None if kw.get("requant") else load_traffic("int8_gemv_%d_n%d" % (n, cols)))}
+        if not args.no_cpu_baseline:
+            entry["cpu_baseline"] = cpu_baseline(
+                wider[0].problem, nbytes_w, "GB/s",
+                "full %dx%d weight, %s, LHS kAlwaysCache (warm)" % (n, n, label), min_secs=0.5, repeats=1)
+        out["more_runs"].append(entry)
         del wider
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_gemv(problems[0])
+    ctx.set_kernel_timing(True)
     del dps
     ctx.clear_prepacked_cache()
     torch.cuda.empty_cache()
     return out
 
 
-def bench_other_configs(ctx, steps, warmup, with_graph=True):
-    """Time (not roofline) of the remaining configurations: small or
-    latency-bound shapes whose gate is parity; reported for completeness."""
+def bench_other_configs(ctx, args):
+    """The remaining benchmark configurations, each with its time per call
+    (mean, min and median over batches of calls), its roofline object (kernel
+    time from HIP events around back-to-back launches) and stock ruy on the
+    host cores at the full shape."""
     from ruy_amd import workloads as W
     out = []
     ctx.set_kernel_timing(False)  # a per-launch event pair would dominate these short steps
-    for name, problem in [("C1 int8 256^3", W.config_int8_gemm(256)),
-                          ("C2 fp32 1024^3", W.config_f32_gemm(1024)),
-                          ("C2 fp32 1024^3 relu6", W.config_f32_gemm(1024, relu6=True)),
-                          ("C3 int8 per-channel 1024x1024x196", W.config_int8_perchannel_conv()),
-                          ("C4 int8xint16 2048x2048x512", W.config_int8_int16())]:
+    configs = [
+        ("C1 int8 256^3", W.config_int8_gemm(256), "mfma-int8",
+         "launch-bound: 33.6 Mop in one launch, smaller than the time to start a kernel"),
+        ("C2 fp32 1024^3", W.config_f32_gemm(1024), "mfma-f32", None),
+        ("C2 fp32 1024^3 relu6", W.config_f32_gemm(1024, relu6=True), "mfma-f32", None),
+        ("C3 int8 per-channel 1024x1024x196", W.config_int8_perchannel_conv(), "mfma-int8",
+         "launch-bound: 0.41 Gop, 64 tiles of 64x64 for 256 CUs"),
+        ("C4 int8xint16 2048x2048x512", W.config_int8_int16(), "mfma-int8",
+         "operations counted once although the int16 operand takes two int8 matrix-instruction passes"),
+    ]
+    for name, problem, bound, note in configs:
         dp = device_problem(problem)
         dp.run(ctx)
         kernel = ctx.last_kernel_name()
-        step_s, _, _ = time_steps(lambda: dp.run(ctx), steps, warmup, ctx)
-        entry = {"config": name, "kernel": kernel, "us_per_step": step_s * 1e6,
-                 "Top/s": problem.ops() / step_s / 1e12}
-        if with_graph and problem.ops() < 1e9:
+        t = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx, settle=False, events_every=10)
+        ops = float(problem.ops())
+        fp = bound == "mfma-f32"
+        peak = F32_MFMA_PEAK_TFLOPS if fp else INT8_MFMA_PEAK_TOPS
+        unit = "TFLOP/s" if fp else "TOP/s"
+        # Back-to-back asynchronous calls: the events around the region see the
+        # kernels (and, for a call of several launches, the gaps between them).
+        achieved = ops / (t["region_ms"] * 1e-3) / 1e12
+        entry = {"config": name, "kernel": kernel, "us_per_step": t["step_s"] * 1e6,
+                 "us_per_step_min": t["step_min_s"] * 1e6, "us_per_step_median": t["step_median_s"] * 1e6,
+                 unit: ops / t["step_s"] / 1e12,
+                 "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": unit,
+                              "frac": achieved / peak, "traffic": None, "kernel_ms": t["region_ms"],
+                              "kernel_ms_is": "stream time per call over back-to-back calls (all launches of a call)"}}
+        if note:
+            entry["roofline"]["note"] = note
+        if not args.no_graph and problem.ops() < 1e9:
             entry["us_per_step_graph"] = graph_replay_us(ctx, dp)
+        if not args.no_cpu_baseline:
+            entry["cpu_baseline"] = cpu_baseline(problem, ops, unit, "full shape M=%d K=%d N=%d" % (
+                problem.M, problem.K, problem.N), min_secs=0.5, repeats=2)
         out.append(entry)
     ctx.set_kernel_timing(True)
     return out
@@ -422,6 +558,11 @@ def main():
         "dtype": "int8",
         "data": "synthetic (SplitMix64-seeded uniform int8, random int32 bias)",
     }
+    if args.zero_operands:
+        line["data"] = "DIAGNOSTIC: all-zero operands (no power limit), not a benchmark figure"
+    if not args.no_cpu_baseline:
+        # How the thread count of every cpu_baseline ("cores") was arrived at.
+        line["host_cpu"] = host_threads()
     if args.workload == "mfma-ceiling":
         rows = bench_mfma_ceiling(ctx)
         best_random = max(r["TOP/s"] for r in rows if r["operands"] == "random bytes")
@@ -441,8 +582,8 @@ def main():
         return
     if args.workload in ("all", "gemm"):
         problem, g = bench_gemm(ctx, args)
-        line.update({"value": g["value"], "ms_per_step": g["ms_per_step"],
-                     "roofline": g["roofline"]})
+        for key in ("value", "ms_per_step", "ms_per_step_min", "ms_per_step_median", "settle_ms", "roofline"):
+            line[key] = g[key]
         if "cpu_baseline" in g:
             line["cpu_baseline"] = g["cpu_baseline"]
         if args.workload == "all":
@@ -457,15 +598,17 @@ def main():
         gv = bench_gemv(ctx, args)
         if args.workload == "gemv":
             line.update({"metric": gv["metric"], "unit": "GB/s", "value": gv["value"],
-                         "ms_per_step": gv["ms_per_step"], "roofline": gv["roofline"],
+                         "ms_per_step": gv["ms_per_step"], "ms_per_step_min": gv["ms_per_step_min"],
+                         "ms_per_step_median": gv["ms_per_step_median"], "settle_ms": gv["settle_ms"],
+                         "roofline": gv["roofline"],
                          "config": {"workload": gv["metric"], "kernel": gv["kernel"]},
-                         "more_columns": gv.get("more_columns")})
+                         "more_runs": gv.get("more_runs")})
             if "cpu_baseline" in gv:
                 line["cpu_baseline"] = gv["cpu_baseline"]
         else:
             line["gemv"] = gv
     if args.workload == "all":
-        line["other_configs"] = bench_other_configs(ctx, args.steps, args.warmup, not args.no_graph)
+        line["other_configs"] = bench_other_configs(ctx, args)
     if args.copy_calibration:
         a = torch.full((256 << 20,), 3, dtype=torch.uint8, device="cuda")
         b = torch.empty_like(a)

@@ -9,7 +9,8 @@ import os
 from . import _structs as S
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libruy_amd.so")
+# RUY_AMD_LIBRARY names another build of the same library (e.g. an experimental one).
+LIB_PATH = os.environ.get("RUY_AMD_LIBRARY") or os.path.join(_HERE, "libruy_amd.so")
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
