@@ -175,6 +175,34 @@ static int32_t int_epilogue(int32_t accum, int i, int j,
   return accum;
 }
 
+/* The part of ruy/reference_mul.h:42-49 that follows the bias: multiplier,
+ * destination zero point, clamp (min first, then max), cast. `raw` holds int32
+ * accumulators that already include the bias and every zero-point term - what
+ * ruy::Mul itself writes into an int32 destination, on which all of its paths
+ * agree exactly (ruy/test.h:1392-1395). */
+int oracle_requantize_i32(const oracle_mat* raw, const oracle_mul_params* p,
+                          const oracle_mat* dst) {
+  if (!raw || !p || !dst || raw->dtype != ORACLE_I32 || !is_int_dtype(dst->dtype) ||
+      raw->rows != dst->rows || raw->cols != dst->cols)
+    return 1;
+  oracle_mul_params no_bias = *p;
+  no_bias.bias = NULL;
+  const int M = dst->rows, N = dst->cols;
+  /* Walk the destination along its contiguous dimension. */
+  const int outer = dst->order == ORACLE_COL_MAJOR ? N : M;
+  const int inner = dst->order == ORACLE_COL_MAJOR ? M : N;
+#pragma omp parallel for schedule(static)
+  for (int o = 0; o < outer; o++) {
+    for (int n = 0; n < inner; n++) {
+      const int i = dst->order == ORACLE_COL_MAJOR ? n : o;
+      const int j = dst->order == ORACLE_COL_MAJOR ? o : n;
+      const int32_t accum = ((const int32_t*)raw->data)[mat_offset(raw, i, j)];
+      store_int_dst(dst, i, j, int_epilogue(accum, i, j, &no_bias, dst));
+    }
+  }
+  return 0;
+}
+
 /* Wrapping dot product of two int16 vectors, widened to int32. The operands
  * hold (value - zero_point), which fits int16 for every legal combination:
  * 8-bit types give [-255, 255], int16 operands require zero_point == 0. */

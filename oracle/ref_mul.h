@@ -15,6 +15,11 @@
  *   oracle_mul         ReferenceMul  ruy/reference_mul.h:29-52
  *                      (element addressing ruy/matrix.h:188-199,
  *                       multiplier selection ruy/apply_multiplier.h:67-79)
+ *   oracle_requantize_i32  the tail of ReferenceMul after the bias,
+ *                      ruy/reference_mul.h:44-49, over a matrix of int32
+ *                      accumulators (for shapes too large for oracle_mul: the
+ *                      accumulators come from stock ruy's fastest path, which
+ *                      is exact for an int32 destination, ruy/test.h:1392-1395)
  *   oracle_validate    ValidateZeroPoints  ruy/validate.h:40-75
  *   oracle_pack_sums   generic PackImpl::Run  ruy/pack.h:105-132 with the
  *                      uint8->int8 conversion of ruy/pack_common.h:36-58
@@ -33,6 +38,12 @@
  *                       invariance under storage order / stride / transposed
  *                       problem; stock ruy (oracle/_ref, Path::kStandardCpp and
  *                       ReferenceMul) when that build is present.
+ *   oracle_requantize_i32 - shares int_epilogue() with oracle_mul, so the
+ *                       known answers above pin its arithmetic; its own
+ *                       indexing is pinned by oracle_requantize_i32(oracle_mul
+ *                       into int32) == oracle_mul into the narrow type, over
+ *                       type tuples, storage orders, strides and both channel
+ *                       dimensions, and by stock ReferenceMul where built.
  *   oracle_pack_sums,
  *   oracle_mul_packed - identity with oracle_mul (ruy/kernel.h:224-232 is
  *                       algebraically reference_mul.h:38 mod 2^32).
@@ -99,6 +110,15 @@ int oracle_validate(const oracle_mat* lhs, const oracle_mat* rhs,
 int oracle_mul(const oracle_mat* lhs, const oracle_mat* rhs,
                const oracle_mul_params* params, const oracle_mat* dst,
                int* overflow);
+
+/* ruy/reference_mul.h:44-49 applied to every element of `raw`, an int32
+ * matrix of accumulators that already include the bias: multiplier (scalar or
+ * per channel), destination zero point, clamp, cast into `dst` (same shape,
+ * any order and stride, uint8 / int8 / int16 / int32). `params->bias` is
+ * ignored. Returns 0 on success. */
+int oracle_requantize_i32(const oracle_mat* raw,
+                          const oracle_mul_params* params,
+                          const oracle_mat* dst);
 
 /* ruy/pack.h:105-132 for an integer source: `src` is the matrix whose COLUMNS
  * are packed (the transposed LHS, or the RHS), `depth_padded` >= src->rows and

@@ -181,6 +181,7 @@ int Dispatch(const oracle_mat* lhs, const oracle_mat* rhs,
   TUPLE(ORACLE_I8, int8_t, ORACLE_I8, int8_t, ORACLE_I32, int32_t, ORACLE_I32, int32_t)
   TUPLE(ORACLE_U8, uint8_t, ORACLE_U8, uint8_t, ORACLE_I32, int32_t, ORACLE_I32, int32_t)
   TUPLE(ORACLE_I8, int8_t, ORACLE_U8, uint8_t, ORACLE_I32, int32_t, ORACLE_I32, int32_t)
+  TUPLE(ORACLE_U8, uint8_t, ORACLE_I8, int8_t, ORACLE_I32, int32_t, ORACLE_I32, int32_t)
   TUPLE(ORACLE_I8, int8_t, ORACLE_I16, int16_t, ORACLE_I32, int32_t, ORACLE_I16, int16_t)
   TUPLE(ORACLE_I16, int16_t, ORACLE_I8, int8_t, ORACLE_I32, int32_t, ORACLE_I16, int16_t)
 #undef TUPLE

@@ -82,12 +82,24 @@ def build_cpp_tests(verbose=True):
          os.path.join(tdir, "api_test.cc"), "-L" + HERE, "-lruy_amd",
          "-Wl,-rpath,$ORIGIN/../../ruy_amd", "-o", os.path.join(tdir, "api_test")],
     ]
+    built = ["tests/cpp/prepacked_cache_test", "tests/cpp/api_test"]
+    # The reference's own example programs, compiled unchanged from where they
+    # lie against this library's ruy:: headers (only where the reference tree is
+    # present; the binaries are build artefacts like the library itself).
+    reference = os.environ.get("RUY_REFERENCE", "/root/reference")
+    for name in ("example", "parametrized_example"):
+        src = os.path.join(reference, "example", name + ".cc")
+        if os.path.exists(src):
+            cmds.append(["g++", "-std=c++14", "-O1", "-I" + os.path.join(ROOT, "include"), src, "-L" + HERE,
+                         "-lruy_amd", "-Wl,-rpath,$ORIGIN/../../ruy_amd", "-o",
+                         os.path.join(tdir, "reference_" + name)])
+            built.append("tests/cpp/reference_" + name)
     for cmd in cmds:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("build failed: %s\n%s%s" % (" ".join(cmd), r.stdout, r.stderr))
     if verbose:
-        print("built tests/cpp/prepacked_cache_test, tests/cpp/api_test")
+        print("built " + ", ".join(built))
 
 
 if __name__ == "__main__":

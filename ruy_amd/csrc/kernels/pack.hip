@@ -467,6 +467,7 @@ __global__ __launch_bounds__(256) void ReorderKernel(const T* src, int64_t src_r
 
 hipError_t LaunchReorder(hipStream_t stream, const DevMat& src, const DevMat& dst) {
   if (dst.rows == 0 || dst.cols == 0) return hipSuccess;
+  if ((int64_t(dst.cols) + 31) / 32 > 65535) return hipErrorInvalidValue;  // grid.y
   const dim3 grid((dst.rows + 31) / 32, (dst.cols + 31) / 32);
   switch (DtypeSize(dst.dtype)) {
     case 1:
@@ -481,6 +482,11 @@ hipError_t LaunchReorder(hipStream_t stream, const DevMat& src, const DevMat& ds
     case 4:
       hipLaunchKernelGGL(ReorderKernel<uint32_t>, grid, dim3(256), 0, stream,
                          static_cast<const uint32_t*>(src.data), src.rs, src.cs, static_cast<uint32_t*>(dst.data),
+                         dst.rs, dst.cs, dst.rows, dst.cols);
+      break;
+    case 8:
+      hipLaunchKernelGGL(ReorderKernel<uint64_t>, grid, dim3(256), 0, stream,
+                         static_cast<const uint64_t*>(src.data), src.rs, src.cs, static_cast<uint64_t*>(dst.data),
                          dst.rs, dst.cs, dst.rows, dst.cols);
       break;
     default:

@@ -591,8 +591,7 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
                                side8 == 0 ? call->lhs_src_key : call->rhs_src_key,
                                side8 == 0 ? N : M, /*u8_depth_step=*/0, &a, err))
     return rc;
-  if (int rc = EnsureOnDevice(ctx, call, side16, err)) return rc;
-  const DevMat& m16 = side16 == 0 ? call->lhs : call->rhs;
+  const DevMat& m16 = side16 == 0 ? call->lhs : call->rhs;  // shape only: its data may still be host memory
   const PackSource src = side16 == 0 ? PackSource{m16.data, m16.rs, m16.cs, m16.rows, m16.cols, m16.dtype}
                                      : PackSource{m16.data, m16.cs, m16.rs, m16.cols, m16.rows, m16.dtype};
   const int32_t ld = RoundUp(K > 0 ? K : 1, 16);
@@ -602,14 +601,62 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     *err = "int16 operand too large for the matrix-core kernel";
     return RUYAMD_E_UNSUPPORTED;
   }
-  int8_t* planes = static_cast<int8_t*>(ctx->ws->Alloc(packed_bytes));
-  if (!planes) {
-    *err = "workspace allocation failed";
-    return RUYAMD_E_HIP;
+  int8_t* planes = nullptr;
+  const int policy16 = side16 == 0 ? call->lhs_cache_policy : call->rhs_cache_policy;
+  const void* key16 = side16 == 0 ? call->lhs_src_key : call->rhs_src_key;
+  if (ShouldCache(policy16, side16 == 0 ? N : M)) {
+    // The two planes are the packed form of the int16 operand: cached like any
+    // other packed matrix (ruy/prepare_packed_matrices.cc:70-95), under a
+    // layout of their own (64 plane vectors per 32 source vectors).
+    PackedMatrix pm;
+    pm.element_size = 1;
+    pm.is_floating_point = false;
+    pm.layout.rows = ld;
+    pm.layout.cols = n_phys;
+    pm.layout.stride = ld;
+    pm.layout.kernel_rows = 16;
+    pm.layout.kernel_cols = 64;
+    const auto action = ctx->cache->Get(key16, &pm, CacheMode(ctx));
+    if (action == PrepackedCache::Action::kMissing && !ctx->no_alloc) {
+      *err = kCaptureCacheMiss;
+      return RUYAMD_E_UNSUPPORTED;
+    }
+    if (action != PrepackedCache::Action::kMissing) {
+      if (!pm.data) {
+        *err = "device allocation for a cached packed matrix failed";
+        return RUYAMD_E_HIP;
+      }
+      if (action == PrepackedCache::Action::kInsertedNewEntry) {
+        if (int rc = EnsureOnDevice(ctx, call, side16, err)) {
+          ctx->cache->Erase(key16, pm);
+          return rc;
+        }
+        const DevMat& m = side16 == 0 ? call->lhs : call->rhs;
+        const PackSource fresh = side16 == 0 ? PackSource{m.data, m.rs, m.cs, m.rows, m.cols, m.dtype}
+                                             : PackSource{m.data, m.cs, m.rs, m.cols, m.rows, m.dtype};
+        if (LaunchPackI16Split(ctx->stream, fresh, static_cast<int8_t*>(pm.data), ld) != hipSuccess) {
+          ctx->cache->Erase(key16, pm);
+          *err = "int16 pack kernel launch failed";
+          return RUYAMD_E_HIP;
+        }
+      }
+      planes = static_cast<int8_t*>(pm.data);
+    }
   }
-  if (LaunchPackI16Split(ctx->stream, src, planes, ld) != hipSuccess) {
-    *err = "int16 pack kernel launch failed";
-    return RUYAMD_E_HIP;
+  if (!planes) {
+    if (int rc = EnsureOnDevice(ctx, call, side16, err)) return rc;
+    const DevMat& m = side16 == 0 ? call->lhs : call->rhs;
+    const PackSource fresh = side16 == 0 ? PackSource{m.data, m.rs, m.cs, m.rows, m.cols, m.dtype}
+                                         : PackSource{m.data, m.cs, m.rs, m.cols, m.rows, m.dtype};
+    planes = static_cast<int8_t*>(ctx->ws->Alloc(packed_bytes));
+    if (!planes) {
+      *err = "workspace allocation failed";
+      return RUYAMD_E_HIP;
+    }
+    if (LaunchPackI16Split(ctx->stream, fresh, planes, ld) != hipSuccess) {
+      *err = "int16 pack kernel launch failed";
+      return RUYAMD_E_HIP;
+    }
   }
   args.k_bytes = RoundUp(K, 16);
   args.a = a.data;
@@ -690,7 +737,62 @@ uint64_t VectorsThatFit(const DevMat& m, int depth) {
   return limit / vector_bytes;
 }
 
+// Generic kernel: an operand whose cache policy asks for it
+// (ruy/prepare_packed_matrices.cc:70-95 caches for every type tuple) is kept
+// in the prepacked cache as a plain depth-contiguous copy in its own element
+// type, with the int32 sums buffer the reference's packed matrices carry for
+// integer types (ruy/prepacked_cache.cc:33-37), so that entry counts and byte
+// accounting behave as in the reference. The kernel then reads the copy.
+int CacheGenericOperand(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
+  DevMat& m = side == 0 ? call->lhs : call->rhs;
+  const int policy = side == 0 ? call->lhs_cache_policy : call->rhs_cache_policy;
+  const void* key = side == 0 ? call->lhs_src_key : call->rhs_src_key;
+  const int count = side == 0 ? m.rows : m.cols;
+  const int depth = side == 0 ? m.cols : m.rows;
+  const int other_width = side == 0 ? call->rhs.cols : call->lhs.rows;
+  if (!ShouldCache(policy, other_width)) return RUYAMD_OK;
+  if ((int64_t(count) + 31) / 32 > 65535 || (int64_t(depth) + 31) / 32 > 65535) return RUYAMD_OK;  // copy kernel's grid
+  PackedMatrix pm;
+  pm.element_size = DtypeSize(m.dtype);
+  pm.is_floating_point = IsFloating(m.dtype);
+  pm.layout.rows = depth;
+  pm.layout.cols = count;
+  pm.layout.stride = depth;
+  pm.zero_point = m.zero_point;
+  const auto action = ctx->cache->Get(key, &pm, CacheMode(ctx));
+  if (action == PrepackedCache::Action::kMissing) {
+    if (ctx->no_alloc) return RUYAMD_OK;  // used from where it lies, for this call only
+    *err = kCaptureCacheMiss;
+    return RUYAMD_E_UNSUPPORTED;
+  }
+  if (!pm.data) {
+    *err = "device allocation for a cached packed matrix failed";
+    return RUYAMD_E_HIP;
+  }
+  DevMat copy = m;
+  copy.data = pm.data;
+  // Vector c of the side (LHS row / RHS column) at c * depth, depth-contiguous.
+  copy.rs = side == 0 ? depth : 1;
+  copy.cs = side == 0 ? 1 : depth;
+  if (action == PrepackedCache::Action::kInsertedNewEntry) {
+    if (int rc = EnsureOnDevice(ctx, call, side, err)) {
+      ctx->cache->Erase(key, pm);
+      return rc;
+    }
+    if (LaunchReorder(ctx->stream, m, copy) != hipSuccess) {
+      ctx->cache->Erase(key, pm);
+      *err = "copy kernel launch failed";
+      return RUYAMD_E_HIP;
+    }
+  }
+  m = copy;
+  (side == 0 ? call->lhs_host_bytes : call->rhs_host_bytes) = 0;  // nothing left to stage
+  return RUYAMD_OK;
+}
+
 int RunGeneric(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
+  if (int rc = CacheGenericOperand(ctx, call, 0, err)) return rc;
+  if (int rc = CacheGenericOperand(ctx, call, 1, err)) return rc;
   if (int rc = EnsureOnDevice(ctx, call, 0, err)) return rc;
   if (int rc = EnsureOnDevice(ctx, call, 1, err)) return rc;
   if (LaunchGeneric(ctx->stream, call->lhs, call->rhs, call->ep, call->dst, call->accum_dtype) != hipSuccess) {

@@ -31,6 +31,8 @@ def _load_oracle():
     lib.oracle_validate.argtypes = [_matp, _matp, _parp, _matp]
     lib.oracle_mul.restype = C.c_int
     lib.oracle_mul.argtypes = [_matp, _matp, _parp, _matp, C.POINTER(C.c_int)]
+    lib.oracle_requantize_i32.restype = C.c_int
+    lib.oracle_requantize_i32.argtypes = [_matp, _parp, _matp]
     lib.oracle_pack_sums.restype = C.c_int
     lib.oracle_pack_sums.argtypes = [_matp, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     lib.oracle_mul_packed.restype = C.c_int
@@ -79,6 +81,43 @@ def oracle_mul(problem, want_overflow=False, fill=0):
                            C.byref(ovf) if want_overflow else None)
     assert rc == 0, "oracle_mul rejected the problem: %d" % rc
     return (out, bool(ovf.value)) if want_overflow else out
+
+
+def raw_problem(problem):
+    """The same product with a raw int32 destination (column-major, no
+    multiplier, no clamp): bias and zero points as in `problem`."""
+    from ruy_amd import workloads as W
+    assert problem.multiplier_fixedpoint_perchannel is None or problem.channel_dimension is not None
+    return W.Problem(problem.name + " raw", problem.lhs, problem.rhs,
+                     W.HostMatrix(S.I32, problem.M, problem.N, S.ORDER_COL_MAJOR), S.I32,
+                     bias=problem.bias, channel_dimension=problem.channel_dimension)
+
+
+def oracle_requantize(problem, raw_storage):
+    """`raw_storage`: the dst storage of raw_problem(problem). Returns the dst
+    storage of `problem` (flat, strided as problem.dst, untouched elements 0)."""
+    raw = raw_problem(problem)
+    out = _fresh_dst(problem)
+    r = raw.dst.struct(raw_storage.ctypes.data)
+    d = problem.dst.struct(out.ctypes.data)
+    p = problem.params_struct()
+    rc = oracle.oracle_requantize_i32(C.byref(r), C.byref(p), C.byref(d))
+    assert rc == 0, rc
+    return out
+
+
+def full_size_expected(problem, threads=16):
+    """The reference's result for a product too large for oracle_mul: int32
+    accumulators from stock ruy's fastest host path on `threads` threads (exact
+    on every path for an int32 destination, ruy/test.h:1392-1395), then the
+    scalar tail of ReferenceMul over every element. None when the stock
+    library is not built."""
+    if stock is None:
+        return None
+    raw = stock_mul(raw_problem(problem), path=0, threads=threads)
+    if raw is None:
+        return None
+    return oracle_requantize(problem, raw)
 
 
 def oracle_mul_packed(problem, depth_round):

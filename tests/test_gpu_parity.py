@@ -324,6 +324,18 @@ def test_full_size_int8_gemm_8192(device_ctx):
     g, w = _sample_block(p, got, rows, cols)
     assert (g == w).all(), "%d mismatches in the sampled block" % (g != w).sum()
 
+    # Every one of the 67 108 864 elements, when the stock reference library is
+    # present: its fastest host path gives the exact int32 accumulators
+    # (ruy/test.h:1392-1395), the checker's scalar tail of ReferenceMul
+    # (ruy/reference_mul.h:44-49) turns them into the int8 result.
+    want = O.full_size_expected(p)
+    if want is not None:
+        announce("T requantized, every element", n)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "%d of %d elements differ, first at %d" % (bad.size, got.size, bad[0])
+    else:
+        announce("T requantized: stock reference library absent, sample + checksum only")
+
     announce("T raw int32 checksum", n)
     raw = W.Problem("raw", p.lhs, p.rhs, W.HostMatrix(S.I32, n, n, S.ORDER_COL_MAJOR), S.I32, bias=p.bias)
     got = O.dense_of(raw, D.device_mul(device_ctx, raw, dst_fill=0)).astype(np.int64)
@@ -422,6 +434,69 @@ def test_prepacked_cache_through_mul(device_ctx):
     finally:
         ctx.set_cache_max_bytes(1 << 28)
     assert ctx.cache_matrix_count() == 0
+
+
+def test_cache_policy_on_generic_tuples_and_int16_operands(device_ctx):
+    """The reference caches a packed operand for every type tuple
+    (ruy/prepare_packed_matrices.cc:70-95). Tuples served by the generic kernel
+    keep a plain depth-contiguous copy (+ int32 sums buffer for integer types,
+    as ruy/prepacked_cache.cc:33-37 counts them); the int16 operand of the
+    int8 x int16 kernel keeps its two int8 planes. Entry counts and bytes are
+    checked, the second call is a hit, results stay those of the checker."""
+    import device_runner as D
+    ctx = device_ctx
+    ctx.clear_prepacked_cache()
+    rng = np.random.default_rng(2718)
+    # fp64 x fp32 (generic kernel), LHS cached: 40 x 50 doubles, no sums.
+    p = W.random_problem(rng, S.F64, S.F32, S.F64, S.F32, 40, 50, 6, 0, 1, 0, strided=True)
+    p.lhs.cache_policy = S.CACHE_ALWAYS
+    dp = D.DeviceProblem(p)
+    want = expected(p)
+    for call in range(2):
+        dp.clear_dst()
+        dp.run(ctx)
+        assert ctx.last_kernel_name() == "generic"
+        compare(p, dp.result(), want, exact_fp=True)
+        assert ctx.cache_matrix_count() == 1 and ctx.cache_buffers_bytes() == 40 * 50 * 8, call
+    # RHS cached too, under the heuristic policy (40 rows > 8: not cached; 6 columns <= 8: the LHS would be).
+    p.rhs.cache_policy = S.CACHE_IF_LARGE_SPEEDUP
+    dp2 = D.DeviceProblem(p)
+    dp2.run(ctx)
+    assert ctx.cache_matrix_count() == 2  # new LHS pointer; the RHS stays uncached
+    compare(p, dp2.result(), want, exact_fp=True)
+    # The generic kernel forced on an int8 product: packed int8 copy + sums.
+    ctx.clear_prepacked_cache()
+    q = W.random_problem(rng, S.I8, S.U8, S.I32, S.I8, 33, 70, 5, 1, 0, 0)
+    q.rhs.cache_policy = S.CACHE_ALWAYS
+    ctx.force_generic_kernel(True)
+    try:
+        got, want_q = run_both(ctx, q)
+    finally:
+        ctx.force_generic_kernel(False)
+    compare(q, got, want_q)
+    assert ctx.cache_matrix_count() == 1 and ctx.cache_buffers_bytes() == 70 * 5 + 5 * 4
+    # int16 x int8, the int16 LHS cached as planes: ceil(40/32)*64 = 128 plane vectors of 64 bytes + sums.
+    ctx.clear_prepacked_cache()
+    r = W.random_problem(rng, S.I16, S.I8, S.I32, S.I16, 40, 64, 4, 1, 0, 0)
+    r.lhs.cache_policy = S.CACHE_ALWAYS
+    dr = D.DeviceProblem(r)
+    want_r = expected(r)
+    for call in range(2):
+        dr.clear_dst()
+        dr.run(ctx)
+        assert ctx.last_kernel_name() == "i8i16_mfma"
+        compare(r, dr.result(), want_r)
+        assert ctx.cache_matrix_count() == 1 and ctx.cache_buffers_bytes() == 128 * 64 + 128 * 4, call
+    # int8 x int16 with the int16 RHS cached (C4's tuple), from host pointers: the
+    # second call finds the planes in the cache and uploads only the int8 side.
+    ctx.clear_prepacked_cache()
+    c4 = W.config_int8_int16(96, 128, 40)
+    c4.rhs.cache_policy = S.CACHE_ALWAYS
+    want_c4 = O.oracle_mul(c4)
+    for call in range(2):
+        assert (D.host_pointer_mul(ctx, c4, dst_fill=0) == want_c4).all()
+        assert ctx.cache_matrix_count() == 1
+    ctx.clear_prepacked_cache()
 
 
 def test_tuned_kernels_are_the_ones_that_run(device_ctx):
@@ -738,6 +813,10 @@ def test_grids_cut_into_two_launches(device_ctx, shape, tup):
             assert err <= REL_FROBENIUS_TOL, err
             continue
         assert (g == w).all(), "%d mismatches in the sampled block" % (g != w).sum()
+        want = O.full_size_expected(p)
+        if want is not None:  # every element (see test_full_size_int8_gemm_8192)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
         raw = W.Problem("raw", p.lhs, p.rhs, W.HostMatrix(S.I32, M, N, S.ORDER_COL_MAJOR), S.I32)
         got = O.dense_of(raw, D.device_mul(device_ctx, raw, dst_fill=0)).astype(np.int64)
         L = p.lhs.dense().astype(np.int64) - p.lhs.zero_point

@@ -324,6 +324,36 @@ def test_packed_form_equals_reference_form(depth_round):
             assert (O.oracle_mul(p) == O.oracle_mul_packed(p, depth_round)).all()
 
 
+@pytest.mark.parametrize("tup", [t for t in cases.INT_TUPLES if t[3] != S.I32], ids=cases.tuple_name)
+def test_requantize_of_raw_accumulators_equals_reference_form(tup):
+    """oracle_requantize_i32 over the int32 result of a product == the product
+    computed straight into the narrow type: the two-step form used for shapes
+    that are too large for oracle_mul. Every order, padded strides, both
+    channel dimensions, scalar and per-channel multipliers as random_problem
+    draws them. A dropped zero point, a bias applied twice, a transposed
+    channel index or a wrong stride would each fail here."""
+    rng = np.random.default_rng(4711 + cases.TYPE_TUPLES.index(tup))
+    seen = set()
+    for shape in [(13, 37, 11), (1, 64, 5), (31, 1, 29), (16, 96, 16), (7, 6, 5)]:
+        for orders in cases.ALL_ORDERS:
+            for strided in (False, True):
+                p = W.random_problem(rng, *tup, *shape, *orders, strided=strided,
+                                     name="%s %s %s %s" % (cases.tuple_name(tup), shape, orders, strided))
+                raw = O.oracle_mul(O.raw_problem(p))
+                assert (O.oracle_requantize(p, raw) == O.oracle_mul(p)).all(), p.name
+                seen.add((p.channel_dimension, p.multiplier_fixedpoint_perchannel is not None, p.bias is not None))
+    assert len(seen) >= 6  # the draw really covered the parameter space
+
+
+def test_requantize_known_answers():
+    """The saturation answers of ruy/test_overflow_dst_zero_point.cc through the
+    two-step form: accumulators first, then the tail."""
+    for dst_dtype, cols, zp in SATURATION_CASES:
+        p, want = saturation_problem(dst_dtype, cols, zp)
+        raw = O.oracle_mul(O.raw_problem(p))
+        assert (O.oracle_requantize(p, raw)[:cols] == want).all()
+
+
 def test_validate_rejects_illegal_zero_points():
     """ruy/validate.h:40-75."""
     def rc(p):
@@ -414,6 +444,20 @@ def test_against_stock_reference_and_standard_cpp(tup):
             # the reference's own tolerance for its x86 SIMD paths: 0 on raw
             # accumulators, 1 on requantized outputs (ruy/test.h:1392-1417)
             assert d <= (0 if tup[3] == S.I32 else 1), (shape, orders, d)
+
+
+@needs_stock
+def test_full_size_expected_is_reference_mul():
+    """The large-shape recipe (stock ruy's fastest path into int32 on several
+    threads, then oracle_requantize_i32) against stock ReferenceMul itself, at
+    sizes ReferenceMul still finishes."""
+    rng = np.random.default_rng(8192)
+    for tup in [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I16), (S.I8, S.U8, S.I32, S.I8)]:
+        for shape, orders in [((300, 520, 270), cases.RCC), ((257, 129, 130), (1, 0, 1)), ((64, 777, 200), (0, 1, 0))]:
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=True)
+            want = O.stock_mul(p, reference=True)
+            got = O.full_size_expected(p, threads=4)
+            assert got is not None and (got == want).all(), (tup, shape, orders)
 
 
 @needs_stock
