@@ -1,0 +1,75 @@
+// The arithmetic of the depth split, shared by the kernels, the host-side
+// planner and a host-only model test: which depth steps a part walks, when a
+// split has no empty part, and who does the write-back.
+//
+// Protocol (tiled kernels, small tiles only). A launch carries `parts`
+// workgroups per destination tile. Each walks its part of the depth steps,
+// stores its raw accumulators to its slice of a scratch buffer, waits until
+// those stores have been performed, and then adds 1 to the tile's arrival
+// counter; the workgroup whose add returns parts - 1 is the last to arrive: it
+// sets the counter back to 0 for the next launch, reads all slices in the order
+// of the parts (so a floating-point sum does not depend on who was last) and
+// runs the write-back. Nobody waits for anybody, so a launch cannot hang.
+//
+// What orders the accesses on the device. The slices and the counter are
+// accessed with agent-scope atomic operations only (relaxed): on gfx942/gfx950
+// those are performed at the point where all XCDs of the device agree (they
+// carry the sc1 bit and do not linger in an XCD's L2). A workgroup issues its
+// counter add only after s_waitcnt vmcnt(0) has returned for its slice stores,
+// i.e. after they have been performed there, and after a workgroup barrier, so
+// every wave's stores are covered; the last arriver issues its slice loads
+// only after the add has returned its value (the loads depend on it through
+// the branch and are issued behind it in program order). These are the two
+// properties the compiler's own agent-scope release and acquire sequences
+// rest on (release: write back, s_waitcnt vmcnt(0), then the atomic; acquire:
+// the atomic, then invalidate): the kernel uses per-access sc1 operations
+// where those sequences write back and invalidate whole caches.
+#ifndef RUY_AMD_CSRC_KERNELS_DEPTH_SPLIT_H_
+#define RUY_AMD_CSRC_KERNELS_DEPTH_SPLIT_H_
+
+#if defined(__HIPCC__)
+#define RUYAMD_HOST_DEVICE __host__ __device__
+#else
+#define RUYAMD_HOST_DEVICE
+#endif
+
+namespace ruyamd {
+namespace depth_split {
+
+// Depth steps per part when `steps` steps are dealt to `parts` parts.
+RUYAMD_HOST_DEVICE inline int StepsPerPart(int steps, int parts) { return (steps + parts - 1) / parts; }
+
+// First step of part `index`.
+RUYAMD_HOST_DEVICE inline int FirstStep(int steps, int parts, int index) {
+  return index * StepsPerPart(steps, parts);
+}
+
+// Number of steps of part `index` (0 if the part lies past the end).
+RUYAMD_HOST_DEVICE inline int StepCount(int steps, int parts, int index) {
+  const int per = StepsPerPart(steps, parts);
+  const int left = steps - index * per;
+  return left < 0 ? 0 : (left < per ? left : per);
+}
+
+// Every part has at least one step (what a launch requires).
+RUYAMD_HOST_DEVICE inline bool NoEmptyPart(int steps, int parts) {
+  return parts >= 1 && (parts - 1) * StepsPerPart(steps, parts) < steps;
+}
+
+// The largest number of parts <= `wanted` that leaves no part empty with
+// the steps dealt as above.
+RUYAMD_HOST_DEVICE inline int PartsWithoutEmpty(int steps, int wanted) {
+  if (wanted < 1 || steps < 1) return 1;
+  const int per = StepsPerPart(steps, wanted);
+  return (steps + per - 1) / per;
+}
+
+// `previous`: what this workgroup's add on the tile's arrival counter returned.
+RUYAMD_HOST_DEVICE inline bool IsLastArrival(unsigned previous, int parts) {
+  return previous == static_cast<unsigned>(parts - 1);
+}
+
+}  // namespace depth_split
+}  // namespace ruyamd
+
+#endif  // RUY_AMD_CSRC_KERNELS_DEPTH_SPLIT_H_

@@ -50,6 +50,7 @@
 
 #include "../epilogue.h"
 #include "../internal.h"
+#include "depth_split.h"
 #include "gemm_i8.h"
 
 namespace ruyamd {
@@ -266,9 +267,8 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   constexpr bool kCanSplitDepth = WM * WN <= 2 && kB == 32;
   const int split = kCanSplitDepth ? args.split_k : 1;
   const int split_index = kCanSplitDepth ? blockIdx.y : 0;
-  const int k_tiles_per_split = (k_tiles_all + split - 1) / split;
-  const int kt_first = split_index * k_tiles_per_split;
-  const int k_tiles = max(0, min(k_tiles_per_split, k_tiles_all - kt_first));
+  const int kt_first = depth_split::FirstStep(k_tiles_all, split, split_index);
+  const int k_tiles = depth_split::StepCount(k_tiles_all, split, split_index);
   constexpr bool kRotateDepth = WM * WN < 16;
   const int rot = kRotateDepth && K % kBK == 0 && k_tiles > 0 ? (tile_m * 5 + split_index * 3) % k_tiles : 0;
   auto phys = [&](int kt) {
@@ -649,9 +649,10 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
   // L2 caches do not see each other's lines: every access to them and to the
   // counter is a device-scope atomic (relaxed: a plain store or load that goes
   // past the caches that are not shared), the stores are awaited before the
-  // counter is touched, and the loads are issued after its value is known.
-  // That costs nothing when no split is asked for, where fences at device
-  // scope would write back and invalidate whole caches.
+  // counter is touched, and the loads are issued after its value is known
+  // (depth_split.h says what this ordering rests on). That costs nothing when
+  // no split is asked for, where fences at device scope would write back and
+  // invalidate whole caches.
   if constexpr (kCanSplitDepth) {
     if (split > 1) {
       typedef unsigned long long u64;
@@ -675,7 +676,7 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
       if (tid == 0)
         *arrived = __hip_atomic_fetch_add(args.split_counters + t, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
-      const bool last = *arrived == unsigned(split - 1);
+      const bool last = depth_split::IsLastArrival(*arrived, split);
       __syncthreads();  // the flag's LDS word is part of the write-back's staging area
       if (!last) return;
       if (tid == 0) __hip_atomic_store(args.split_counters + t, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -868,7 +869,7 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   if (split != 1) {
     const int k_tiles = (args.k_bytes + BK - 1) / BK;
     if (WM * WN > 2 || Traits::kBlock != 32 || split < 1 || !args.split_partials || !args.split_counters || total > kSplitCounters ||
-        (split - 1) * ((k_tiles + split - 1) / split) >= k_tiles)
+        !depth_split::NoEmptyPart(k_tiles, split))
       return hipErrorInvalidValue;
   }
   hipLaunchKernelGGL(kernel, dim3(grid, split), dim3(C::kThreads), lds_bytes, stream, args);
@@ -1056,8 +1057,7 @@ inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, Model model)
   if (tiles == 0 || tiles > kSplitCounters) return DepthSplit();
   int parts = std::min({num_cus / tiles, k_tiles / kMinStepsPerPart, kMaxParts});
   if (parts < 2) return DepthSplit();
-  const int steps_per_part = (k_tiles + parts - 1) / parts;
-  parts = (k_tiles + steps_per_part - 1) / steps_per_part;  // no empty part
+  parts = depth_split::PartsWithoutEmpty(k_tiles, parts);
   DepthSplit split;
   split.parts = parts;
   split.partial_bytes = size_t(parts) * tiles * bm * bn * 4;

@@ -4,9 +4,21 @@
 // (ruy/kernel.h:174-241 is the reference's counterpart), so its grid must be
 // legal for every int-sized destination, including tall row-major ones whose
 // tile-row count exceeds HIP's 65535 limit on grid.y.
+//
+// Depth split: the arrival-counter protocol of the tiled kernels, modelled
+// with host threads in place of workgroups (one thread per part of a tile).
+// The model uses the same arithmetic header as the kernels and checks what
+// does not depend on the hardware: the parts cover every depth step exactly
+// once whatever the remainder, exactly one workgroup per tile elects itself,
+// it sees every part, the sum is taken in part order, and the counters are
+// back at zero for the next launch.
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
+#include <thread>
+#include <vector>
 
+#include "kernels/depth_split.h"
 #include "kernels/launch_geometry.h"
 
 static int g_failures = 0;
@@ -52,9 +64,105 @@ static void TestElementwiseBlocks() {
   EXPECT(ruyamd::ElementwiseBlocks(int64_t(1) << 40, 256) == ruyamd::kMaxGridX);
 }
 
+namespace ds = ruyamd::depth_split;
+
+static void TestDepthPartsCoverEveryStepOnce() {
+  for (int steps = 1; steps <= 300; ++steps) {
+    for (int wanted = 1; wanted <= 40; ++wanted) {
+      const int parts = ds::PartsWithoutEmpty(steps, wanted);
+      EXPECT(parts >= 1 && parts <= wanted);
+      EXPECT(ds::NoEmptyPart(steps, parts));
+      std::vector<int> covered(steps, 0);
+      for (int z = 0; z < parts; ++z) {
+        const int first = ds::FirstStep(steps, parts, z), count = ds::StepCount(steps, parts, z);
+        EXPECT(count >= 1);
+        for (int k = first; k < first + count; ++k) {
+          EXPECT(k < steps);
+          if (k < steps) ++covered[k];
+        }
+      }
+      for (int k = 0; k < steps; ++k) EXPECT(covered[k] == 1);
+      // A part index past the last part walks nothing (what a kernel launched
+      // with more grid rows than parts would see).
+      EXPECT(ds::StepCount(steps, parts, parts) == 0);
+    }
+  }
+  EXPECT(!ds::NoEmptyPart(10, 7));  // 7 parts of 2 steps: parts 5 and 6 would be empty
+  EXPECT(ds::PartsWithoutEmpty(10, 7) == 5);
+}
+
+// One "launch": tiles x parts threads. Thread (t, z) computes the partial sum
+// of its depth steps of tile t (step k of tile t contributes value(t, k)),
+// stores it to its slice, counts itself in, and if it was the last to arrive
+// resets the counter, adds the slices up in part order and writes the result.
+// fetch_add is acq_rel here: on the device the same ordering comes from
+// waiting for the slice stores before the add and issuing the slice loads
+// after it (see depth_split.h).
+struct SplitModel {
+  int tiles, steps;
+  std::vector<std::atomic<unsigned>> counters;
+  std::vector<double> slices;  // [tile][part]
+  std::vector<double> result;  // [tile]
+  std::vector<std::atomic<int>> finishers;
+  SplitModel(int tiles_, int steps_, int max_parts)
+      : tiles(tiles_), steps(steps_), counters(tiles_), slices(size_t(tiles_) * max_parts), result(tiles_),
+        finishers(tiles_) {
+    for (auto& c : counters) c.store(0);
+  }
+  static double Value(int tile, int k) { return 1.0 / (1 + tile + 3 * k); }  // order of summation matters
+  void Launch(int parts, unsigned shuffle) {
+    for (auto& f : finishers) f.store(0);
+    std::vector<std::thread> threads;
+    const int total = tiles * parts;
+    for (int n = 0; n < total; ++n) {
+      // A different arrival order every launch.
+      const int id = int((n * 7919u + shuffle * 104729u) % unsigned(total));
+      threads.emplace_back([this, id, parts] {
+        const int t = id / parts, z = id % parts;
+        double part = 0;
+        const int first = ds::FirstStep(steps, parts, z);
+        for (int k = first; k < first + ds::StepCount(steps, parts, z); ++k) part += Value(t, k);
+        slices[size_t(t) * parts + z] = part;
+        const unsigned previous = counters[t].fetch_add(1u, std::memory_order_acq_rel);
+        if (!ds::IsLastArrival(previous, parts)) return;
+        counters[t].store(0u, std::memory_order_relaxed);
+        double sum = 0;
+        for (int p = 0; p < parts; ++p) sum += slices[size_t(t) * parts + p];
+        result[t] = sum;
+        finishers[t].fetch_add(1);
+      });
+    }
+    for (auto& th : threads) th.join();
+  }
+};
+
+static void TestDepthSplitArrivalProtocol() {
+  const int tiles = 6, steps = 37, max_parts = 8;
+  SplitModel model(tiles, steps, max_parts);
+  for (int launch = 0; launch < 24; ++launch) {
+    const int parts = ds::PartsWithoutEmpty(steps, 2 + launch % (max_parts - 1));
+    model.Launch(parts, unsigned(launch));
+    for (int t = 0; t < tiles; ++t) {
+      EXPECT(model.finishers[t].load() == 1);      // exactly one workgroup did the write-back
+      EXPECT(model.counters[t].load() == 0);       // left at zero for the next launch
+      // Reference: the same parts, summed in part order by one thread.
+      double want = 0;
+      for (int z = 0; z < parts; ++z) {
+        double part = 0;
+        const int first = ds::FirstStep(steps, parts, z);
+        for (int k = first; k < first + ds::StepCount(steps, parts, z); ++k) part += SplitModel::Value(t, k);
+        want += part;
+      }
+      EXPECT(model.result[t] == want);  // bit for bit: the order does not depend on who arrived last
+    }
+  }
+}
+
 int main() {
   TestGenericGrid();
   TestElementwiseBlocks();
+  TestDepthPartsCoverEveryStepOnce();
+  TestDepthSplitArrivalProtocol();
   if (g_failures) {
     std::fprintf(stderr, "host_logic_test: %d failure(s)\n", g_failures);
     return 1;
