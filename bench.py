@@ -491,12 +491,31 @@ def bench_other_configs(ctx, args):
             entry["roofline"]["note"] = note
         if not args.no_graph and problem.ops() < 1e9:
             entry["us_per_step_graph"] = graph_replay_us(ctx, dp)
+        if problem.ops() < 1e9:
+            entry["us_per_product_batch32"] = batch_us(ctx, problem)
         if not args.no_cpu_baseline:
             entry["cpu_baseline"] = cpu_baseline(problem, ops, unit, "full shape M=%d K=%d N=%d" % (
                 problem.M, problem.K, problem.N), min_secs=0.5, repeats=2)
         out.append(entry)
     ctx.set_kernel_timing(True)
     return out
+
+
+def batch_us(ctx, problem, count=32, repeats=50):
+    """Per-product time of ruyamd_mul_batch over `count` products of this
+    configuration (each on its own device buffers): one launch instead of
+    `count` calls."""
+    import torch
+    from ruy_amd import device_problem as D
+    dps = [D.DeviceProblem(problem, dst_fill=0) for _ in range(count)]
+    for _ in range(5):
+        D.run_batch(ctx, dps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        D.run_batch(ctx, dps)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / (repeats * count) * 1e6
 
 
 def graph_replay_us(ctx, dp, calls=32, replays=20):

@@ -148,6 +148,24 @@ RUYAMD_API int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs,
                           const ruyamd_mul_params* params,
                           const ruyamd_mat* dst);
 
+/* n independent products in one call: lhs[i] * rhs[i] -> dst[i] under
+ * params[i], for i in [0, n). The results are those of n ruyamd_mul calls; no
+ * destination may overlap any other buffer of the batch. The reference has no
+ * such function: its niche is small matrices (README.md:12-19) and a CPU
+ * caller simply loops over ruy::Mul (ruy/ruy.h:36-48), which on a device costs
+ * a kernel launch and the host work of a call per product. When all products
+ * have the same shape, layout, types, zero points and MulParams values, every
+ * buffer is device memory, the operands can be used where they lie (8-bit,
+ * depth-contiguous, 16-byte aligned) and the shape is one the tiled kernel
+ * runs on its smallest tile, the whole batch is one launch per 32 products
+ * (only the buffer addresses differ from product to product). Any other batch
+ * is executed as n calls enqueued back to back on the context's stream with a
+ * single wait at the end. */
+RUYAMD_API int ruyamd_mul_batch(ruyamd_ctx* ctx, int n, const ruyamd_mat* lhs,
+                                const ruyamd_mat* rhs,
+                                const ruyamd_mul_params* params,
+                                const ruyamd_mat* dst);
+
 /* ruyamd_mul for callers that cannot allocate device memory: code whose
  * stream is being captured into a graph, tight serving loops, harnesses that
  * forbid hipMalloc. It has no counterpart in the reference. Same arguments,

@@ -36,6 +36,7 @@ PROTOTYPES = {
     "ruyamd_ctx_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "ruyamd_ctx_destroy": (None, [_ctx]),
     "ruyamd_mul": (C.c_int, [_ctx, _matp, _matp, _parp, _matp]),
+    "ruyamd_mul_batch": (C.c_int, [_ctx, C.c_int, _matp, _matp, _parp, _matp]),
     "ruyamd_mul_no_alloc": (C.c_int, [_ctx, _matp, _matp, _parp, _matp]),
     "ruyamd_ctx_set_stream": (C.c_int, [_ctx, C.c_void_p]),
     "ruyamd_ctx_set_synchronous": (C.c_int, [_ctx, C.c_int]),

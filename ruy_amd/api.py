@@ -342,6 +342,18 @@ class Context:
             self._h, _address(x), _address(m), _address(e), _address(out), n))
 
 
+def mul_batch(items, context):
+    """`items`: a sequence of (lhs, rhs, mul_params, dst) as for mul(). One call
+    of ruyamd_mul_batch; a CPU caller of the reference would loop over ruy::Mul."""
+    n = len(items)
+    ls, rs, ps, ds = (S.Mat * n)(), (S.Mat * n)(), (S.MulParamsStruct * n)(), (S.Mat * n)()
+    for i, (lhs, rhs, mul_params, dst) in enumerate(items):
+        if mul_params.dst_dtype != dst.dtype:
+            raise ValueError("MulParams DstScalar does not match the destination matrix")
+        ls[i], rs[i], ps[i], ds[i] = lhs.to_struct(), rhs.to_struct(), mul_params.to_struct(), dst.to_struct()
+    context._check(lib.ruyamd_mul_batch(context._h, n, ls, rs, ps, ds))
+
+
 def mul(lhs, rhs, mul_params, context, dst):
     """ruy::Mul (ruy/ruy.h:96-102)."""
     if mul_params.dst_dtype != dst.dtype:

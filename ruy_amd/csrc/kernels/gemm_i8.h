@@ -64,6 +64,19 @@ struct GemmArgs {
   uint32_t* split_counters = nullptr;
 };
 
+// Buffers of the products of a batched launch (GemmArgs holds what they have
+// in common): operand, destination and per-channel parameter pointers of
+// product z, the latter null where the common arguments have none.
+constexpr int kGemmBatchMax = 32;
+struct GemmBatch {
+  const void* a[kGemmBatchMax];
+  const void* b[kGemmBatchMax];
+  void* dst[kGemmBatchMax];
+  const void* bias[kGemmBatchMax];
+  const int32_t* mult_fixedpoint[kGemmBatchMax];
+  const int32_t* mult_exponent[kGemmBatchMax];
+};
+
 // How a launch of these arguments should split the depth: the number of parts
 // (1 = no split) and the bytes of split_partials it needs. `kind`: which
 // launcher the arguments are for.
@@ -80,6 +93,12 @@ int GemmDepthSplitCounters();
 // one that has a variant with the sums fused in.
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
+// `count` <= kGemmBatchMax products of the shape and parameters of `args`, each
+// on its own buffers, in one launch. Only for arguments that run on the
+// smallest tile (GemmI8CanFuseSums), without sums arrays (zero points 0, or the
+// sums fused) and without a depth split.
+hipError_t LaunchGemmI8Batch(hipStream_t stream, const GemmArgs& args, const GemmBatch& batch, int count,
+                             int num_cus);
 hipError_t LaunchGemmF32(hipStream_t stream, const GemmArgs& args, int num_cus);
 // int8 x int16: `b` is the int16 operand split by LaunchPackI16Split. On the
 // smallest tile (GemmI8I16CanFuseSums) fuse_sums / fused_a_factor work as in

@@ -195,4 +195,18 @@ hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
   return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);
 }
 
+hipError_t LaunchGemmI8Batch(hipStream_t stream, const GemmArgs& args, const GemmBatch& batch, int count,
+                             int num_cus) {
+  const bool flip = args.a_flip != 0 || args.b_flip != 0;
+  if (!GemmI8CanFuseSums(args, num_cus) || (flip && args.k_bytes % 128 != 0)) return hipErrorInvalidValue;
+  if (args.ep.lhs_sums || args.ep.rhs_sums || (!args.fuse_sums && (args.ep.lhs_zero_point || args.ep.rhs_zero_point)))
+    return hipErrorInvalidValue;  // sums arrays are per product: only the fused form is batched
+  if (flip) {
+    return args.fuse_sums ? mfma_gemm::LaunchSmallestTileBatch<Int8Traits, true, true>(stream, args, batch, count)
+                          : mfma_gemm::LaunchSmallestTileBatch<Int8Traits, false, true>(stream, args, batch, count);
+  }
+  return args.fuse_sums ? mfma_gemm::LaunchSmallestTileBatch<Int8Traits, true>(stream, args, batch, count)
+                        : mfma_gemm::LaunchSmallestTileBatch<Int8Traits>(stream, args, batch, count);
+}
+
 }  // namespace ruyamd

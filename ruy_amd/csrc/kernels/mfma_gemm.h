@@ -62,6 +62,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 
 
+inline int TileCount(const GemmArgs& args, int bm, int bn);
+
 constexpr int kGranule = 16;            // bytes per lane per load
 constexpr int kSplitCounters = 1024;    // tiles a depth-split launch may have (one counter each)
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any num_records we accept
@@ -167,7 +169,7 @@ struct Cfg {
 // values the arithmetic is defined on.
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false>
-__global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
+__device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
                 "fused sums exist for the tiles with one block (one block per plane) per wave only");
   static_assert(!kFlip || WM * WN == 1, "in-place uint8 operands exist for the single-block tile only");
@@ -848,6 +850,47 @@ __global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
 
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false>
+__global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
+  MfmaGemmBody<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>(args);
+}
+
+// Several products of one shape in one launch: grid.z counts the products,
+// which differ only in where their buffers lie. (What a CPU caller of the
+// reference does with a loop over ruy::Mul - its niche is small matrices,
+// README.md:12-19 - costs a kernel launch per product on a device.)
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
+          bool kDepthWaves = false>
+__global__ __launch_bounds__(256) void MfmaGemmBatchKernel(GemmArgs args, GemmBatch batch) {
+  const int z = blockIdx.z;
+  args.a = batch.a[z];
+  args.b = batch.b[z];
+  args.dst.data = batch.dst[z];
+  args.ep.bias = batch.bias[z];
+  args.ep.mult_fixedpoint = batch.mult_fixedpoint[z];
+  args.ep.mult_exponent = batch.mult_exponent[z];
+  MfmaGemmBody<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>(args);
+}
+
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
+          bool kDepthWaves = false>
+hipError_t LaunchBatch(hipStream_t stream, const GemmArgs& args, const GemmBatch& batch, int count) {
+  using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB, Traits::kBlock>;
+  if (count < 1 || count > kGemmBatchMax || args.split_k != 1) return hipErrorInvalidValue;
+  const int total = TileCount(args, C::kBM, C::kBN);
+  const int grid = ((total + 7) / 8) * 8;
+  const size_t lds_bytes = kDepthWaves ? size_t(4 * 2 * 128 * BK) : size_t(C::kLdsBytes);
+  auto kernel = MfmaGemmBatchKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>;
+  if (lds_bytes > 48 * 1024) {
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    if (attr != hipSuccess) return attr;
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid, 1, count), dim3(C::kThreads), lds_bytes, stream, args, batch);
+  return hipGetLastError();
+}
+
+template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
+          bool kDepthWaves = false>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB, Traits::kBlock>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
@@ -1077,6 +1120,16 @@ hipError_t LaunchSmallestTile(hipStream_t stream, const GemmArgs& args) {
   if ((k_tiles + parts - 1) / parts < kDepthWays)
     return Launch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, false>(stream, args);
   return Launch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, true>(stream, args);
+}
+
+template <typename Traits, bool kFusedSums = false, bool kFlip = false>
+hipError_t LaunchSmallestTileBatch(hipStream_t stream, const GemmArgs& args, const GemmBatch& batch, int count) {
+  constexpr int kWN = Traits::kSplitB ? 2 : 1;
+  constexpr int kDepthWays = 4 / kWN;
+  const int k_tiles = (args.k_bytes + 127) / 128;
+  if (k_tiles < kDepthWays)
+    return LaunchBatch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, false>(stream, args, batch, count);
+  return LaunchBatch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, true>(stream, args, batch, count);
 }
 
 template <typename Traits>

@@ -9,6 +9,7 @@
 #include <cstring>
 #include <limits>
 #include <string>
+#include <vector>
 
 #include "context.h"
 #include "internal.h"
@@ -195,6 +196,45 @@ class NoAllocScope {
   ruyamd_ctx* ctx_;
 };
 
+// The dispatcher's view of one call: matrices as strided device views (the
+// source operands may still be host memory, which the dispatcher stages when a
+// kernel is about to read them), the write-back parameters, cache keys.
+void FillCall(const ruyamd_mat& lhs, const ruyamd_mat& rhs, const ruyamd_mul_params& p, const ruyamd_mat& dst,
+              const void* bias_d, const void* mf_d, const void* me_d, void* dst_d, MulCall* out) {
+  MulCall& call = *out;
+  call.lhs = ToDevMat(lhs, lhs.data);
+  call.rhs = ToDevMat(rhs, rhs.data);
+  call.dst = ToDevMat(dst, dst_d);
+  call.lhs_src_key = lhs.data;
+  call.rhs_src_key = rhs.data;
+  call.lhs_cache_policy = lhs.cache_policy;
+  call.rhs_cache_policy = rhs.cache_policy;
+  call.accum_dtype = p.accum_dtype;
+  Epilogue& ep = call.ep;
+  ep.bias = bias_d;
+  ep.mult_fixedpoint = static_cast<const int32_t*>(mf_d);
+  ep.mult_exponent = static_cast<const int32_t*>(me_d);
+  ep.mult_fixedpoint_scalar = p.multiplier_fixedpoint;
+  ep.mult_exponent_scalar = p.multiplier_exponent;
+  ep.dst_zero_point = dst.zero_point;
+  ep.channel_is_col = p.channel_dimension == RUYAMD_CHANNEL_COL;
+  const bool fp = IsFloating(dst.dtype);
+  ep.requantize = !fp && dst.dtype != RUYAMD_DTYPE_I32;
+  if (fp) {
+    ep.clamp_min_f = static_cast<float>(p.clamp_min);
+    ep.clamp_max_f = static_cast<float>(p.clamp_max);
+    ep.clamp_min_d = p.clamp_min;
+    ep.clamp_max_d = p.clamp_max;
+  } else if (dst.dtype == RUYAMD_DTYPE_I32) {
+    // ruy/mul_params.h:291-293: no clamping of raw accumulators.
+    ep.clamp_min_i = std::numeric_limits<int32_t>::lowest();
+    ep.clamp_max_i = std::numeric_limits<int32_t>::max();
+  } else {
+    ep.clamp_min_i = ClampToInt32(p.clamp_min);
+    ep.clamp_max_i = ClampToInt32(p.clamp_max);
+  }
+}
+
 int MulImpl(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs, const ruyamd_mul_params* p,
             const ruyamd_mat* dst, bool no_alloc) {
   if (!ctx) return RUYAMD_E_INVALID;
@@ -263,39 +303,9 @@ int MulImpl(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs, const
   }
 
   MulCall call;
-  call.lhs = ToDevMat(*lhs, lhs->data);
-  call.rhs = ToDevMat(*rhs, rhs->data);
+  FillCall(*lhs, *rhs, *p, *dst, bias_d, mf_d, me_d, dst_d, &call);
   if (!lhs_dev) call.lhs_host_bytes = StorageElements(*lhs) * DtypeSize(lhs->dtype);
   if (!rhs_dev) call.rhs_host_bytes = StorageElements(*rhs) * DtypeSize(rhs->dtype);
-  call.dst = ToDevMat(*dst, dst_d);
-  call.lhs_src_key = lhs->data;
-  call.rhs_src_key = rhs->data;
-  call.lhs_cache_policy = lhs->cache_policy;
-  call.rhs_cache_policy = rhs->cache_policy;
-  call.accum_dtype = p->accum_dtype;
-  Epilogue& ep = call.ep;
-  ep.bias = bias_d;
-  ep.mult_fixedpoint = static_cast<const int32_t*>(mf_d);
-  ep.mult_exponent = static_cast<const int32_t*>(me_d);
-  ep.mult_fixedpoint_scalar = p->multiplier_fixedpoint;
-  ep.mult_exponent_scalar = p->multiplier_exponent;
-  ep.dst_zero_point = dst->zero_point;
-  ep.channel_is_col = p->channel_dimension == RUYAMD_CHANNEL_COL;
-  const bool fp = IsFloating(dst->dtype);
-  ep.requantize = !fp && dst->dtype != RUYAMD_DTYPE_I32;
-  if (fp) {
-    ep.clamp_min_f = static_cast<float>(p->clamp_min);
-    ep.clamp_max_f = static_cast<float>(p->clamp_max);
-    ep.clamp_min_d = p->clamp_min;
-    ep.clamp_max_d = p->clamp_max;
-  } else if (dst->dtype == RUYAMD_DTYPE_I32) {
-    // ruy/mul_params.h:291-293: no clamping of raw accumulators.
-    ep.clamp_min_i = std::numeric_limits<int32_t>::lowest();
-    ep.clamp_max_i = std::numeric_limits<int32_t>::max();
-  } else {
-    ep.clamp_min_i = ClampToInt32(p->clamp_min);
-    ep.clamp_max_i = ClampToInt32(p->clamp_max);
-  }
 
   std::string err;
   const int rc = RunMul(ctx, &call, &err);
@@ -343,6 +353,100 @@ using namespace ruyamd;
 extern "C" int ruyamd_mul(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
                           const ruyamd_mul_params* p, const ruyamd_mat* dst) {
   return MulImpl(ctx, lhs, rhs, p, dst, /*no_alloc=*/false);
+}
+
+namespace ruyamd {
+namespace {
+
+bool SameDescriptor(const ruyamd_mat& a, const ruyamd_mat& b) {
+  return a.rows == b.rows && a.cols == b.cols && a.stride == b.stride && a.zero_point == b.zero_point &&
+         a.order == b.order && a.dtype == b.dtype && a.cache_policy == b.cache_policy;
+}
+
+bool SameParams(const ruyamd_mul_params& a, const ruyamd_mul_params& b) {
+  return (a.bias != nullptr) == (b.bias != nullptr) &&
+         (a.multiplier_fixedpoint_perchannel != nullptr) == (b.multiplier_fixedpoint_perchannel != nullptr) &&
+         (a.multiplier_exponent_perchannel != nullptr) == (b.multiplier_exponent_perchannel != nullptr) &&
+         a.multiplier_fixedpoint == b.multiplier_fixedpoint && a.multiplier_exponent == b.multiplier_exponent &&
+         a.clamp_min == b.clamp_min && a.clamp_max == b.clamp_max && a.accum_dtype == b.accum_dtype &&
+         a.channel_dimension == b.channel_dimension;
+}
+
+// The single-launch form of a batch: every product validated, all of one shape
+// and parameter set, every buffer device memory. *handled says whether the
+// batch was enqueued that way.
+int TryBatchLaunch(ruyamd_ctx* ctx, int n, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
+                   const ruyamd_mul_params* params, const ruyamd_mat* dst, bool* handled) {
+  *handled = false;
+  for (int i = 0; i < n; ++i) {
+    if (int rc = Validate(ctx, &lhs[i], &rhs[i], &params[i], &dst[i])) return rc;
+    if (i > 0 && !(SameDescriptor(lhs[i], lhs[0]) && SameDescriptor(rhs[i], rhs[0]) &&
+                   SameDescriptor(dst[i], dst[0]) && SameParams(params[i], params[0])))
+      return RUYAMD_OK;
+  }
+  if (dst[0].rows == 0 || dst[0].cols == 0) return RUYAMD_OK;
+  if (!(ruyamd_ctx_get_runtime_enabled_paths(ctx) & RUYAMD_PATH_GFX950)) return RUYAMD_OK;  // the loop reports it
+  int current_device = -1;
+  if (hipGetDevice(&current_device) != hipSuccess || current_device != ctx->device) {
+    if (hipSetDevice(ctx->device) != hipSuccess) return Fail(ctx, RUYAMD_E_HIP, "hipSetDevice failed");
+  }
+  std::vector<BatchBuffers> items(static_cast<std::size_t>(n));
+  for (int i = 0; i < n; ++i) {
+    const void* pointers[] = {lhs[i].data, rhs[i].data, dst[i].data, params[i].bias,
+                              params[i].multiplier_fixedpoint_perchannel, params[i].multiplier_exponent_perchannel};
+    for (const void* ptr : pointers)
+      if (ptr && !IsDevicePointer(ptr)) return RUYAMD_OK;
+    items[i].lhs = lhs[i].data;
+    items[i].rhs = rhs[i].data;
+    items[i].dst = dst[i].data;
+    items[i].bias = params[i].bias;
+    items[i].mult_fixedpoint = params[i].multiplier_fixedpoint_perchannel;
+    items[i].mult_exponent = params[i].multiplier_exponent_perchannel;
+  }
+  MulCall first;
+  FillCall(lhs[0], rhs[0], params[0], dst[0], params[0].bias, params[0].multiplier_fixedpoint_perchannel,
+           params[0].multiplier_exponent_perchannel, dst[0].data, &first);
+  CaptureScope capture_scope(ctx);  // (timing is skipped while the stream records a graph)
+  std::string err;
+  if (int rc = RunMulBatch(ctx, first, items.data(), n, handled, &err)) return Fail(ctx, rc, err);
+  if (!*handled) return RUYAMD_OK;
+  ctx->last_used_path = RUYAMD_PATH_GFX950;
+  if (ctx->synchronous && !ctx->capturing) {
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess)
+      return Fail(ctx, RUYAMD_E_HIP, std::string("kernel execution failed: ") + hipGetErrorString(hipGetLastError()));
+  }
+  return RUYAMD_OK;
+}
+
+}  // namespace
+}  // namespace ruyamd
+
+extern "C" int ruyamd_mul_batch(ruyamd_ctx* ctx, int n, const ruyamd_mat* lhs, const ruyamd_mat* rhs,
+                                const ruyamd_mul_params* params, const ruyamd_mat* dst) {
+  if (!ctx || n < 0) return RUYAMD_E_INVALID;
+  if (n == 0) return RUYAMD_OK;
+  if (!lhs || !rhs || !params || !dst) return Fail(ctx, RUYAMD_E_INVALID, "null argument");
+  ctx->performance_advisories = 0;
+  bool handled = false;
+  if (int rc = TryBatchLaunch(ctx, n, lhs, rhs, params, dst, &handled)) return rc;
+  if (handled) return RUYAMD_OK;
+  // Anything else: the products one after another on the stream, with one
+  // wait at the end instead of one per product.
+  const bool synchronous = ctx->synchronous;
+  ctx->synchronous = false;
+  int advisories = 0, rc = RUYAMD_OK;
+  for (int i = 0; i < n && rc == RUYAMD_OK; ++i) {
+    rc = MulImpl(ctx, &lhs[i], &rhs[i], &params[i], &dst[i], /*no_alloc=*/false);
+    advisories |= ctx->performance_advisories;
+  }
+  ctx->synchronous = synchronous;
+  ctx->performance_advisories = advisories;
+  if (rc != RUYAMD_OK) return rc;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  const bool capturing = hipStreamIsCapturing(ctx->stream, &status) == hipSuccess && status == hipStreamCaptureStatusActive;
+  if (synchronous && !capturing && hipStreamSynchronize(ctx->stream) != hipSuccess)
+    return Fail(ctx, RUYAMD_E_HIP, std::string("kernel execution failed: ") + hipGetErrorString(hipGetLastError()));
+  return RUYAMD_OK;
 }
 
 extern "C" int ruyamd_mul_no_alloc(ruyamd_ctx* ctx, const ruyamd_mat* lhs, const ruyamd_mat* rhs,

@@ -113,6 +113,19 @@ int LaunchPendingPacks8(ruyamd_ctx* ctx, PendingPack8* a, PendingPack8* b, std::
   return RUYAMD_OK;
 }
 
+// In place: already int8 (or uint8 that the kernel flips on the way in, if the
+// depth is a whole number of `u8_depth_step`; 0 = never), depth-contiguous,
+// 16-byte aligned base and pitch, depth a multiple of 16, and small enough for
+// a buffer descriptor.
+bool UsableInPlace8(const PackSource& src, int u8_depth_step) {
+  const int32_t K = src.K;
+  const bool is_u8 = src.dtype == RUYAMD_DTYPE_U8;
+  const uint64_t extent = src.count > 0 ? uint64_t(src.count - 1) * uint64_t(src.stride_c) + K : 0;
+  const bool u8_ok = !is_u8 || (u8_depth_step > 0 && K % u8_depth_step == 0);
+  return u8_ok && src.stride_k == 1 && K % 16 == 0 && K > 0 && (reinterpret_cast<uintptr_t>(src.data) & 15) == 0 &&
+         (src.stride_c % 16 == 0 || src.count == 1) && extent < (uint64_t(1) << 31);
+}
+
 // Prepares one side: from the cache, in place, or packed into the workspace
 // (with `defer`, that pack is only set up, for LaunchPendingPacks8).
 // `src` views the side as `count` depth vectors (LHS rows / RHS columns).
@@ -185,13 +198,8 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
 
   if (int rc = EnsureOnDevice(ctx, call, side, err)) return rc;
   src = view();
-  // In place: already int8, depth-contiguous, 16-byte aligned base and pitch,
-  // depth a multiple of 16, and small enough for a buffer descriptor.
   const uint64_t extent = src.count > 0 ? uint64_t(src.count - 1) * uint64_t(src.stride_c) + K : 0;
-  const bool u8_ok = !is_u8 || (u8_depth_step > 0 && K % u8_depth_step == 0);
-  const bool direct = u8_ok && src.stride_k == 1 && K % 16 == 0 && K > 0 &&
-                      (reinterpret_cast<uintptr_t>(src.data) & 15) == 0 &&
-                      (src.stride_c % 16 == 0 || src.count == 1) && extent < (uint64_t(1) << 31);
+  const bool direct = UsableInPlace8(src, u8_depth_step);
   if (direct) {
     out->data = static_cast<const int8_t*>(src.data);
     out->ld = src.count == 1 ? ld : static_cast<int32_t>(src.stride_c);
@@ -245,6 +253,50 @@ void PlanDepthSplit(ruyamd_ctx* ctx, GemmKind kind, GemmArgs* args) {
   args->split_k = split.parts;
   args->split_partials = partials;
   args->split_counters = counters;
+}
+
+// Arguments of the tiled int8 kernel for prepared operands `a` (LHS) and `b`
+// (RHS), everything but the sums arrays and the depth split. Returns whether
+// the operands were swapped (row-major destination). When sums are pending on
+// operands used in place and the problem runs on the smallest tile,
+// args->fuse_sums is set: the kernel forms them itself (one launch instead of
+// two or three) and the zero point that multiplies a side's sums moves from
+// the write-back to the fused factor.
+bool SetupInt8Gemm(ruyamd_ctx* ctx, const MulCall& call, const Operand8& a, const Operand8& b, int32_t lzp,
+                   int32_t rzp, GemmArgs* out) {
+  GemmArgs& args = *out;
+  const int M = call.lhs.rows, K = call.lhs.cols, N = call.rhs.cols;
+  args.k_bytes = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
+  const bool swap = SetupDestination(call, &args);
+  args.ep.zp_product_depth =
+      static_cast<int32_t>(static_cast<uint32_t>(lzp) * static_cast<uint32_t>(rzp) * static_cast<uint32_t>(K));
+  const Operand8& x = swap ? b : a;
+  const Operand8& y = swap ? a : b;
+  args.a = x.data;
+  args.b = y.data;
+  args.a_bytes = x.bytes;
+  args.b_bytes = y.bytes;
+  args.lda = x.ld;
+  args.ldb = y.ld;
+  args.a_flip = x.flip;
+  args.b_flip = y.flip;
+  args.M = swap ? N : M;
+  args.N = swap ? M : N;
+  args.n_logical = args.N;
+  args.ep.lhs_zero_point = swap ? rzp : lzp;
+  args.ep.rhs_zero_point = swap ? lzp : rzp;
+  if ((a.sums_pending || b.sums_pending) && GemmI8CanFuseSums(args, ctx->multiprocessor_count)) {
+    args.fuse_sums = 1;
+    if (x.sums_pending) {
+      args.fused_a_factor = args.ep.rhs_zero_point;
+      args.ep.rhs_zero_point = 0;
+    }
+    if (y.sums_pending) {
+      args.fused_b_factor = args.ep.lhs_zero_point;
+      args.ep.lhs_zero_point = 0;
+    }
+  }
+  return swap;
 }
 
 int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
@@ -326,43 +378,13 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     return RUYAMD_OK;
   }
   GemmArgs args;
-  args.k_bytes = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
-  const bool swap = SetupDestination(*call, &args);
-  args.ep.zp_product_depth = zp_product_depth;
-  const Operand8& x = swap ? b : a;
-  const Operand8& y = swap ? a : b;
-  args.a = x.data;
-  args.b = y.data;
-  args.a_bytes = x.bytes;
-  args.b_bytes = y.bytes;
-  args.lda = x.ld;
-  args.ldb = y.ld;
-  args.a_flip = x.flip;
-  args.b_flip = y.flip;
-  args.M = swap ? N : M;
-  args.N = swap ? M : N;
-  args.n_logical = args.N;
-  args.ep.lhs_zero_point = swap ? rzp : lzp;
-  args.ep.rhs_zero_point = swap ? lzp : rzp;
-  if ((a.sums_pending || b.sums_pending) && GemmI8CanFuseSums(args, ctx->multiprocessor_count)) {
-    // A small problem on operands used in place: the kernel forms the pending
-    // sums itself (one launch instead of two or three). The zero point that
-    // multiplies a side's sums moves from the write-back to the fused factor.
-    args.fuse_sums = 1;
-    if (x.sums_pending) {
-      args.fused_a_factor = args.ep.rhs_zero_point;
-      args.ep.rhs_zero_point = 0;
-    }
-    if (y.sums_pending) {
-      args.fused_b_factor = args.ep.lhs_zero_point;
-      args.ep.lhs_zero_point = 0;
-    }
-  } else {
+  const bool swap = SetupInt8Gemm(ctx, *call, a, b, lzp, rzp, &args);
+  if (!args.fuse_sums) {
     if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
     if (int rc = MaterializeSums(ctx, &b, K, err)) return rc;
   }
-  args.ep.lhs_sums = x.sums;
-  args.ep.rhs_sums = y.sums;
+  args.ep.lhs_sums = (swap ? b : a).sums;
+  args.ep.rhs_sums = (swap ? a : b).sums;
   PlanDepthSplit(ctx, GemmKind::kInt8, &args);
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
@@ -694,6 +716,73 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
 }
 
 }  // namespace
+
+int RunMulBatch(ruyamd_ctx* ctx, const MulCall& first, const BatchBuffers* items, int n, bool* handled,
+                std::string* err) {
+  *handled = false;
+  const DevMat& lhs = first.lhs;
+  const DevMat& rhs = first.rhs;
+  const int M = lhs.rows, K = lhs.cols, N = rhs.cols;
+  if (ctx->force_generic || n < 1 || !Is8Bit(lhs.dtype) || !Is8Bit(rhs.dtype)) return RUYAMD_OK;
+  if (M <= kSkinnyKernelWidth || N <= kSkinnyKernelWidth || K <= 0) return RUYAMD_OK;
+  if (ShouldCache(first.lhs_cache_policy, N) || ShouldCache(first.rhs_cache_policy, M)) return RUYAMD_OK;
+  GemmArgs shape;
+  shape.M = M;
+  shape.N = N;
+  if (!GemmI8CanFuseSums(shape, ctx->multiprocessor_count)) return RUYAMD_OK;  // not the smallest tile
+  const int u8_depth_step = 128;
+  const int32_t lzp = lhs.dtype == RUYAMD_DTYPE_U8 ? lhs.zero_point - 128 : lhs.zero_point;
+  const int32_t rzp = rhs.dtype == RUYAMD_DTYPE_U8 ? rhs.zero_point - 128 : rhs.zero_point;
+  // Every product's operands must be usable where they lie (a packed copy or a
+  // sums array would be scratch memory per product).
+  for (int z = 0; z < n; ++z) {
+    const PackSource l{items[z].lhs, lhs.rs, lhs.cs, lhs.rows, lhs.cols, lhs.dtype};
+    const PackSource r{items[z].rhs, rhs.cs, rhs.rs, rhs.cols, rhs.rows, rhs.dtype};
+    if (!UsableInPlace8(l, u8_depth_step) || !UsableInPlace8(r, u8_depth_step)) return RUYAMD_OK;
+  }
+  auto in_place = [&](const DevMat& m, int count, int64_t stride_c, bool need_sums) {
+    Operand8 op;
+    op.data = static_cast<const int8_t*>(m.data);
+    op.ld = count == 1 ? RoundUp(K, 16) : static_cast<int32_t>(stride_c);
+    op.bytes = static_cast<uint32_t>(uint64_t(count - 1) * uint64_t(stride_c) + K);
+    op.sums_pending = need_sums;
+    op.count = count;
+    op.flip = m.dtype == RUYAMD_DTYPE_U8 ? kFlipU8 : 0;
+    return op;
+  };
+  const Operand8 a = in_place(lhs, M, lhs.rs, rzp != 0);
+  const Operand8 b = in_place(rhs, N, rhs.cs, lzp != 0);
+  GemmArgs args;
+  const bool swap = SetupInt8Gemm(ctx, first, a, b, lzp, rzp, &args);
+  if ((a.sums_pending || b.sums_pending) && !args.fuse_sums) return RUYAMD_OK;
+  // 16-byte stores need every product's destination aligned, not only the first one's.
+  for (int z = 0; z < n; ++z)
+    if (reinterpret_cast<uintptr_t>(items[z].dst) & 15) args.dst_vector_ok = 0;
+  const bool timed = ctx->TimingBegin();
+  hipError_t launched = hipSuccess;
+  for (int z0 = 0; z0 < n && launched == hipSuccess; z0 += kGemmBatchMax) {
+    const int count = std::min(kGemmBatchMax, n - z0);
+    GemmBatch batch = {};
+    for (int z = 0; z < count; ++z) {
+      const BatchBuffers& it = items[z0 + z];
+      batch.a[z] = swap ? it.rhs : it.lhs;
+      batch.b[z] = swap ? it.lhs : it.rhs;
+      batch.dst[z] = it.dst;
+      batch.bias[z] = it.bias;
+      batch.mult_fixedpoint[z] = it.mult_fixedpoint;
+      batch.mult_exponent[z] = it.mult_exponent;
+    }
+    launched = LaunchGemmI8Batch(ctx->stream, args, batch, count, ctx->multiprocessor_count);
+  }
+  if (timed) ctx->TimingEnd();
+  if (launched != hipSuccess) {
+    *err = "batched int8 MFMA kernel launch failed";
+    return RUYAMD_E_HIP;
+  }
+  ctx->last_kernel = RUYAMD_KERNEL_I8_MFMA;
+  *handled = true;
+  return RUYAMD_OK;
+}
 
 int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
   DevMat& m = side == 0 ? call->lhs : call->rhs;

@@ -36,6 +36,26 @@ int EnsureOnDevice(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err);
 // ctx->stream. Returns a RUYAMD_* code; on failure *err holds the reason.
 int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err);
 
+// The buffers of one product of a batch (device memory; null where the batch
+// has no such buffer).
+struct BatchBuffers {
+  const void* lhs = nullptr;
+  const void* rhs = nullptr;
+  void* dst = nullptr;
+  const void* bias = nullptr;
+  const int32_t* mult_fixedpoint = nullptr;
+  const int32_t* mult_exponent = nullptr;
+};
+
+// `n` products that agree with `first` in everything but where their buffers
+// lie (items[0] holds the buffers of `first` itself): runs them as single
+// launches of up to 32 products each if they qualify - 8-bit operands usable in
+// place, a shape that runs on the smallest tile of the tiled kernel, no cache
+// policy in effect - and sets *handled. Otherwise nothing has been enqueued
+// and *handled is false.
+int RunMulBatch(ruyamd_ctx* ctx, const MulCall& first, const BatchBuffers* items, int n, bool* handled,
+                std::string* err);
+
 }  // namespace ruyamd
 
 #endif  // RUY_AMD_CSRC_PLAN_H_

@@ -80,6 +80,15 @@ class DeviceProblem:
         return everything[self.guard:self.guard + self.n_dst].copy()
 
 
+def run_batch(ctx, device_problems):
+    """One ruyamd_mul_batch call over the given DeviceProblems."""
+    n = len(device_problems)
+    ls, rs, ps, ds = (S.Mat * n)(), (S.Mat * n)(), (S.MulParamsStruct * n)(), (S.Mat * n)()
+    for i, dp in enumerate(device_problems):
+        ls[i], rs[i], ps[i], ds[i] = dp.lhs_s, dp.rhs_s, dp.par_s, dp.dst_s
+    ctx._check(api.lib.ruyamd_mul_batch(ctx._h, n, ls, rs, ps, ds))
+
+
 def device_mul(ctx, problem, dst_fill=0x5A, misalign=0, entry=None):
     """dst storage (numpy, same layout as problem.dst) computed on the GPU from
     device-resident operands; untouched elements keep the fill byte."""
