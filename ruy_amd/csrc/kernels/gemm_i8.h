@@ -106,6 +106,16 @@ hipError_t LaunchGemmF32(hipStream_t stream, const GemmArgs& args, int num_cus);
 bool GemmI8I16CanFuseSums(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus);
 
+// The same product with `b` the int16 operand itself, used in place (no
+// LaunchPackI16Split): depth-contiguous, base and pitch 16-byte aligned, a
+// depth that is a multiple of 16; ldb and b_bytes count bytes of int16 data, N
+// still counts plane vectors (64 per 32 columns, as if packed) and n_logical
+// the columns. Exists for launches on the smallest tile whose parts have at
+// least two depth steps each (GemmI8I16CanUseRawInt16, asked after split_k
+// has been set).
+bool GemmI8I16CanUseRawInt16(const GemmArgs& args, int num_cus);
+hipError_t LaunchGemmI8I16Raw(hipStream_t stream, const GemmArgs& args, int num_cus);
+
 // Skinny multiplication: `rows` wide-side vectors against narrow_count <= 16
 // narrow-side vectors, all depth-contiguous int8 with the same alignment rules
 // as GemmI8Args. `swapped` = 0: the wide side is the LHS (rows of dst), the

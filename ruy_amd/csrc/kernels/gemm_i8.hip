@@ -28,6 +28,7 @@ struct Int8Traits {
   }
   static __device__ __forceinline__ void DrainMma() {}
   static constexpr int kBlock = 32;
+  static constexpr bool kRawB = false;
   // The 256x256 tile runs on 16x16 blocks (below).
   using LargeTile = Int8Traits16;
   static constexpr bool kSplitB = false;
@@ -154,6 +155,14 @@ struct Int8SplitTraits : Int8Traits {
   }
 };
 
+// The same with the int16 operand read where it lies and split into its planes
+// on the way from LDS to the matrix instructions (smallest tile, depth dealt
+// to the waves): no pack launch.
+struct Int8SplitRawTraits : Int8SplitTraits {
+  using LargeTile = Int8SplitRawTraits;
+  static constexpr bool kRawB = true;
+};
+
 }  // namespace
 
 bool GemmI8I16CanFuseSums(const GemmArgs& args, int num_cus) {
@@ -166,6 +175,19 @@ hipError_t LaunchGemmI8I16(hipStream_t stream, const GemmArgs& args, int num_cus
     return mfma_gemm::LaunchSmallestTile<Int8SplitTraits, true>(stream, args);
   }
   return mfma_gemm::LaunchBest<Int8SplitTraits>(stream, args, num_cus);
+}
+
+bool GemmI8I16CanUseRawInt16(const GemmArgs& args, int num_cus) {
+  if (!GemmI8I16CanFuseSums(args, num_cus)) return false;  // not the smallest tile
+  const int k_tiles = (args.k_bytes + 127) / 128;
+  const int parts = args.split_k > 1 ? args.split_k : 1;
+  return (k_tiles + parts - 1) / parts >= 2;  // the schedule that deals the depth to the waves
+}
+
+hipError_t LaunchGemmI8I16Raw(hipStream_t stream, const GemmArgs& args, int num_cus) {
+  if (!GemmI8I16CanUseRawInt16(args, num_cus)) return hipErrorInvalidValue;
+  return args.fuse_sums ? mfma_gemm::Launch<Int8SplitRawTraits, 1, 2, 128, 4, true, false, true>(stream, args)
+                        : mfma_gemm::Launch<Int8SplitRawTraits, 1, 2, 128, 4, false, false, true>(stream, args);
 }
 
 DepthSplit GemmDepthSplit(const GemmArgs& args, int num_cus, GemmKind kind) {

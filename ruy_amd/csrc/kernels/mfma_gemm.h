@@ -448,6 +448,17 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // d, d+2, ... The partial pieces are added through LDS afterwards, which
     // leaves wave (wave_m, wave_n) with its WM x WN blocks as in the other
     // schedule.
+    //
+    // Traits::kRawB (plane-split kernel only): `b` is the int16 operand itself,
+    // depth-contiguous, ldb and b_bytes in bytes of int16 data, and N still
+    // counts plane vectors (64 per 32 columns of it). A depth step of a column
+    // is then 256 bytes, brought into LDS as they are; the two int8 planes
+    // (high byte; low byte with its top bit flipped, i.e. minus 128) are cut
+    // out of the fragment reads with v_perm_b32, so there is no pack kernel.
+    // Bytes past the depth read as zero and would give a low plane of -128,
+    // which does not matter: the `a` fragments they meet are zero.
+    constexpr bool kRawB = Traits::kRawB;
+    static_assert(!kRawB || Traits::kSplitB, "");
     constexpr int kColWays = Traits::kSplitB ? 2 : 1;
     constexpr int kDepthWays = 4 / kColWays;
     const int depth_way = wave / kColWays;
@@ -465,23 +476,39 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       const int r = (n % 8) * 8 + lane / 8;  // row inside its operand's tile
       const int g = (lane % 8) ^ Swizzle<BK>(r);
       gk[n] = g * kGranule;
-      if (n < 8)
+      if (n < 8) {
         goff[n] = m0 + r < args.M ? uint32_t(m0 + r) * uint32_t(args.lda) + g * kGranule : kOutOfRange;
-      else
+      } else if constexpr (!kRawB) {
         goff[n] = n0 + col_way * 64 + r < args.N
                       ? uint32_t(n0 + col_way * 64 + r) * uint32_t(args.ldb) + g * kGranule
                       : kOutOfRange;
+      } else {
+        // Load n fills the 256-byte depth runs of columns 4*(n-8) .. +3 of this
+        // wave's 32 columns, 16 granules each, swizzled by the column number.
+        const int rb = (n - 8) * 4 + lane / 16;
+        const int gb = (lane % 16) ^ (rb & 15);
+        const int col = n0 / 2 + col_way * 32 + rb;
+        gk[n] = gb * kGranule;
+        goff[n] = col < args.n_logical ? uint32_t(col) * uint32_t(args.ldb) + gb * kGranule : kOutOfRange;
+      }
     }
+    // Depth offset and limit of the b operand in bytes: twice those of `a`
+    // when it is int16 data.
+    constexpr int kBScale = kRawB ? 2 : 1;
     auto issue_step = [&](int step, int slot) {
       const int kbase = phys(step) * kBK;
       const uint32_t dst = ring_base + slot * kSlotBytes;
       if (kbase + kBK <= K) {
 #pragma unroll
-        for (int n = 0; n < kLoads; ++n) LoadToLds16(dst + n * 1024, goff[n], uint32_t(kbase), n < 8 ? a_rsrc : b_rsrc);
+        for (int n = 0; n < kLoads; ++n)
+          LoadToLds16(dst + n * 1024, goff[n], uint32_t(n < 8 ? kbase : kBScale * kbase), n < 8 ? a_rsrc : b_rsrc);
       } else {
 #pragma unroll
-        for (int n = 0; n < kLoads; ++n)
-          LoadToLds16(dst + n * 1024, kbase + gk[n] < K ? goff[n] + kbase : kOutOfRange, n < 8 ? a_rsrc : b_rsrc);
+        for (int n = 0; n < kLoads; ++n) {
+          const int scale = n < 8 ? 1 : kBScale;
+          LoadToLds16(dst + n * 1024, scale * kbase + gk[n] < scale * K ? goff[n] + scale * kbase : kOutOfRange,
+                      n < 8 ? a_rsrc : b_rsrc);
+        }
       }
     };
     struct Frags4 {
@@ -494,7 +521,27 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         f.a[i] = *reinterpret_cast<const v4i*>(base + off + i * 32 * kBK);
-        f.b[i] = *reinterpret_cast<const v4i*>(base + 64 * kBK + off + i * 32 * kBK);
+        if constexpr (!kRawB) f.b[i] = *reinterpret_cast<const v4i*>(base + 64 * kBK + off + i * 32 * kBK);
+      }
+      if constexpr (kRawB) {
+        // The lane's 16 depth values of column frag_row are 32 bytes of int16
+        // data: granules 4*ks + 2*frag_half and the next one of that column.
+        const char* col = base + 64 * kBK + frag_row * 256;
+        const int g0 = ks * 4 + frag_half * 2;
+        const v4i first = *reinterpret_cast<const v4i*>(col + (((g0) ^ (frag_row & 15)) << 4));
+        const v4i second = *reinterpret_cast<const v4i*>(col + (((g0 + 1) ^ (frag_row & 15)) << 4));
+        // Even bytes are the low bytes, odd bytes the high bytes (little endian).
+        v4i high, low;
+        high[0] = __builtin_amdgcn_perm(first[1], first[0], 0x07050301);
+        high[1] = __builtin_amdgcn_perm(first[3], first[2], 0x07050301);
+        high[2] = __builtin_amdgcn_perm(second[1], second[0], 0x07050301);
+        high[3] = __builtin_amdgcn_perm(second[3], second[2], 0x07050301);
+        low[0] = __builtin_amdgcn_perm(first[1], first[0], 0x06040200) ^ int(0x80808080u);
+        low[1] = __builtin_amdgcn_perm(first[3], first[2], 0x06040200) ^ int(0x80808080u);
+        low[2] = __builtin_amdgcn_perm(second[1], second[0], 0x06040200) ^ int(0x80808080u);
+        low[3] = __builtin_amdgcn_perm(second[3], second[2], 0x06040200) ^ int(0x80808080u);
+        f.b[0] = high;  // the high plane's 32 vectors come first in the packed form, too
+        f.b[1] = low;
       }
     };
     typename Traits::Acc full[2][2], rows_sum[2], cols_sum[2];

@@ -665,11 +665,65 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
       planes = static_cast<int8_t*>(pm.data);
     }
   }
+  // Common arguments (the operand-b fields follow below).
+  args.k_bytes = RoundUp(K, 16);
+  args.a = a.data;
+  args.a_bytes = a.bytes;
+  args.lda = a.ld;
+  args.M = swap ? N : M;
+  args.N = n_phys;
+  args.n_logical = src.count;
+  args.ep.rhs_sums = nullptr;
+  args.ep.lhs_zero_point = 0;
+  args.ep.rhs_zero_point = -128;  // the low plane stores (v & 0xff) - 128
+  args.ep.zp_product_depth = 0;
+  bool fuse_decided = false;
+  auto decide_sums = [&]() -> int {
+    if (fuse_decided) return RUYAMD_OK;
+    fuse_decided = true;
+    if (a.sums_pending && GemmI8I16CanFuseSums(args, ctx->multiprocessor_count)) {
+      // Small problem, int8 side used in place: the kernel forms its row sums.
+      args.fuse_sums = 1;
+      args.fused_a_factor = args.ep.rhs_zero_point;
+      args.ep.rhs_zero_point = 0;
+    } else if (int rc = MaterializeSums(ctx, &a, K, err)) {
+      return rc;
+    }
+    args.ep.lhs_sums = a.sums;
+    return RUYAMD_OK;
+  };
   if (!planes) {
     if (int rc = EnsureOnDevice(ctx, call, side16, err)) return rc;
     const DevMat& m = side16 == 0 ? call->lhs : call->rhs;
     const PackSource fresh = side16 == 0 ? PackSource{m.data, m.rs, m.cs, m.rows, m.cols, m.dtype}
                                          : PackSource{m.data, m.cs, m.rs, m.cols, m.rows, m.dtype};
+    // The int16 operand where it lies, split into planes inside the kernel: no
+    // pack launch. Needs the layout of an in-place operand and a launch on the
+    // smallest tile with at least two depth steps per part.
+    const uint64_t extent16 = fresh.count > 0 ? (uint64_t(fresh.count - 1) * uint64_t(fresh.stride_c) + K) * 2 : 0;
+    const bool layout_ok = fresh.stride_k == 1 && K % 16 == 0 && K > 0 &&
+                           (reinterpret_cast<uintptr_t>(fresh.data) & 15) == 0 &&
+                           ((fresh.stride_c * 2) % 16 == 0 || fresh.count == 1) && extent16 < (uint64_t(1) << 31);
+    if (layout_ok) {
+      args.b = fresh.data;
+      args.b_bytes = static_cast<uint32_t>(extent16);
+      args.ldb = fresh.count == 1 ? RoundUp(K, 16) * 2 : static_cast<int32_t>(fresh.stride_c * 2);
+      if (int rc = decide_sums()) return rc;
+      PlanDepthSplit(ctx, GemmKind::kInt8Int16, &args);
+      if (GemmI8I16CanUseRawInt16(args, ctx->multiprocessor_count)) {
+        const bool timed = ctx->TimingBegin();
+        const hipError_t launched = LaunchGemmI8I16Raw(ctx->stream, args, ctx->multiprocessor_count);
+        if (timed) ctx->TimingEnd();
+        if (launched != hipSuccess) {
+          *err = "int8 x int16 matrix-core kernel launch failed";
+          return RUYAMD_E_HIP;
+        }
+        ctx->last_kernel = RUYAMD_KERNEL_I8I16_MFMA;
+        return RUYAMD_OK;
+      }
+      // Not that launch after all: the planes are packed as usual. (A depth
+      // split planned above stays valid: it depends on the shape only.)
+    }
     planes = static_cast<int8_t*>(ctx->ws->Alloc(packed_bytes));
     if (!planes) {
       *err = "workspace allocation failed";
@@ -680,30 +734,11 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
       return RUYAMD_E_HIP;
     }
   }
-  args.k_bytes = RoundUp(K, 16);
-  args.a = a.data;
-  args.a_bytes = a.bytes;
-  args.lda = a.ld;
   args.b = planes;
   args.b_bytes = static_cast<uint32_t>(packed_bytes);
   args.ldb = ld;
-  args.M = swap ? N : M;
-  args.N = n_phys;
-  args.n_logical = src.count;
-  args.ep.rhs_sums = nullptr;
-  args.ep.lhs_zero_point = 0;
-  args.ep.rhs_zero_point = -128;  // the low plane stores (v & 0xff) - 128
-  args.ep.zp_product_depth = 0;
-  if (a.sums_pending && GemmI8I16CanFuseSums(args, ctx->multiprocessor_count)) {
-    // Small problem, int8 side used in place: the kernel forms its row sums.
-    args.fuse_sums = 1;
-    args.fused_a_factor = args.ep.rhs_zero_point;
-    args.ep.rhs_zero_point = 0;
-  } else if (int rc = MaterializeSums(ctx, &a, K, err)) {
-    return rc;
-  }
-  args.ep.lhs_sums = a.sums;
-  PlanDepthSplit(ctx, GemmKind::kInt8Int16, &args);
+  if (int rc = decide_sums()) return rc;
+  if (args.split_k == 1) PlanDepthSplit(ctx, GemmKind::kInt8Int16, &args);
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8I16(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
