@@ -45,6 +45,7 @@
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
+#include <utility>
 
 #include <algorithm>
 
@@ -104,6 +105,16 @@ __device__ __forceinline__ void LoadToLds16(uint32_t lds_base, uint32_t voffset,
       :
       : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
       : "memory");
+}
+
+// f(std::integral_constant<int, 0>()), ..., f(std::integral_constant<int, N - 1>()).
+template <class F, int... Is>
+__device__ __forceinline__ void StaticForEach(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>()), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void StaticFor(F&& f) {
+  StaticForEach(f, std::make_integer_sequence<int, (N > 0 ? N : 0)>());
 }
 
 template <int N>
@@ -395,36 +406,61 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
       for (int r = 0; r < kFrags; ++r) read_one(kt_next, ks_next, r, next);
     }
-#pragma unroll
-    for (int n = 0; n < kMmas; ++n) {
+    // The instruction index and everything derived from it are compile-time
+    // constants (StaticFor), so that register arrays are always indexed by
+    // constants whatever the loop unroller would have made of nested loops.
+    StaticFor<kMmas>([&](auto n_constant) {
+      constexpr int n = decltype(n_constant)::value;
       __builtin_amdgcn_sched_barrier(0);
       Traits::Mma(cur.a[n / kBB], cur.b[n % kBB], acc[n / kBB][n % kBB]);
-      if constexpr (kFusedSums) {
+      if constexpr (kFusedSums && n == 0) {
         // Once per sub-step. The plane-split operand has zero point 0 by
         // definition, so its column sums are never needed.
-        if (n == 0) {
-          Traits::Mma(cur.a[0], ones, sum_a);
-          if constexpr (!Traits::kSplitB) Traits::Mma(ones, cur.b[0], sum_b);
-        }
+        Traits::Mma(cur.a[0], ones, sum_a);
+        if constexpr (!Traits::kSplitB) Traits::Mma(ones, cur.b[0], sum_b);
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (!kReadsFirst && n < kReadSlots) {
-#pragma unroll
-        for (int r = n * kFrags / kReadSlots; r < (n + 1) * kFrags / kReadSlots; ++r)
-          read_one(kt_next, ks_next, r, next);
+      if constexpr (!kReadsFirst && n < kReadSlots) {
+        constexpr int kFirst = n * kFrags / kReadSlots;
+        StaticFor<(n + 1) * kFrags / kReadSlots - kFirst>([&](auto r) {
+          read_one(kt_next, ks_next, kFirst + decltype(r)::value, next);
+        });
       }
       if (kt_dma >= 0) {
-#pragma unroll
-        for (int l = n * C::kLoadsPerStage / kMmas; l < (n + 1) * C::kLoadsPerStage / kMmas; ++l) {
+        constexpr int kFirst = n * C::kLoadsPerStage / kMmas;
+        StaticFor<(n + 1) * C::kLoadsPerStage / kMmas - kFirst>([&](auto l) {
           if (decltype(dma_is_full_step)::value)
-            issue_one_full(kt_dma, l);
+            issue_one_full(kt_dma, kFirst + decltype(l)::value);
           else
-            issue_one(kt_dma, l);
-        }
+            issue_one(kt_dma, kFirst + decltype(l)::value);
+        });
       }
-    }
+    });
     __builtin_amdgcn_sched_barrier(0);
   };
+
+  // ---- what the write-back needs per destination row ----
+  // After the transposition (below) a lane owns 16 consecutive rows of one
+  // column at a time, the same rows for every column it writes: everything
+  // that depends only on the row is gathered once. Rows past the end are
+  // clamped to the last row (their results are never stored) so that the
+  // loads carry no per-lane branches and can all be in flight together. The
+  // largest tile issues these loads here, ahead of the main loop, which hides
+  // their latency (a lone wave per SIMD has nothing else to run while it
+  // waits); the smaller tiles, which live on fewer registers, load them
+  // when the write-back starts.
+  constexpr bool kEarlyRowState = kB == 16;
+  constexpr int kChunksPerCol = WM * 32 / 16;
+  const Epilogue& ep = args.ep;
+  typename Traits::RowState rows;
+  auto load_row_state = [&]() {
+    const int first_row = m0 + wave_m * (WM * 32) + (lane % kChunksPerCol) * 16;
+    int row_idx[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) row_idx[q] = min(first_row + q, args.M - 1);
+    rows.Load(ep, row_idx);
+  };
+  if constexpr (kEarlyRowState) load_row_state();
 
   // ---- software pipeline ----
   // Fragments are double-buffered in registers: while the matrix instructions
@@ -651,26 +687,48 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     __syncthreads();
     Frags f[2];
     read_frags(0, 0, f[0]);
-    auto ring_step = [&](int kt, auto dma_is_full_step) {
+    // The fragments of consecutive sub-steps alternate between f[0] and f[1].
+    // `parity`: which of the two the step's first sub-step finds its fragments
+    // in (always 0 when a ring step has an even number of sub-steps).
+    auto ring_step = [&](int kt, auto dma_is_full_step, auto parity) {
+      constexpr int kParity = decltype(parity)::value;
 #pragma unroll
       for (int ks = 0; ks < C::kKSteps; ++ks) {
+        Frags& cur = f[(kParity + ks) & 1];
+        Frags& next = f[(kParity + ks + 1) & 1];
         if (ks + 1 < C::kKSteps) {
-          sub_step(f[ks & 1], f[(ks + 1) & 1], kt, ks + 1, -1, dma_is_full_step);
+          sub_step(cur, next, kt, ks + 1, -1, dma_is_full_step);
         } else {
           WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
           __syncthreads();
-          sub_step(f[ks & 1], f[0], kt + 1, 0, kt + C::kStages, dma_is_full_step);
+          sub_step(cur, next, kt + 1, 0, kt + C::kStages, dma_is_full_step);
         }
       }
     };
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
     // While the step whose loads are being issued (kt + kStages) lies entirely
     // inside the depth, the cheap form of the loads is used; the last few steps
     // (a partial step and the ones past the end, which fetch zeros) take the
     // bounds-tested form.
     int kt = 0;
     const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
-    for (; kt < full_end; ++kt) ring_step(kt, std::true_type());
-    for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type());
+    if constexpr (C::kKSteps % 2 == 0) {
+      for (; kt < full_end; ++kt) ring_step(kt, std::true_type(), Even());
+      for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type(), Even());
+    } else {
+      // One sub-step per ring step: the steps are taken in pairs, so that each
+      // finds its fragments in a buffer known at compile time.
+      for (; kt + 1 < full_end; kt += 2) {
+        ring_step(kt, std::true_type(), Even());
+        ring_step(kt + 1, std::true_type(), Odd());
+      }
+      for (; kt + 1 < k_tiles; kt += 2) {
+        ring_step(kt, std::false_type(), Even());
+        ring_step(kt + 1, std::false_type(), Odd());
+      }
+      if (kt < k_tiles) ring_step(kt, std::false_type(), Even());
+    }
   }
   Traits::DrainMma();  // (matrix instructions the compiler does not see: let the last ones finish)
   WaitVmcnt<0>();
@@ -768,24 +826,13 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   constexpr int kPitch = C::kEpiloguePitch;  // ints; keeps the b128 writes conflict-free
   constexpr int kHalfCols = C::kEpilogueBlockCols * 32;  // columns staged at a time
   int* region = reinterpret_cast<int*>(lds) + wave * (kHalfCols * kPitch);
-  constexpr int kChunksPerCol = kRows / 16;
   constexpr int kColsPerPass = 64 / kChunksPerCol;
-  const Epilogue& ep = args.ep;
   const int elt = args.dst_elt;
   char* dst_base = static_cast<char*>(args.dst.data);
   const int64_t ldd = args.dst.cs;
   const int chunk = lane % kChunksPerCol;
   const int i0 = m0 + wave_m * kRows + chunk * 16;
-
-  // Everything that depends only on the destination row is the same for all
-  // columns this lane will write: gather it once. Rows past the end are
-  // clamped to the last row (their results are never stored) so that the
-  // loads carry no per-lane branches and can all be in flight together.
-  int row_idx[16];
-#pragma unroll
-  for (int q = 0; q < 16; ++q) row_idx[q] = min(i0 + q, args.M - 1);
-  typename Traits::RowState rows;
-  rows.Load(ep, row_idx);
+  if constexpr (!kEarlyRowState) load_row_state();
 
   // The accumulators go to LDS in straight-line code (their register indices
   // must be compile-time constants); everything after that is a compact loop,
@@ -832,21 +879,44 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       }
     }
     __builtin_amdgcn_wave_barrier();
-#pragma unroll 1
-    for (int pass = 0; pass < kHalfCols / kColsPerPass; ++pass) {
+    // A lone wave per SIMD has nothing to hide an LDS read behind: the 16
+    // values of the next pass are requested before those of this pass are
+    // worked on (except in the 32x32-block kernels with the most accumulators,
+    // which have no registers to spare for it).
+    constexpr bool kReadAhead = kB == 16 || WM * WN <= 4;
+    constexpr int kPassUnroll = kReadAhead ? 2 : 1;
+    constexpr int kPasses = kHalfCols / kColsPerPass;
+    struct Staged {
+      v4i w[4];
+    };
+    auto read_pass = [&](int pass, Staged& into) {
+      const int c = pass * kColsPerPass + lane / kChunksPerCol;
+      const v4i* src = reinterpret_cast<const v4i*>(region + c * kPitch + chunk * 16);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) into.w[q] = src[q];
+    };
+    Staged ahead;
+    if constexpr (kReadAhead) read_pass(0, ahead);
+#pragma unroll kPassUnroll
+    for (int pass = 0; pass < kPasses; ++pass) {
+      Staged now;
+      if constexpr (kReadAhead) {
+        now = ahead;
+        if (pass + 1 < kPasses) read_pass(pass + 1, ahead);
+      } else {
+        read_pass(pass, now);
+      }
       const int c = pass * kColsPerPass + lane / kChunksPerCol;  // column inside the staged half
       const int j = (Traits::kSplitB ? n0 / 2 : n0) +
                     (wave_n * C::kLogicalWN + half * C::kEpilogueBlockCols) * 32 + c;
       if (j >= args.n_logical || i0 >= args.M) continue;
       int32_t vals[16];
-      const v4i* src = reinterpret_cast<const v4i*>(region + c * kPitch + chunk * 16);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const v4i w = src[q];
-        vals[4 * q + 0] = w[0];
-        vals[4 * q + 1] = w[1];
-        vals[4 * q + 2] = w[2];
-        vals[4 * q + 3] = w[3];
+        vals[4 * q + 0] = now.w[q][0];
+        vals[4 * q + 1] = now.w[q][1];
+        vals[4 * q + 2] = now.w[q][2];
+        vals[4 * q + 3] = now.w[q][3];
       }
       Traits::Finish(vals, rows, j, ep);
       const bool full = i0 + 16 <= args.M;
