@@ -469,16 +469,16 @@ def bench_other_configs(ctx, args):
     out = []
     ctx.set_kernel_timing(False)  # a per-launch event pair would dominate these short steps
     configs = [
-        ("C1 int8 256^3", W.config_int8_gemm(256), "mfma-int8",
+        ("C1 int8 256^3", W.config_int8_gemm(256), "mfma-int8", "c1_int8_256",
          "launch-bound: 33.6 Mop in one launch, smaller than the time to start a kernel"),
-        ("C2 fp32 1024^3", W.config_f32_gemm(1024), "mfma-f32", None),
-        ("C2 fp32 1024^3 relu6", W.config_f32_gemm(1024, relu6=True), "mfma-f32", None),
-        ("C3 int8 per-channel 1024x1024x196", W.config_int8_perchannel_conv(), "mfma-int8",
+        ("C2 fp32 1024^3", W.config_f32_gemm(1024), "mfma-f32", "c2_f32_1024", None),
+        ("C2 fp32 1024^3 relu6", W.config_f32_gemm(1024, relu6=True), "mfma-f32", "c2_f32_1024", None),
+        ("C3 int8 per-channel 1024x1024x196", W.config_int8_perchannel_conv(), "mfma-int8", "c3_int8_perchannel",
          "launch-bound: 0.41 Gop, 64 tiles of 64x64 for 256 CUs"),
-        ("C4 int8xint16 2048x2048x512", W.config_int8_int16(), "mfma-int8",
+        ("C4 int8xint16 2048x2048x512", W.config_int8_int16(), "mfma-int8", "c4_int8_int16",
          "operations counted once although the int16 operand takes two int8 matrix-instruction passes"),
     ]
-    for name, problem, bound, note in configs:
+    for name, problem, bound, traffic_key, note in configs:
         dp = device_problem(problem)
         dp.run(ctx)
         kernel = ctx.last_kernel_name()
@@ -494,7 +494,8 @@ def bench_other_configs(ctx, args):
                  "us_per_step_min": t["step_min_s"] * 1e6, "us_per_step_median": t["step_median_s"] * 1e6,
                  unit: ops / t["step_s"] / 1e12,
                  "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": unit,
-                              "frac": achieved / peak, "traffic": None, "kernel_ms": t["region_ms"],
+                              "frac": achieved / peak, "traffic": load_traffic(traffic_key),
+                              "kernel_ms": t["region_ms"],
                               "kernel_ms_is": "stream time per call over back-to-back calls (all launches of a call)"}}
         if note:
             entry["roofline"]["note"] = note
