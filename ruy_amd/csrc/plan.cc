@@ -972,6 +972,17 @@ const void* Advance(const void* p, int64_t elements, int element_size) {
 }  // namespace
 
 int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
+  if (ctx->capturing && !ctx->no_alloc) {
+    // A call that cannot be recorded should record nothing: an operand with a
+    // cache policy that was never packed is found out here, before the other
+    // side's pack or sums kernel has gone into the caller's graph.
+    const bool lhs_missing = ShouldCache(call->lhs_cache_policy, call->rhs.cols) && !ctx->cache->HasSource(call->lhs_src_key);
+    const bool rhs_missing = ShouldCache(call->rhs_cache_policy, call->lhs.rows) && !ctx->cache->HasSource(call->rhs_src_key);
+    if (lhs_missing || rhs_missing) {
+      *err = kCaptureCacheMiss;
+      return RUYAMD_E_UNSUPPORTED;
+    }
+  }
   const TunedPath path = ctx->force_generic ? TunedPath::kNone : TunedPathFor(*call);
   if (path == TunedPath::kNone) return RunGeneric(ctx, call, err);
   const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;

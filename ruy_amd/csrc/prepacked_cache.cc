@@ -59,6 +59,12 @@ bool PrepackedCache::Erase(const void* src_data, const PackedMatrix& packed_matr
   return true;
 }
 
+bool PrepackedCache::HasSource(const void* src_data) const {
+  for (const auto& kv : cache_)
+    if (kv.first.src_data == src_data) return true;
+  return false;
+}
+
 void PrepackedCache::EjectUntilRoomFor(std::ptrdiff_t new_bytes) {
   while (!cache_.empty() && buffers_bytes_ + new_bytes > max_buffers_bytes_) {
     if (!EjectOne()) break;

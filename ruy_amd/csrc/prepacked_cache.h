@@ -86,6 +86,11 @@ class PrepackedCache final {
   // was removed. (No counterpart in the reference, whose pack cannot fail.)
   bool Erase(const void* src_data, const PackedMatrix& packed_matrix);
 
+  // Whether any entry was packed from this source pointer (whatever its layout
+  // and zero point): a cheap test ahead of work that would be wasted if the
+  // exact entry turned out to be missing.
+  bool HasSource(const void* src_data) const;
+
   std::ptrdiff_t BuffersBytes() const { return buffers_bytes_; }
   int MatrixCount() const { return static_cast<int>(cache_.size()); }
   std::ptrdiff_t MaxBuffersBytes() const { return max_buffers_bytes_; }

@@ -195,7 +195,9 @@ static void TestEraseAfterFailedPack() {
     EXPECT(cache.Get(d1.data(), &m1) == kInserted);
     EXPECT(cache.Get(d2.data(), &m2) == kInserted);
     EXPECT(cache.BuffersBytes() == 307 && cache.MatrixCount() == 2);
+    EXPECT(cache.HasSource(d1.data()) && cache.HasSource(d2.data()));
     EXPECT(cache.Erase(d1.data(), m1));
+    EXPECT(!cache.HasSource(d1.data()) && cache.HasSource(d2.data()));
     EXPECT(cache.BuffersBytes() == 27 && cache.MatrixCount() == 1);
     EXPECT(g_live_allocations == live_before + 2);  // only m2's data and sums are left
     EXPECT(!cache.Erase(d1.data(), m1));            // already gone
