@@ -19,6 +19,15 @@ __device__ __forceinline__ int32_t RequantHigh(int32_t x, int32_t m, int s) {
   return (__mulhi(x, m) + (1 << (s - 1))) >> s;
 }
 
+// v_med3_i32 (the compiler forms it from min/max only for constant bounds).
+// An instruction of this encoding takes one scalar operand at most: the lower
+// bound travels in a vector register.
+__device__ __forceinline__ int32_t Median3(int32_t x, int32_t lo, int32_t hi) {
+  int32_t r;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(lo), "s"(hi));
+  return r;
+}
+
 struct Int8Traits16;
 
 struct Int8Traits {
@@ -41,26 +50,29 @@ struct Int8Traits {
   static __device__ __forceinline__ int FromRawBits(int w) { return w; }
 
   struct RowState {
-    uint32_t add[16];
+    uint32_t add[16];  // after Load: the row's bias (or 0); after Prepare: everything added to the row's sums
+    int32_t sums[16];  // the row's operand sum over the depth (or 0)
     int32_t m[16];
     int32_t e[16];
+    // Loads only, nothing computed on what they bring: a caller may issue them
+    // long before the values are needed without waiting for them here.
     __device__ __forceinline__ void Load(const Epilogue& ep, const int (&row_idx)[16]) {
       const bool row_channel = !ep.channel_is_col;
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        add[q] = static_cast<uint32_t>(ep.zp_product_depth);
+        add[q] = 0;
+        sums[q] = 0;
         m[q] = ep.mult_fixedpoint_scalar;
         e[q] = ep.mult_exponent_scalar;
       }
       if (ep.bias && row_channel) {
         const int32_t* bias = static_cast<const int32_t*>(ep.bias);
 #pragma unroll
-        for (int q = 0; q < 16; ++q) add[q] += static_cast<uint32_t>(bias[row_idx[q]]);
+        for (int q = 0; q < 16; ++q) add[q] = static_cast<uint32_t>(bias[row_idx[q]]);
       }
       if (ep.rhs_zero_point) {
 #pragma unroll
-        for (int q = 0; q < 16; ++q)
-          add[q] -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[row_idx[q]]);
+        for (int q = 0; q < 16; ++q) sums[q] = ep.lhs_sums[row_idx[q]];
       }
       if (ep.mult_fixedpoint && row_channel) {
 #pragma unroll
@@ -69,6 +81,13 @@ struct Int8Traits {
           e[q] = ep.mult_exponent[row_idx[q]];
         }
       }
+    }
+    // Once, when the write-back starts.
+    __device__ __forceinline__ void Prepare(const Epilogue& ep) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        add[q] += static_cast<uint32_t>(ep.zp_product_depth) -
+                  static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(sums[q]);
     }
   };
 
@@ -104,12 +123,12 @@ struct Int8Traits {
         for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], rows.m[q], rows.e[q]);
       }
     }
+    // The host hands over ordered clamp bounds (clamp_min <= clamp_max), for
+    // which min-then-max is the median of the three.
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
-      int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
-      v = v > ep.clamp_max_i ? ep.clamp_max_i : v;
-      v = v < ep.clamp_min_i ? ep.clamp_min_i : v;
-      vals[q] = v;
+      const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
+      vals[q] = Median3(v, ep.clamp_min_i, ep.clamp_max_i);
     }
   }
 };

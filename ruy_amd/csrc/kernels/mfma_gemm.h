@@ -36,7 +36,9 @@
 // accumulators are combined), Bits(x, x2) (accumulator element - or combined
 // pair - as raw 32 bits), RawBits(x) / FromRawBits(w) (one accumulator element
 // to and from raw 32 bits),
-// RowState (per-destination-row write-back parameters, gathered once per lane)
+// RowState (per-destination-row write-back parameters, gathered once per lane:
+// Load() issues the loads and computes nothing from them, Prepare() does the
+// rest when the write-back starts)
 // and Finish(vals, rows, j, ep), which turns 16 raw accumulators of column j
 // into 16 destination values (as raw 32-bit words).
 #ifndef RUY_AMD_CSRC_KERNELS_MFMA_GEMM_H_
@@ -105,6 +107,17 @@ __device__ __forceinline__ void LoadToLds16(uint32_t lds_base, uint32_t voffset,
       :
       : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
       : "memory");
+}
+
+// Low 32 bits of a * b as one v_mul_lo_u32. Given `a * b + c` the compiler
+// picks the 64-bit multiply-add with an undefined upper half of c, and the
+// register it takes for that half may be one that still awaits a load issued
+// earlier (the row parameters of the largest tile), for which the wave then
+// waits.
+__device__ __forceinline__ uint32_t MulLo(uint32_t a, uint32_t b) {
+  uint32_t r;
+  asm("v_mul_lo_u32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
 }
 
 // f(std::integral_constant<int, 0>()), ..., f(std::integral_constant<int, N - 1>()).
@@ -248,7 +261,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     const int r = chunk * C::kRowsPerLoad + lane / C::kGranulesPerRow;
     const int g = (lane % C::kGranulesPerRow) ^ Swizzle<BK>(r);
     const int row = m0 + r;
-    a_goff[i] = row < args.M ? uint32_t(row) * uint32_t(args.lda) + g * kGranule : kOutOfRange;
+    a_goff[i] = row < args.M ? MulLo(row, args.lda) + g * kGranule : kOutOfRange;
     a_k[i] = g * kGranule;
   }
   uint32_t b_goff[C::kBLoads];
@@ -259,7 +272,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     const int r = chunk * C::kRowsPerLoad + lane / C::kGranulesPerRow;
     const int g = (lane % C::kGranulesPerRow) ^ Swizzle<BK>(r);
     const int col = n0 + r;
-    b_goff[i] = col < args.N ? uint32_t(col) * uint32_t(args.ldb) + g * kGranule : kOutOfRange;
+    b_goff[i] = col < args.N ? MulLo(col, args.ldb) + g * kGranule : kOutOfRange;
     b_k[i] = g * kGranule;
   }
   // Issues the loads of depth step kt into ring slot kt % kStages. Steps past
@@ -447,8 +460,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // loads carry no per-lane branches and can all be in flight together. The
   // largest tile issues these loads here, ahead of the main loop, which hides
   // their latency (a lone wave per SIMD has nothing else to run while it
-  // waits); the smaller tiles, which live on fewer registers, load them
-  // when the write-back starts.
+  // waits): loads only, what is computed from them waits until the write-back
+  // starts, or the wave would sit out their latency right here. The smaller
+  // tiles, which live on fewer registers, load them when the write-back starts.
   constexpr bool kEarlyRowState = kB == 16;
   constexpr int kChunksPerCol = WM * 32 / 16;
   const Epilogue& ep = args.ep;
@@ -833,6 +847,10 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int chunk = lane % kChunksPerCol;
   const int i0 = m0 + wave_m * kRows + chunk * 16;
   if constexpr (!kEarlyRowState) load_row_state();
+  rows.Prepare(ep);
+  const int64_t col_bytes = ldd * elt;  // from one destination column to the next
+  const int j_first = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * C::kLogicalWN * 32 + lane / kChunksPerCol;
+  char* const lane_out = dst_base + (int64_t(j_first) * ldd + i0) * elt;
 
   // The accumulators go to LDS in straight-line code (their register indices
   // must be compile-time constants); everything after that is a compact loop,
@@ -920,7 +938,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       }
       Traits::Finish(vals, rows, j, ep);
       const bool full = i0 + 16 <= args.M;
-      char* out = dst_base + (int64_t(j) * ldd + i0) * elt;
+      // This lane's address at the wave's first staged column, plus what the
+      // pass adds (the same for every lane: scalar arithmetic).
+      char* out = lane_out + int64_t(half * kHalfCols + pass * kColsPerPass) * col_bytes;
       if (full && args.dst_vector_ok) {
         if (elt == 1) {
           v4i w;

@@ -232,6 +232,11 @@ void FillCall(const ruyamd_mat& lhs, const ruyamd_mat& rhs, const ruyamd_mul_par
   } else {
     ep.clamp_min_i = ClampToInt32(p.clamp_min);
     ep.clamp_max_i = ClampToInt32(p.clamp_max);
+    // min(x, clamp_max) first, then max(., clamp_min) (ruy/reference_mul.h:47-48):
+    // with clamp_min above clamp_max every result is clamp_min. Raising
+    // clamp_max to clamp_min says the same and lets kernels clamp with one
+    // median-of-three instruction, which needs ordered bounds.
+    if (ep.clamp_max_i < ep.clamp_min_i) ep.clamp_max_i = ep.clamp_min_i;
   }
 }
 
