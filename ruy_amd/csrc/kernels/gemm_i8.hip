@@ -38,6 +38,7 @@ struct Int8Traits {
   static __device__ __forceinline__ void DrainMma() {}
   static constexpr int kBlock = 32;
   static constexpr bool kRawB = false;
+  static constexpr bool kStaggered = false;
   // The 256x256 tile runs on 16x16 blocks (below).
   using LargeTile = Int8Traits16;
   static constexpr bool kSplitB = false;
@@ -155,6 +156,7 @@ struct Int8Traits16 : Int8Traits {
   }
   static __device__ __forceinline__ void DrainMma() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
   static constexpr int kBlock = 16;
+  static constexpr bool kStaggered = true;  // the operands' rings half a step apart (see the kernel)
   using LargeTile = Int8Traits16;
 };
 

@@ -694,6 +694,122 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           for (int e = 0; e < 4; ++e) acc[0][j][4 * q + e] += Traits::FromRawBits(w[e]);
         }
     }
+  } else if constexpr (Traits::kStaggered) {
+    // ---- the largest int8 tile: the two operands' rings half a step apart ----
+    // A direct-to-LDS load of 1 KiB keeps the CU's one address unit busy for 16
+    // cycles, and a ring step of this tile needs 64 of them, 1024 of the 2048
+    // cycles its matrix instructions take. With one ring for both operands a
+    // slot comes free in the middle of a ring step (when the fragments of the
+    // step's second sub-step have been read), so all 64 loads had to be issued
+    // during that second sub-step, which kept the address unit busy throughout
+    // it and the matrix instructions waiting behind the loads. Here the A half
+    // and the B half of a slot are freed at different times, and every
+    // sub-step carries the loads of one operand:
+    //   sub-step (kt, 0): matrix instructions on A(kt,0) x B(kt,0); A(kt,1)
+    //     fragments read; loads of B for ring step kt+2 issued;
+    //   sub-step (kt, 1): matrix instructions on A(kt,1) x B(kt,1); A(kt+1,0)
+    //     fragments read; loads of A for ring step kt+2 issued.
+    // For B's half-slot to be free at the start of ring step kt, B's fragments
+    // are read a whole ring step ahead: the instructions of a sub-step walk the
+    // blocks column by column, so that B fragment j is used by eight
+    // consecutive instructions, after which its registers take the fragment of
+    // the same column and sub-step of ring step kt+1 (two instructions later;
+    // for the last column that is the second instruction of the next
+    // sub-step). No more registers than two sets of fragments, as before.
+    //
+    // One barrier per sub-step, in front of its ninth instruction, so that the
+    // few LDS reads issued just before it have the first eight to finish
+    // behind. It says: every wave has the fragments it wanted from the half-slot
+    // that this sub-step's loads overwrite (B: read up to the second
+    // instruction of this sub-step; A: read during the previous sub-step), and
+    // the loads that the reads behind it rely on have landed for all waves -
+    // all but the eight issued during the previous sub-step, which belong to
+    // the other operand and are older than nothing this sub-step reads.
+    static_assert(kB == 16 && C::kKSteps == 2 && C::kStages == 2 && kAB == 8 && kBB == 8 && C::kALoads == 8 &&
+                      C::kBLoads == 8 && !kFlip && !kFusedSums,
+                  "the staggered schedule is written for the 256x256 tile of 16x16 blocks");
+    struct AFrags {
+      v4i a[kAB];
+    };
+    AFrags fa[2];
+    v4i fb[2][kBB];
+    auto read_a = [&](int kt, int ks, int i, AFrags& f) {
+      const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
+      f.a[i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * kB * kBK);
+    };
+    auto read_b = [&](int kt, int ks, int j, v4i& into) {
+      const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
+      into = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * kB * kBK);
+    };
+    // B of step 0, A of step 0, B of step 1, A of step 1: the order in which
+    // the loop goes on issuing them, so that "all but the last eight" means
+    // the same before the loop as inside it.
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int l = 0; l < C::kBLoads; ++l) issue_one(st, C::kALoads + l);
+#pragma unroll
+      for (int l = 0; l < C::kALoads; ++l) issue_one(st, l);
+    }
+    WaitVmcnt<C::kALoads>();
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kAB; ++i) read_a(0, 0, i, fa[0]);
+#pragma unroll
+    for (int j = 0; j < kBB; ++j) read_b(0, 0, j, fb[0][j]);
+#pragma unroll
+    for (int j = 0; j + 1 < kBB; ++j) read_b(0, 1, j, fb[1][j]);
+    auto staggered_sub_step = [&](int kt, auto ks_constant, auto full) {
+      constexpr int ks = decltype(ks_constant)::value;
+      const AFrags& cur = fa[ks];
+      AFrags& next = fa[1 - ks];
+      const int kt_next = ks == 0 ? kt : kt + 1;
+      StaticFor<kMmas>([&](auto n_constant) {
+        constexpr int n = decltype(n_constant)::value;
+        constexpr int j = n / kAB;
+        constexpr int i = n % kAB;
+        if constexpr (n == 8) {
+          WaitVmcnt<8>();
+          __syncthreads();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        Traits::Mma(cur.a[i], fb[ks][j], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        // The last column's B fragment of the sub-step before this one.
+        if constexpr (n == 1) {
+          if constexpr (ks == 0)
+            read_b(kt, 1, kBB - 1, fb[1][kBB - 1]);
+          else
+            read_b(kt + 1, 0, kBB - 1, fb[0][kBB - 1]);
+        }
+        // Column jj is done with: its fragment of the next ring step.
+        if constexpr (n >= 9 && (n - 9) % kAB == 0 && (n - 9) / kAB < kBB - 1) {
+          constexpr int jj = (n - 9) / kAB;
+          read_b(kt + 1, ks, jj, fb[ks][jj]);
+        }
+        // The A fragments of the next sub-step.
+        if constexpr (n >= 9 && n % 2 == 1 && (n - 9) / 2 < kAB) read_a(kt_next, 1 - ks, (n - 9) / 2, next);
+        // This sub-step's share of the loads of ring step kt + 2.
+        if constexpr (n >= 12 && (n - 12) % 6 == 0 && (n - 12) / 6 < 8) {
+          constexpr int l = (ks == 0 ? C::kALoads : 0) + (n - 12) / 6;
+          if (decltype(full)::value)
+            issue_one_full(kt + C::kStages, l);
+          else
+            issue_one(kt + C::kStages, l);
+        }
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    int kt = 0;
+    const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
+    for (; kt < full_end; ++kt) {
+      staggered_sub_step(kt, std::integral_constant<int, 0>(), std::true_type());
+      staggered_sub_step(kt, std::integral_constant<int, 1>(), std::true_type());
+    }
+    for (; kt < k_tiles; ++kt) {
+      staggered_sub_step(kt, std::integral_constant<int, 0>(), std::false_type());
+      staggered_sub_step(kt, std::integral_constant<int, 1>(), std::false_type());
+    }
   } else {
 #pragma unroll
     for (int s = 0; s < C::kStages; ++s) issue(s);
