@@ -37,6 +37,7 @@ struct F32Traits {
   static __device__ __forceinline__ int RawBits(float x) { return __float_as_int(x); }
   static __device__ __forceinline__ float FromRawBits(int w) { return __int_as_float(w); }
 
+  struct EdgeParams {};  // (kernels on 16x16 blocks only)
   struct RowState {
     float bias[16];
     __device__ __forceinline__ void Load(const Epilogue& ep, const int (&row_idx)[16]) {

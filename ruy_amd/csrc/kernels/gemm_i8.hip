@@ -50,6 +50,7 @@ struct Int8Traits {
   static __device__ __forceinline__ int RawBits(int x) { return x; }
   static __device__ __forceinline__ int FromRawBits(int w) { return w; }
 
+  struct EdgeParams {};  // (kernels on 16x16 blocks only)
   struct RowState {
     uint32_t add[16];  // after Load: the row's bias (or 0); after Prepare: everything added to the row's sums
     int32_t sums[16];  // the row's operand sum over the depth (or 0)
@@ -158,6 +159,148 @@ struct Int8Traits16 : Int8Traits {
   static constexpr int kBlock = 16;
   static constexpr bool kStaggered = true;  // the operands' rings half a step apart (see the kernel)
   using LargeTile = Int8Traits16;
+
+  // ---- write-back parameters of the 16x16-block kernel ----
+  // A wave's 128 rows and 128 columns each have three write-back parameters:
+  // what is added to the accumulator (bias, zero-point corrections; the
+  // constant part sits with the rows), and the multiplier and exponent that
+  // apply if the channels run along that dimension. Lane l fetches them for
+  // rows and columns l and l + 64 of the wave when the workgroup starts
+  // (EdgeParams: loads only, nothing computed, so nobody waits for them), and
+  // the wave puts them into an LDS area of its own when the write-back starts
+  // (Stage). From there every lane reads those of the rows and columns its
+  // accumulators belong to: LDS reads, so that inside the write-back loops
+  // nothing waits on the vector-memory counter, which would also mean waiting
+  // for the stores just issued.
+  static constexpr int kParamInts = 6 * 128;  // per wave: row add, m, e; column add, m, e
+  struct EdgeParams {
+    int32_t bias[4], sums[4], m[4], e[4];  // [0..1]: rows l, l + 64; [2..3]: columns l, l + 64
+  };
+  static __device__ __forceinline__ void LoadEdgeParams(const Epilogue& ep, const int (&row)[2], const int (&col)[2],
+                                                        EdgeParams& p) {
+    const bool row_channel = !ep.channel_is_col;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      p.bias[k] = 0;
+      p.sums[k] = 0;
+      p.m[k] = ep.mult_fixedpoint_scalar;
+      p.e[k] = ep.mult_exponent_scalar;
+    }
+    // (Register arrays: constant indices only.)
+    const int32_t* bias = static_cast<const int32_t*>(ep.bias);
+    if (bias && row_channel) {
+      p.bias[0] = bias[row[0]];
+      p.bias[1] = bias[row[1]];
+    }
+    if (bias && !row_channel) {
+      p.bias[2] = bias[col[0]];
+      p.bias[3] = bias[col[1]];
+    }
+    if (ep.rhs_zero_point) {
+      p.sums[0] = ep.lhs_sums[row[0]];
+      p.sums[1] = ep.lhs_sums[row[1]];
+    }
+    if (ep.lhs_zero_point) {
+      p.sums[2] = ep.rhs_sums[col[0]];
+      p.sums[3] = ep.rhs_sums[col[1]];
+    }
+    if (ep.mult_fixedpoint && row_channel) {
+      p.m[0] = ep.mult_fixedpoint[row[0]];
+      p.m[1] = ep.mult_fixedpoint[row[1]];
+      p.e[0] = ep.mult_exponent[row[0]];
+      p.e[1] = ep.mult_exponent[row[1]];
+    }
+    if (ep.mult_fixedpoint && !row_channel) {
+      p.m[2] = ep.mult_fixedpoint[col[0]];
+      p.m[3] = ep.mult_fixedpoint[col[1]];
+      p.e[2] = ep.mult_exponent[col[0]];
+      p.e[3] = ep.mult_exponent[col[1]];
+    }
+  }
+  static __device__ __forceinline__ void Stage(const Epilogue& ep, const EdgeParams& p, int* area, int lane) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool is_row = k < 2;
+      const uint32_t zp = static_cast<uint32_t>(is_row ? ep.rhs_zero_point : ep.lhs_zero_point);
+      const uint32_t add = static_cast<uint32_t>(p.bias[k]) - zp * static_cast<uint32_t>(p.sums[k]) +
+                           (is_row ? static_cast<uint32_t>(ep.zp_product_depth) : 0u);
+      int* base = area + (is_row ? 0 : 3 * 128) + lane + (k & 1) * 64;
+      base[0] = static_cast<int32_t>(add);
+      base[128] = p.m[k];
+      base[256] = p.e[k];
+    }
+  }
+  // Which form of the arithmetic a launch needs, decided once so that the
+  // write-back loops carry no branches on it: a lone wave pays for every
+  // branch with an empty instruction buffer.
+  enum FinishMode { kRaw = 0, kScalarHigh, kScalar, kPerRow, kPerColumn, kFinishModes };
+  static __device__ __forceinline__ int ModeOf(const Epilogue& ep) {
+    if (!ep.requantize) return kRaw;
+    if (ep.mult_fixedpoint) return ep.channel_is_col ? kPerColumn : kPerRow;
+    return ep.mult_exponent_scalar <= -2 ? kScalarHigh : kScalar;
+  }
+  struct RowParams {
+    v4i add[4], m[4], e[4];
+  };
+  // The parameters of 16 of the wave's rows: four consecutive ones from
+  // `first` on in each of four blocks 16 rows apart.
+  template <int kMode>
+  static __device__ __forceinline__ void ReadRowParams(const int* area, int first, RowParams& r) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) r.add[b] = *reinterpret_cast<const v4i*>(area + first + 16 * b);
+    if constexpr (kMode == kPerRow) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        r.m[b] = *reinterpret_cast<const v4i*>(area + 128 + first + 16 * b);
+        r.e[b] = *reinterpret_cast<const v4i*>(area + 256 + first + 16 * b);
+      }
+    }
+  }
+  struct ColParams {
+    int32_t add, m, e;
+  };
+  template <int kMode>
+  static __device__ __forceinline__ void ReadColParams(const int* area, int col, ColParams& c) {
+    c.add = area[3 * 128 + col];
+    if constexpr (kMode == kPerColumn) {
+      c.m = area[4 * 128 + col];
+      c.e = area[5 * 128 + col];
+    }
+  }
+  // vals[4 * b + v]: row v of block b's four. The arithmetic of
+  // Int8Traits::Finish.
+  template <int kMode>
+  static __device__ __forceinline__ void Finish16(int32_t (&vals)[16], const RowParams& r, const ColParams& c,
+                                                  const Epilogue& ep) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      vals[q] = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(r.add[q / 4][q % 4]) +
+                                     static_cast<uint32_t>(c.add));
+    if constexpr (kMode == kScalarHigh) {
+      const int32_t m = ep.mult_fixedpoint_scalar;
+      const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
+#pragma unroll
+      for (int q = 0; q < 16; ++q) vals[q] = RequantHigh(vals[q], m, high_shift);
+    } else if constexpr (kMode == kScalar) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        vals[q] = MultiplyByQuantizedMultiplier(vals[q], ep.mult_fixedpoint_scalar, ep.mult_exponent_scalar);
+    } else if constexpr (kMode == kPerColumn) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], c.m, c.e);
+    } else if constexpr (kMode == kPerRow) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        vals[q] = MultiplyByQuantizedMultiplier(vals[q], r.m[q / 4][q % 4], r.e[q / 4][q % 4]);
+    }
+    // (kRaw: the bounds are those of int32, ruy/mul_params.h:291-293, and the
+    // zero point of an int32 destination is zero: the same code serves.)
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
+      vals[q] = Median3(v, ep.clamp_min_i, ep.clamp_max_i);
+    }
+  }
 };
 
 // int8 x int16 (ruy/kernel_avx512.cc:55-626 instantiated for a 16-bit RHS,

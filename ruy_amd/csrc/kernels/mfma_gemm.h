@@ -175,8 +175,12 @@ struct Cfg {
   static constexpr int kEpilogueBlockCols = kLogicalWN >= 2 ? kLogicalWN / 2 : 1;
   static constexpr int kEpiloguePitch = WM * 32 + 4;
   static constexpr int kEpilogueBytes = 4 * kEpilogueBlockCols * 32 * kEpiloguePitch * 4;
-  static constexpr int kLdsBytes =
-      kStages * kStageBytes > kEpilogueBytes ? kStages * kStageBytes : kEpilogueBytes;
+  // 16x16 blocks: no staging (the write-back transposes between lanes), but
+  // 3 KiB of write-back parameters per wave behind the ring.
+  static constexpr int kParamBytes = 4 * 6 * 128 * 4;
+  static constexpr int kLdsBytes = BLOCK == 16 ? kStages * kStageBytes + kParamBytes
+                                               : (kStages * kStageBytes > kEpilogueBytes ? kStages * kStageBytes
+                                                                                         : kEpilogueBytes);
 };
 
 // kFusedSums (64x64 tile of the int8 kernel only): the kernel also forms the
@@ -453,17 +457,12 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   };
 
   // ---- what the write-back needs per destination row ----
-  // After the transposition (below) a lane owns 16 consecutive rows of one
-  // column at a time, the same rows for every column it writes: everything
-  // that depends only on the row is gathered once. Rows past the end are
-  // clamped to the last row (their results are never stored) so that the
-  // loads carry no per-lane branches and can all be in flight together. The
-  // largest tile issues these loads here, ahead of the main loop, which hides
-  // their latency (a lone wave per SIMD has nothing else to run while it
-  // waits): loads only, what is computed from them waits until the write-back
-  // starts, or the wave would sit out their latency right here. The smaller
-  // tiles, which live on fewer registers, load them when the write-back starts.
-  constexpr bool kEarlyRowState = kB == 16;
+  // 32x32 blocks: after the transposition (below) a lane owns 16 consecutive
+  // rows of one column at a time, the same rows for every column it writes:
+  // everything that depends only on the row is gathered once, when the
+  // write-back starts. Rows past the end are clamped to the last row (their
+  // results are never stored) so that the loads carry no per-lane branches and
+  // can all be in flight together.
   constexpr int kChunksPerCol = WM * 32 / 16;
   const Epilogue& ep = args.ep;
   typename Traits::RowState rows;
@@ -474,7 +473,17 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     for (int q = 0; q < 16; ++q) row_idx[q] = min(first_row + q, args.M - 1);
     rows.Load(ep, row_idx);
   };
-  if constexpr (kEarlyRowState) load_row_state();
+  // 16x16 blocks: each lane fetches the parameters of two of the wave's rows
+  // and two of its columns here, ahead of the main loop (loads only); the
+  // write-back hands them round through LDS.
+  typename Traits::EdgeParams edge;
+  if constexpr (kB == 16) {
+    const int row = m0 + wave_m * (WM * 32) + lane;
+    const int col = n0 + wave_n * (WN * 32) + lane;
+    const int row_idx[2] = {min(row, args.M - 1), min(row + 64, args.M - 1)};
+    const int col_idx[2] = {min(col, args.n_logical - 1), min(col + 64, args.n_logical - 1)};
+    Traits::LoadEdgeParams(ep, row_idx, col_idx, edge);
+  }
 
   // ---- software pipeline ----
   // Fragments are double-buffered in registers: while the matrix instructions
@@ -944,7 +953,150 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     }
   }
 
-  // ---- fused write-back ----
+  // ---- fused write-back, 16x16 blocks ----
+  // The destination is column-major here (rows contiguous; the host swaps the
+  // operands for a row-major destination). Lane l holds, of every block,
+  // column l%16 and the four consecutive rows 4*(l/16) .. +3. The write-back
+  // arithmetic runs on the values where they are (16 at a time: the lane's
+  // four rows in four row blocks of one block column, whose 16 rows are what a
+  // RowState describes). What is left to do for a vector store is to gather a
+  // block's 16 rows of a column, which sit in the four lanes l%16 + {0, 16, 32,
+  // 48}, into one of them: a 4 x 4 transposition of 32-bit words between those
+  // lanes (four words a lane, one per row block), for which the hardware has
+  // register-to-register swaps of lane rows. Afterwards lane l owns rows
+  // 0 .. 15 of block 4*half + l/16 of its column and writes them with 16-byte
+  // stores. No LDS is involved.
+  if constexpr (kB == 16) {
+    static_assert(!Traits::kSplitB && kAB == 8 && kBB == 8, "");
+    const int elt = args.dst_elt;
+    char* const dst_base = static_cast<char*>(args.dst.data);
+    const int64_t ldd = args.dst.cs;
+    // The wave's parameter area (behind the ring): written and read by this
+    // wave only, and LDS operations of a wave complete in order.
+    int* const area = reinterpret_cast<int*>(lds + C::kStages * C::kStageBytes) + wave * Traits::kParamInts;
+    Traits::Stage(ep, edge, area, lane);
+    const int col0 = n0 + wave_n * (WN * 32) + (lane & 15);
+    // reg k of lane row q  <->  reg q of lane row k (lane rows: 16 lanes each).
+    auto transpose = [](int (&r)[4]) {
+      auto a = __builtin_amdgcn_permlane32_swap(r[0], r[2], false, false);
+      auto b = __builtin_amdgcn_permlane32_swap(r[1], r[3], false, false);
+      auto c = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);
+      auto d = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+      r[0] = c[0];
+      r[1] = c[1];
+      r[2] = d[0];
+      r[3] = d[1];
+    };
+    // kMode: the form of the write-back arithmetic (Traits::ModeOf); kElt: bytes
+    // per destination element. Compile-time, so that the loop below is
+    // straight-line code apart from its one branch on the counter.
+    auto half_pass = [&](auto half_constant, auto mode_constant, auto elt_constant) {
+      constexpr int half = decltype(half_constant)::value;
+      constexpr int kMode = decltype(mode_constant)::value;
+      constexpr int kElt = decltype(elt_constant)::value;
+      typename Traits::RowParams row_params;
+      Traits::template ReadRowParams<kMode>(area, half * 64 + 4 * (lane >> 4), row_params);
+      // After the transposition: the 16 rows this lane stores.
+      const int row0 = m0 + wave_m * (WM * 32) + (half * 4 + (lane >> 4)) * 16;
+      const bool rows_full = row0 + 16 <= args.M;
+      // A compact loop over the block columns: only the gathering of a
+      // column's accumulators, whose register numbers must be constants, is
+      // written out eight times, behind a branch on the (wave-uniform) counter.
+      // The column's parameters are read one trip ahead.
+      typename Traits::ColParams col_params, col_ahead;
+      Traits::template ReadColParams<kMode>(area, lane & 15, col_ahead);
+#pragma unroll 1
+      for (int bj = 0; bj < kBB; ++bj) {
+        const int j = col0 + bj * 16;
+        col_params = col_ahead;
+        Traits::template ReadColParams<kMode>(area, ((bj + 1) & (kBB - 1)) * 16 + (lane & 15), col_ahead);
+        int32_t vals[16];
+        StaticFor<kBB>([&](auto bj_constant) {
+          constexpr int kBj = decltype(bj_constant)::value;
+          if (bj == kBj) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+              for (int v = 0; v < 4; ++v)
+                vals[4 * b + v] = Traits::Bits(acc[half * 4 + b][kBj][v], acc[half * 4 + b][kBj][v]);
+          }
+        });
+        Traits::template Finish16<kMode>(vals, row_params, col_params, ep);
+        // w[p][k]: after the transposition, word p of the kElt words that hold
+        // rows 4k .. 4k+3 of the lane's block. Every lane takes part in the
+        // swaps; columns and rows past the end are left out when storing.
+        int w[kElt][4];
+        if constexpr (kElt == 1) {
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            w[0][b] = (vals[4 * b] & 0xff) | ((vals[4 * b + 1] & 0xff) << 8) | ((vals[4 * b + 2] & 0xff) << 16) |
+                      (vals[4 * b + 3] << 24);
+        } else if constexpr (kElt == 2) {
+#pragma unroll
+          for (int b = 0; b < 4; ++b) {
+            w[0][b] = (vals[4 * b] & 0xffff) | (vals[4 * b + 1] << 16);
+            w[1][b] = (vals[4 * b + 2] & 0xffff) | (vals[4 * b + 3] << 16);
+          }
+        } else {
+#pragma unroll
+          for (int p = 0; p < 4; ++p)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) w[p][b] = vals[4 * b + p];
+        }
+#pragma unroll
+        for (int p = 0; p < kElt; ++p) transpose(w[p]);
+        if (j < args.n_logical && row0 < args.M) {
+          char* out = dst_base + (int64_t(j) * ldd + row0) * kElt;
+          if (rows_full && args.dst_vector_ok) {
+            // Memory order: rows 4k .. 4k+3 are words w[0][k] .. w[kElt-1][k].
+#pragma unroll
+            for (int x = 0; x < kElt; ++x) {
+              v4i o;
+#pragma unroll
+              for (int y = 0; y < 4; ++y) o[y] = w[(4 * x + y) % kElt][(4 * x + y) / kElt];
+              reinterpret_cast<v4i*>(out)[x] = o;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              if (row0 + r < args.M) {
+                if constexpr (kElt == 1)
+                  reinterpret_cast<int8_t*>(out)[r] = static_cast<int8_t>(w[0][r / 4] >> (8 * (r % 4)));
+                else if constexpr (kElt == 2)
+                  reinterpret_cast<int16_t*>(out)[r] = static_cast<int16_t>(w[(r % 4) / 2][r / 4] >> (16 * (r % 2)));
+                else
+                  reinterpret_cast<int32_t*>(out)[r] = w[r % 4][r / 4];
+              }
+            }
+          }
+        }
+      }
+    };
+    auto write_back = [&](auto mode_constant, auto elt_constant) {
+      half_pass(std::integral_constant<int, 0>(), mode_constant, elt_constant);
+      half_pass(std::integral_constant<int, 1>(), mode_constant, elt_constant);
+    };
+    // An int32 destination takes the raw form, and only it does; the others
+    // are one or two bytes wide.
+    const int mode = Traits::ModeOf(ep);
+    if (mode == Traits::kRaw) {
+      write_back(std::integral_constant<int, Traits::kRaw>(), std::integral_constant<int, 4>());
+    } else {
+      StaticFor<Traits::kFinishModes>([&](auto mode_constant) {
+        if constexpr (decltype(mode_constant)::value != Traits::kRaw) {
+          if (mode == decltype(mode_constant)::value) {
+            if (elt == 1)
+              write_back(mode_constant, std::integral_constant<int, 1>());
+            else
+              write_back(mode_constant, std::integral_constant<int, 2>());
+          }
+        }
+      });
+    }
+    return;
+  }
+
+  // ---- fused write-back, 32x32 blocks ----
   // The destination is column-major here (rows contiguous; the host swaps the
   // operands for a row-major destination). In a 32x32 accumulator block lane l
   // holds column l%32 and rows 8*(v/4) + 4*(l/32) + v%4, so a lane's values are
@@ -962,7 +1114,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int64_t ldd = args.dst.cs;
   const int chunk = lane % kChunksPerCol;
   const int i0 = m0 + wave_m * kRows + chunk * 16;
-  if constexpr (!kEarlyRowState) load_row_state();
+  load_row_state();
   rows.Prepare(ep);
   const int64_t col_bytes = ldd * elt;  // from one destination column to the next
   const int j_first = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * C::kLogicalWN * 32 + lane / kChunksPerCol;
