@@ -49,7 +49,6 @@ struct F32Traits {
         for (int q = 0; q < 16; ++q) bias[q] = b[row_idx[q]];
       }
     }
-    __device__ __forceinline__ void Prepare(const Epilogue&) {}
   };
 
   static __device__ __forceinline__ void Finish(int32_t (&vals)[16], const RowState& rows, int j,

@@ -52,29 +52,26 @@ struct Int8Traits {
 
   struct EdgeParams {};  // (kernels on 16x16 blocks only)
   struct RowState {
-    uint32_t add[16];  // after Load: the row's bias (or 0); after Prepare: everything added to the row's sums
-    int32_t sums[16];  // the row's operand sum over the depth (or 0)
+    uint32_t add[16];
     int32_t m[16];
     int32_t e[16];
-    // Loads only, nothing computed on what they bring: a caller may issue them
-    // long before the values are needed without waiting for them here.
     __device__ __forceinline__ void Load(const Epilogue& ep, const int (&row_idx)[16]) {
       const bool row_channel = !ep.channel_is_col;
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        add[q] = 0;
-        sums[q] = 0;
+        add[q] = static_cast<uint32_t>(ep.zp_product_depth);
         m[q] = ep.mult_fixedpoint_scalar;
         e[q] = ep.mult_exponent_scalar;
       }
       if (ep.bias && row_channel) {
         const int32_t* bias = static_cast<const int32_t*>(ep.bias);
 #pragma unroll
-        for (int q = 0; q < 16; ++q) add[q] = static_cast<uint32_t>(bias[row_idx[q]]);
+        for (int q = 0; q < 16; ++q) add[q] += static_cast<uint32_t>(bias[row_idx[q]]);
       }
       if (ep.rhs_zero_point) {
 #pragma unroll
-        for (int q = 0; q < 16; ++q) sums[q] = ep.lhs_sums[row_idx[q]];
+        for (int q = 0; q < 16; ++q)
+          add[q] -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[row_idx[q]]);
       }
       if (ep.mult_fixedpoint && row_channel) {
 #pragma unroll
@@ -83,13 +80,6 @@ struct Int8Traits {
           e[q] = ep.mult_exponent[row_idx[q]];
         }
       }
-    }
-    // Once, when the write-back starts.
-    __device__ __forceinline__ void Prepare(const Epilogue& ep) {
-#pragma unroll
-      for (int q = 0; q < 16; ++q)
-        add[q] += static_cast<uint32_t>(ep.zp_product_depth) -
-                  static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(sums[q]);
     }
   };
 
@@ -154,6 +144,10 @@ struct Int8Traits16 : Int8Traits {
   using Acc = v4i;
   static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+  // The same with zero in place of the accumulator going in.
+  static __device__ __forceinline__ void MmaFromZero(const v4i& a, const v4i& b, Acc& acc) {
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ void DrainMma() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
   static constexpr int kBlock = 16;

@@ -36,9 +36,7 @@
 // accumulators are combined), Bits(x, x2) (accumulator element - or combined
 // pair - as raw 32 bits), RawBits(x) / FromRawBits(w) (one accumulator element
 // to and from raw 32 bits),
-// RowState (per-destination-row write-back parameters, gathered once per lane:
-// Load() issues the loads and computes nothing from them, Prepare() does the
-// rest when the write-back starts)
+// RowState (per-destination-row write-back parameters, gathered once per lane)
 // and Finish(vals, rows, j, ep), which turns 16 raw accumulators of column j
 // into 16 destination values (as raw 32-bit words).
 #ifndef RUY_AMD_CSRC_KERNELS_MFMA_GEMM_H_
@@ -376,12 +374,17 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   };
 
   typename Traits::Acc acc[kAB][kBB];
+  auto clear_accumulators = [&]() {
 #pragma unroll
-  for (int i = 0; i < kAB; ++i)
+    for (int i = 0; i < kAB; ++i)
 #pragma unroll
-    for (int j = 0; j < kBB; ++j)
+      for (int j = 0; j < kBB; ++j)
 #pragma unroll
-      for (int v = 0; v < kAccElems; ++v) acc[i][j][v] = 0;
+        for (int v = 0; v < kAccElems; ++v) acc[i][j][v] = 0;
+  };
+  // (The staggered schedule starts its first matrix instructions from zero
+  // instead: 256 register writes fewer per tile.)
+  if constexpr (!Traits::kStaggered) clear_accumulators();
 
   typename Traits::Acc sum_a, sum_b;  // kFusedSums: row sums of a / column sums of b, in every column / row
 #pragma unroll
@@ -768,7 +771,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     for (int j = 0; j < kBB; ++j) read_b(0, 0, j, fb[0][j]);
 #pragma unroll
     for (int j = 0; j + 1 < kBB; ++j) read_b(0, 1, j, fb[1][j]);
-    auto staggered_sub_step = [&](int kt, auto ks_constant, auto full) {
+    // `first`: the tile's first sub-step, whose matrix instructions start from
+    // zero instead of from the accumulators (which nobody has cleared).
+    auto staggered_sub_step = [&](int kt, auto ks_constant, auto full, auto first) {
       constexpr int ks = decltype(ks_constant)::value;
       const AFrags& cur = fa[ks];
       AFrags& next = fa[1 - ks];
@@ -782,7 +787,10 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           __syncthreads();
         }
         __builtin_amdgcn_sched_barrier(0);
-        Traits::Mma(cur.a[i], fb[ks][j], acc[i][j]);
+        if constexpr (decltype(first)::value)
+          Traits::MmaFromZero(cur.a[i], fb[ks][j], acc[i][j]);
+        else
+          Traits::Mma(cur.a[i], fb[ks][j], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         // The last column's B fragment of the sub-step before this one.
         if constexpr (n == 1) {
@@ -809,15 +817,26 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       });
       __builtin_amdgcn_sched_barrier(0);
     };
-    int kt = 0;
     const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
+    using Sub0 = std::integral_constant<int, 0>;
+    using Sub1 = std::integral_constant<int, 1>;
+    int kt = 1;
+    if (full_end > 0) {
+      staggered_sub_step(0, Sub0(), std::true_type(), std::true_type());
+      staggered_sub_step(0, Sub1(), std::true_type(), std::false_type());
+    } else if (k_tiles > 0) {
+      staggered_sub_step(0, Sub0(), std::false_type(), std::true_type());
+      staggered_sub_step(0, Sub1(), std::false_type(), std::false_type());
+    } else {
+      clear_accumulators();
+    }
     for (; kt < full_end; ++kt) {
-      staggered_sub_step(kt, std::integral_constant<int, 0>(), std::true_type());
-      staggered_sub_step(kt, std::integral_constant<int, 1>(), std::true_type());
+      staggered_sub_step(kt, Sub0(), std::true_type(), std::false_type());
+      staggered_sub_step(kt, Sub1(), std::true_type(), std::false_type());
     }
     for (; kt < k_tiles; ++kt) {
-      staggered_sub_step(kt, std::integral_constant<int, 0>(), std::false_type());
-      staggered_sub_step(kt, std::integral_constant<int, 1>(), std::false_type());
+      staggered_sub_step(kt, Sub0(), std::false_type(), std::false_type());
+      staggered_sub_step(kt, Sub1(), std::false_type(), std::false_type());
     }
   } else {
 #pragma unroll
@@ -1115,7 +1134,6 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int chunk = lane % kChunksPerCol;
   const int i0 = m0 + wave_m * kRows + chunk * 16;
   load_row_state();
-  rows.Prepare(ep);
   const int64_t col_bytes = ldd * elt;  // from one destination column to the next
   const int j_first = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * C::kLogicalWN * 32 + lane / kChunksPerCol;
   char* const lane_out = dst_base + (int64_t(j_first) * ldd + i0) * elt;
