@@ -118,6 +118,16 @@ __device__ __forceinline__ uint32_t MulLo(uint32_t a, uint32_t b) {
   return r;
 }
 
+// The two halves of the above for callers that have an instruction of their
+// own to put between them (M0 must be written one wait state ahead of the load
+// that uses it; here that slot does useful work instead of a no-op).
+__device__ __forceinline__ void SetLdsTarget(uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0" : : "s"(lds_base));
+}
+__device__ __forceinline__ void LoadToLdsTarget16(uint32_t voffset, uint32_t soffset, v4i rsrc) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+
 // f(std::integral_constant<int, 0>()), ..., f(std::integral_constant<int, N - 1>()).
 template <class F, int... Is>
 __device__ __forceinline__ void StaticForEach(F&& f, std::integer_sequence<int, Is...>) {
@@ -806,13 +816,19 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         }
         // The A fragments of the next sub-step.
         if constexpr (n >= 9 && n % 2 == 1 && (n - 9) / 2 < kAB) read_a(kt_next, 1 - ks, (n - 9) / 2, next);
-        // This sub-step's share of the loads of ring step kt + 2.
+        // This sub-step's share of the loads of ring step kt + 2. Inside the
+        // depth: the LDS address goes to M0 behind the instruction before.
+        if constexpr (decltype(full)::value && n >= 11 && (n - 11) % 6 == 0 && (n - 11) / 6 < 8) {
+          constexpr int l = (n - 11) / 6;
+          const uint32_t stage = lds_base + ((kt + C::kStages) % C::kStages) * C::kStageBytes;
+          SetLdsTarget(stage + (ks == 0 ? C::kBM * kBK : 0) + (wave * C::kALoads + l) * 1024);
+        }
         if constexpr (n >= 12 && (n - 12) % 6 == 0 && (n - 12) / 6 < 8) {
-          constexpr int l = (ks == 0 ? C::kALoads : 0) + (n - 12) / 6;
-          if (decltype(full)::value)
-            issue_one_full(kt + C::kStages, l);
+          constexpr int l = (n - 12) / 6;
+          if constexpr (decltype(full)::value)
+            LoadToLdsTarget16(ks == 0 ? b_goff[l] : a_goff[l], uint32_t(kt + C::kStages) * kBK, ks == 0 ? b_rsrc : a_rsrc);
           else
-            issue_one(kt + C::kStages, l);
+            issue_one(kt + C::kStages, (ks == 0 ? C::kALoads : 0) + l);
         }
       });
       __builtin_amdgcn_sched_barrier(0);
