@@ -26,7 +26,7 @@ struct F32Traits {
   static __device__ __forceinline__ void DrainMma() {}
   static constexpr int kBlock = 32;
   static constexpr bool kRawB = false;
-  static constexpr bool kStaggered = false;
+  static constexpr bool kPaired = false;
   using LargeTile = F32Traits;
   static constexpr bool kSplitB = false;
   static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kF32;

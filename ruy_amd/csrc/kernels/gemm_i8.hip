@@ -38,7 +38,7 @@ struct Int8Traits {
   static __device__ __forceinline__ void DrainMma() {}
   static constexpr int kBlock = 32;
   static constexpr bool kRawB = false;
-  static constexpr bool kStaggered = false;
+  static constexpr bool kPaired = false;
   // The 256x256 tile runs on 16x16 blocks (below).
   using LargeTile = Int8Traits16;
   static constexpr bool kSplitB = false;
@@ -136,10 +136,13 @@ struct Int8Traits {
 // itself: given the builtin, the compiler's register allocator moves dozens of
 // these small accumulators between registers on every trip round the loop.
 // The compiler's hazard checks do not look inside inline assembly; the kernel
-// keeps what they would have ensured: consecutive instructions never share an
-// accumulator, an accumulator is next touched 63 instructions later, and
-// DrainMma() stands between the last instruction and the first ordinary read
-// of an accumulator.
+// keeps what they would have ensured: an accumulator is only ever touched by
+// these instructions between the first one and DrainMma(), which stands
+// between the last one and the first ordinary read of an accumulator. Two of
+// them in a row on the same accumulator (the paired schedule) are the one
+// dependency the matrix pipe resolves itself, by handing the block from one
+// instruction to the next; any other accumulator is next touched 126
+// instructions later.
 struct Int8Traits16 : Int8Traits {
   using Acc = v4i;
   static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
@@ -151,7 +154,7 @@ struct Int8Traits16 : Int8Traits {
   }
   static __device__ __forceinline__ void DrainMma() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
   static constexpr int kBlock = 16;
-  static constexpr bool kStaggered = true;  // the operands' rings half a step apart (see the kernel)
+  static constexpr bool kPaired = true;  // both depth halves of a ring step on one accumulator in a row (see the kernel)
   using LargeTile = Int8Traits16;
 
   // ---- write-back parameters of the 16x16-block kernel ----

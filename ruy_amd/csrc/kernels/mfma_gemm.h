@@ -158,6 +158,10 @@ __device__ __forceinline__ int LdsOffset(int r, int g) {
   return r * BK + ((g ^ Swizzle<BK>(r)) << 4);
 }
 
+// The paired schedule of the largest int8 tile (see the kernel): the block
+// column (of eight) at position `cp` of half `h` of a ring step of the given parity.
+constexpr int PairedColumnAt(int parity, int h, int cp) { return (parity ^ h) == 0 ? cp : 7 - cp; }
+
 template <int WM, int WN, int BK, int STAGES, bool SPLIT_B = false, int BLOCK = 32>
 struct Cfg {
   static constexpr int kBM = 2 * WM * 32;
@@ -392,9 +396,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
         for (int v = 0; v < kAccElems; ++v) acc[i][j][v] = 0;
   };
-  // (The staggered schedule starts its first matrix instructions from zero
+  // (The paired schedule starts its first matrix instructions from zero
   // instead: 256 register writes fewer per tile.)
-  if constexpr (!Traits::kStaggered) clear_accumulators();
+  if constexpr (!Traits::kPaired) clear_accumulators();
 
   typename Traits::Acc sum_a, sum_b;  // kFusedSums: row sums of a / column sums of b, in every column / row
 #pragma unroll
@@ -716,56 +720,52 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           for (int e = 0; e < 4; ++e) acc[0][j][4 * q + e] += Traits::FromRawBits(w[e]);
         }
     }
-  } else if constexpr (Traits::kStaggered) {
-    // ---- the largest int8 tile: the two operands' rings half a step apart ----
-    // A direct-to-LDS load of 1 KiB keeps the CU's one address unit busy for 16
-    // cycles, and a ring step of this tile needs 64 of them, 1024 of the 2048
-    // cycles its matrix instructions take. With one ring for both operands a
-    // slot comes free in the middle of a ring step (when the fragments of the
-    // step's second sub-step have been read), so all 64 loads had to be issued
-    // during that second sub-step, which kept the address unit busy throughout
-    // it and the matrix instructions waiting behind the loads. Here the A half
-    // and the B half of a slot are freed at different times, and every
-    // sub-step carries the loads of one operand:
-    //   sub-step (kt, 0): matrix instructions on A(kt,0) x B(kt,0); A(kt,1)
-    //     fragments read; loads of B for ring step kt+2 issued;
-    //   sub-step (kt, 1): matrix instructions on A(kt,1) x B(kt,1); A(kt+1,0)
-    //     fragments read; loads of A for ring step kt+2 issued.
-    // For B's half-slot to be free at the start of ring step kt, B's fragments
-    // are read a whole ring step ahead: the instructions of a sub-step walk the
-    // blocks column by column, so that B fragment j is used by eight
-    // consecutive instructions, after which its registers take the fragment of
-    // the same column and sub-step of ring step kt+1 (two instructions later;
-    // for the last column that is the second instruction of the next
-    // sub-step). No more registers than two sets of fragments, as before.
+  } else if constexpr (Traits::kPaired) {
+    // ---- the largest int8 tile: both depth halves of a ring step on one accumulator in a row ----
+    // Two matrix instructions in a row on the same accumulator block (the two
+    // 64-byte halves of a 128-byte ring step) pass the block from one to the
+    // other without the trip through the register file in between, which on
+    // random operand bytes, where the power limit sets the clock, is worth 5 %
+    // to a bare loop of these instructions. So a ring step is 64 such pairs,
+    // and the fragments of both halves are in registers at once: 16 for A and
+    // 16 for B, the registers the other schedules use as two buffers.
     //
-    // One barrier per sub-step, in front of its ninth instruction, so that the
-    // few LDS reads issued just before it have the first eight to finish
-    // behind. It says: every wave has the fragments it wanted from the half-slot
-    // that this sub-step's loads overwrite (B: read up to the second
-    // instruction of this sub-step; A: read during the previous sub-step), and
-    // the loads that the reads behind it rely on have landed for all waves -
-    // all but the eight issued during the previous sub-step, which belong to
-    // the other operand and are older than nothing this sub-step reads.
+    // Without a second buffer a fragment's registers can only take their next
+    // value once the last pair that needs them has been issued, and it must
+    // have arrived from LDS before the first pair of the next ring step that
+    // needs it. The order of the pairs leaves every fragment at least 56
+    // instructions between the two: the tile is walked as two halves of four
+    // block rows each, every half column by column (four pairs a column), the
+    // second half in the opposite column order of the first, and the next ring
+    // step's first half in the column order of this one's second half.
+    //   A rows 0-3 are done with after the first half: their next values are
+    //     read during the second half.
+    //   A rows 4-7 are done with at the end: their next values are read during
+    //     the first half of the next ring step (which does not need them).
+    //   B column at position p of the second half is done with 8 (p + 1)
+    //     instructions into that half and is needed 8 p instructions into the
+    //     next ring step. The first four are read as they come free, the last
+    //     four during the first instructions of the next ring step.
+    // Ring: two slots. The B half of slot kt % 2 has been read by every wave
+    // once the "last four" reads of step kt are done (barrier 1, in front of
+    // instruction 16), the A half once rows 4-7 have been read (barrier 2, in
+    // front of instruction 64); the loads of step kt + 2 follow each barrier,
+    // one every sixth instruction. Barrier 2 is also where every wave has waited
+    // for all its loads but the eight just issued, i.e. for everything of step
+    // kt + 1, which the second half starts to read.
     static_assert(kB == 16 && C::kKSteps == 2 && C::kStages == 2 && kAB == 8 && kBB == 8 && C::kALoads == 8 &&
                       C::kBLoads == 8 && !kFlip && !kFusedSums,
-                  "the staggered schedule is written for the 256x256 tile of 16x16 blocks");
-    struct AFrags {
-      v4i a[kAB];
-    };
-    AFrags fa[2];
-    v4i fb[2][kBB];
-    auto read_a = [&](int kt, int ks, int i, AFrags& f) {
+                  "the paired schedule is written for the 256x256 tile of 16x16 blocks");
+    v4i fa[2][kAB];  // [depth half][block row]
+    v4i fb[2][kBB];  // [depth half][block column]
+    auto read_a = [&](int kt, int ks, int i) {
       const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
-      f.a[i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * kB * kBK);
+      fa[ks][i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * kB * kBK);
     };
-    auto read_b = [&](int kt, int ks, int j, v4i& into) {
+    auto read_b = [&](int kt, int ks, int j) {
       const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
-      into = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * kB * kBK);
+      fb[ks][j] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * kB * kBK);
     };
-    // B of step 0, A of step 0, B of step 1, A of step 1: the order in which
-    // the loop goes on issuing them, so that "all but the last eight" means
-    // the same before the loop as inside it.
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
 #pragma unroll
@@ -773,87 +773,109 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
       for (int l = 0; l < C::kALoads; ++l) issue_one(st, l);
     }
-    WaitVmcnt<C::kALoads>();
+    WaitVmcnt<C::kALoads + C::kBLoads>();
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < kAB; ++i) read_a(0, 0, i, fa[0]);
+    for (int i = 0; i < kAB / 2; ++i) {
+      read_a(0, 0, i);
+      read_a(0, 1, i);
+    }
 #pragma unroll
-    for (int j = 0; j < kBB; ++j) read_b(0, 0, j, fb[0][j]);
-#pragma unroll
-    for (int j = 0; j + 1 < kBB; ++j) read_b(0, 1, j, fb[1][j]);
-    // `first`: the tile's first sub-step, whose matrix instructions start from
-    // zero instead of from the accumulators (which nobody has cleared).
-    auto staggered_sub_step = [&](int kt, auto ks_constant, auto full, auto first) {
-      constexpr int ks = decltype(ks_constant)::value;
-      const AFrags& cur = fa[ks];
-      AFrags& next = fa[1 - ks];
-      const int kt_next = ks == 0 ? kt : kt + 1;
-      StaticFor<kMmas>([&](auto n_constant) {
+    for (int cp = 0; cp < kBB / 2; ++cp) {
+      read_b(0, 0, cp);
+      read_b(0, 1, cp);
+    }
+    // The bounds-tested form of a load for the last ring steps. The depth
+    // granule a lane fetches (after the swizzle) depends on the parity of the
+    // load's number only and is the same for both operands: two registers
+    // instead of the sixteen of a_k / b_k, in code that has none to spare.
+    const int tail_k[2] = {a_k[0], a_k[1]};
+    auto issue_tail = [&](int kt_load, auto is_b, int l) {
+      const int kbase = kt_load * kBK;
+      const uint32_t stage = lds_base + (kt_load % C::kStages) * C::kStageBytes;
+      const uint32_t goff = decltype(is_b)::value ? b_goff[l] : a_goff[l];
+      const uint32_t off = kbase + tail_k[l & 1] < K ? goff + kbase : kOutOfRange;
+      LoadToLds16(stage + (decltype(is_b)::value ? C::kBM * kBK : 0) + (wave * C::kALoads + l) * 1024, off,
+                  decltype(is_b)::value ? b_rsrc : a_rsrc);
+    };
+    // Barrier 1 stands in front of this instruction; the eight B loads follow it.
+    constexpr int kBarrier1 = 24, kLoadB0 = 26, kLoadBStride = 5;
+    static_assert(kLoadB0 > kBarrier1 && kLoadB0 + 7 * kLoadBStride < 64, "");
+    auto paired_step = [&](int kt, auto parity_constant, auto full, auto first) {
+      constexpr int kParity = decltype(parity_constant)::value;
+      StaticFor<2 * kMmas>([&](auto n_constant) {
         constexpr int n = decltype(n_constant)::value;
-        constexpr int j = n / kAB;
-        constexpr int i = n % kAB;
-        if constexpr (n == 8) {
+        constexpr int pair = n / 2;
+        constexpr int ks = n % 2;
+        constexpr int h = pair / 32;
+        constexpr int cp = (pair % 32) / 4;
+        constexpr int rp = pair % 4;
+        constexpr int j = PairedColumnAt(kParity, h, cp);
+        constexpr int i = 4 * h + (cp % 2 == 0 ? rp : 3 - rp);
+        if constexpr (n == kBarrier1) __syncthreads();
+        if constexpr (n == 64) {
           WaitVmcnt<8>();
           __syncthreads();
         }
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (decltype(first)::value)
-          Traits::MmaFromZero(cur.a[i], fb[ks][j], acc[i][j]);
+        if constexpr (decltype(first)::value && ks == 0)
+          Traits::MmaFromZero(fa[ks][i], fb[ks][j], acc[i][j]);
         else
-          Traits::Mma(cur.a[i], fb[ks][j], acc[i][j]);
+          Traits::Mma(fa[ks][i], fb[ks][j], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
-        // The last column's B fragment of the sub-step before this one.
-        if constexpr (n == 1) {
-          if constexpr (ks == 0)
-            read_b(kt, 1, kBB - 1, fb[1][kBB - 1]);
-          else
-            read_b(kt + 1, 0, kBB - 1, fb[0][kBB - 1]);
+        // The last four columns of this step's first half (needed from instruction 32 on).
+        if constexpr (n < 16 && n % 2 == 0) read_b(kt, n / 2 % 2, PairedColumnAt(kParity, 0, 4 + n / 4));
+        // A rows 4-7 of this step.
+        if constexpr (n >= kBarrier1 + 1 && n < kBarrier1 + 25 && (n - kBarrier1) % 3 == 1)
+          read_a(kt, (n - kBarrier1 - 1) / 3 % 2, 4 + (n - kBarrier1 - 1) / 6);
+        // A rows 0-3 of the next step.
+        if constexpr (n >= 65 && n < 81 && n % 2 == 1) read_a(kt + 1, (n - 65) / 2 % 2, (n - 65) / 4);
+        // The first four columns of the second half, as they come free.
+        if constexpr (n >= 72 && n < 104 && (n % 8 == 0 || n % 8 == 2))
+          read_b(kt + 1, n % 8 / 2, PairedColumnAt(kParity, 1, (n - 72) / 8));
+        // The loads of ring step kt + 2: B behind barrier 1, A behind barrier 2.
+        // Inside the depth the LDS address goes to M0 behind the instruction before.
+        constexpr bool kLoadB = n >= kLoadB0 && n < 64 && (n - kLoadB0) % kLoadBStride == 0;
+        constexpr bool kLoadA = n >= 66 && n < 112 && (n - 66) % 6 == 0;
+        constexpr bool kTargetB = n + 1 >= kLoadB0 && n + 1 < 64 && (n + 1 - kLoadB0) % kLoadBStride == 0;
+        constexpr bool kTargetA = n + 1 >= 66 && n + 1 < 112 && (n + 1 - 66) % 6 == 0;
+        if constexpr (decltype(full)::value && (kTargetA || kTargetB)) {
+          constexpr int l = kTargetB ? (n + 1 - kLoadB0) / kLoadBStride : (n + 1 - 66) / 6;
+          const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
+          SetLdsTarget(stage + (kTargetB ? C::kBM * kBK : 0) + (wave * C::kALoads + l) * 1024);
         }
-        // Column jj is done with: its fragment of the next ring step.
-        if constexpr (n >= 9 && (n - 9) % kAB == 0 && (n - 9) / kAB < kBB - 1) {
-          constexpr int jj = (n - 9) / kAB;
-          read_b(kt + 1, ks, jj, fb[ks][jj]);
-        }
-        // The A fragments of the next sub-step.
-        if constexpr (n >= 9 && n % 2 == 1 && (n - 9) / 2 < kAB) read_a(kt_next, 1 - ks, (n - 9) / 2, next);
-        // This sub-step's share of the loads of ring step kt + 2. Inside the
-        // depth: the LDS address goes to M0 behind the instruction before.
-        if constexpr (decltype(full)::value && n >= 11 && (n - 11) % 6 == 0 && (n - 11) / 6 < 8) {
-          constexpr int l = (n - 11) / 6;
-          const uint32_t stage = lds_base + ((kt + C::kStages) % C::kStages) * C::kStageBytes;
-          SetLdsTarget(stage + (ks == 0 ? C::kBM * kBK : 0) + (wave * C::kALoads + l) * 1024);
-        }
-        if constexpr (n >= 12 && (n - 12) % 6 == 0 && (n - 12) / 6 < 8) {
-          constexpr int l = (n - 12) / 6;
+        if constexpr (kLoadA || kLoadB) {
+          constexpr int l = kLoadB ? (n - kLoadB0) / kLoadBStride : (n - 66) / 6;
           if constexpr (decltype(full)::value)
-            LoadToLdsTarget16(ks == 0 ? b_goff[l] : a_goff[l], uint32_t(kt + C::kStages) * kBK, ks == 0 ? b_rsrc : a_rsrc);
+            LoadToLdsTarget16(kLoadB ? b_goff[l] : a_goff[l], uint32_t(kt + C::kStages) * kBK, kLoadB ? b_rsrc : a_rsrc);
           else
-            issue_one(kt + C::kStages, (ks == 0 ? C::kALoads : 0) + l);
+            issue_tail(kt + C::kStages, std::integral_constant<bool, kLoadB>(), l);
         }
       });
       __builtin_amdgcn_sched_barrier(0);
     };
     const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
-    using Sub0 = std::integral_constant<int, 0>;
-    using Sub1 = std::integral_constant<int, 1>;
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
     int kt = 1;
     if (full_end > 0) {
-      staggered_sub_step(0, Sub0(), std::true_type(), std::true_type());
-      staggered_sub_step(0, Sub1(), std::true_type(), std::false_type());
+      paired_step(0, Even(), std::true_type(), std::true_type());
     } else if (k_tiles > 0) {
-      staggered_sub_step(0, Sub0(), std::false_type(), std::true_type());
-      staggered_sub_step(0, Sub1(), std::false_type(), std::false_type());
+      paired_step(0, Even(), std::false_type(), std::true_type());
     } else {
       clear_accumulators();
     }
-    for (; kt < full_end; ++kt) {
-      staggered_sub_step(kt, Sub0(), std::true_type(), std::false_type());
-      staggered_sub_step(kt, Sub1(), std::true_type(), std::false_type());
+    for (; kt + 1 < full_end; kt += 2) {
+      paired_step(kt, Odd(), std::true_type(), std::false_type());
+      paired_step(kt + 1, Even(), std::true_type(), std::false_type());
     }
-    for (; kt < k_tiles; ++kt) {
-      staggered_sub_step(kt, Sub0(), std::false_type(), std::false_type());
-      staggered_sub_step(kt, Sub1(), std::false_type(), std::false_type());
+    // (Straight-line loop bodies only: with a branch on the step's parity in
+    // the loop the register allocator moves accumulators through scratch memory.)
+    for (; kt + 1 < k_tiles; kt += 2) {
+      paired_step(kt, Odd(), std::false_type(), std::false_type());
+      paired_step(kt + 1, Even(), std::false_type(), std::false_type());
     }
+    if (kt < k_tiles) paired_step(kt, Odd(), std::false_type(), std::false_type());
   } else {
 #pragma unroll
     for (int s = 0; s < C::kStages; ++s) issue(s);
