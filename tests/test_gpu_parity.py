@@ -825,6 +825,36 @@ def test_grids_cut_into_two_launches(device_ctx, shape, tup):
         assert ((got.sum(axis=1) % 2**32) == (L @ R.sum(axis=1)) % 2**32).all()
 
 
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I16), (S.I8, S.U8, S.I32, S.I32)],
+                         ids=cases.tuple_name)
+def test_largest_tile_over_depth_step_counts(device_ctx, tup):
+    """A 4096 x 4096 destination is one round of 256x256 tiles, whose main loop
+    takes its 128-byte depth steps in pairs (an even and an odd form) after a
+    first step of its own, with a separate form of the loads for the last
+    steps: depths of one to seven steps, whole and partial last steps, depths
+    that are not a multiple of 16 (packed operands), ragged destination edges,
+    per-channel parameters and zero points as the random problem draws them,
+    all three destination widths. Every element where the stock reference
+    library is built (see test_full_size_int8_gemm_8192), a sample of rows and
+    columns either side of every tile edge otherwise and in any case."""
+    import device_runner as D
+    rng = np.random.default_rng(4242 + tup[3])
+    for K, M, N in [(16, 4096, 4096), (112, 4096, 4096), (128, 4000, 4090), (144, 4096, 4096), (256, 4096, 3900),
+                    (300, 4096, 4096), (384, 4096, 4096), (500, 3850, 4096), (640, 4096, 4096), (896, 4096, 4096)]:
+        p = W.random_problem(rng, *tup, M, K, N, *cases.RCC, strided=False,
+                             name="%s %s" % (cases.tuple_name(tup), (M, K, N)))
+        announce(p.name)
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        assert device_ctx.last_kernel_name() == "i8_mfma"
+        rows, cols = _boundary_sample(rng, M), _boundary_sample(rng, N)
+        g, w = _sample_block(p, got, rows, cols)
+        assert (g == w).all(), "%s: %d mismatches in the sampled block" % (p.name, (g != w).sum())
+        want = O.full_size_expected(p)
+        if want is not None:
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+
+
 @pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I16), (S.I8, S.I16, S.I32, S.I16),
                                  (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
 def test_base_addresses_that_are_not_aligned(device_ctx, tup):
