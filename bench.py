@@ -247,7 +247,7 @@ def bench_mfma_ceiling(ctx, settle_ms=150.0, only_best=False):
     registers or re-read from LDS, all-zero or uniformly random operands."""
     out = []
     combos = [(1, 0, 1)] if only_best else [(i, l, r) for i in (0, 1) for l in (0, 1) for r in (0, 1)]
-    names = ("v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8")
+    names = ("v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8 (two in a row per accumulator block)")
     for instruction, from_lds, random_operands in combos:
         tops, ms = ctx.mfma_ceiling(instruction, from_lds, random_operands, settle_ms)
         out.append({"instruction": names[instruction],
