@@ -246,8 +246,9 @@ def bench_mfma_ceiling(ctx, settle_ms=150.0, only_best=False):
     (ruyamd_diag_mfma_ceiling): both instruction shapes, fragments kept in
     registers or re-read from LDS, all-zero or uniformly random operands."""
     out = []
-    combos = [(1, 0, 1)] if only_best else [(i, l, r) for i in (0, 1) for l in (0, 1) for r in (0, 1)]
-    names = ("v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8 (two in a row per accumulator block)")
+    combos = [(1, 0, 1)] if only_best else [(i, l, r) for i in (0, 2, 1) for l in (0, 1) for r in (0, 1)]
+    names = ("v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8 (two in a row per accumulator block)",
+             "v_mfma_i32_16x16x64_i8 (every instruction on another accumulator)")
     for instruction, from_lds, random_operands in combos:
         tops, ms = ctx.mfma_ceiling(instruction, from_lds, random_operands, settle_ms)
         out.append({"instruction": names[instruction],

@@ -285,9 +285,10 @@ RUYAMD_API int ruyamd_apply_multiplier(ruyamd_ctx* ctx, const int32_t* x,
 
 /* What the int8 matrix instructions sustain on this card when nothing else
  * runs: one wave per SIMD, each with the 128 x 128 accumulator tile of the
- * large GEMM tile, issuing `instruction` 0 = v_mfma_i32_32x32x32_i8 or
- * 1 = v_mfma_i32_16x16x64_i8 (in that tile's order: two in a row on each
- * accumulator block) back to back on fragments held in registers
+ * large GEMM tile, issuing `instruction` 0 = v_mfma_i32_32x32x32_i8,
+ * 1 = v_mfma_i32_16x16x64_i8 in that tile's order (two in a row on each
+ * accumulator block) or 2 = the same instructions with every one on another
+ * accumulator than the one before, back to back on fragments held in registers
  * (`operands_from_lds` = 0) or re-read from LDS with one workgroup barrier per
  * 128 bytes of depth (1); operands all zero (`random_operands` = 0) or
  * uniformly random bytes (1). The card is first kept under this load for

@@ -17,7 +17,7 @@ extern "C" int ruyamd_diag_mfma_ceiling(ruyamd_ctx* ctx, int instruction, int op
     ctx->last_error = msg;
     return code;
   };
-  if (!tera_ops_per_second || !ms_per_launch || instruction < 0 || instruction > 1 || settle_ms < 0)
+  if (!tera_ops_per_second || !ms_per_launch || instruction < 0 || instruction > 2 || settle_ms < 0)
     return fail(RUYAMD_E_INVALID, "bad argument");
   if (hipSetDevice(ctx->device) != hipSuccess) return fail(RUYAMD_E_HIP, "hipSetDevice failed");
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;

@@ -10,6 +10,8 @@
 // the 256 x 256 GEMM tile. One iteration is a depth of 128 bytes:
 //   instruction 0: 4 x (4 + 4 fragments, 16 v_mfma_i32_32x32x32_i8)
 //   instruction 1: 2 x (8 + 8 fragments), 64 pairs of v_mfma_i32_16x16x64_i8
+//     (the two depth halves of a block back to back on its accumulator)
+//   instruction 2: the same 128 instructions, one depth half after the other
 // i.e. 2 * 128^3 operations per wave and iteration in both forms, and the same
 // 32 KiB of fragment bytes.
 #include <hip/hip_runtime.h>
@@ -102,16 +104,30 @@ __global__ __launch_bounds__(256) void MfmaCeilingKernel(const v4i* operands, in
             b[ks][i] = *reinterpret_cast<const v4i*>(lds + ((t + i * 4096 + ks * 1024 + 512 + it * 64) & (kLdsBytes - 16)));
           }
       }
+      // Accumulator tied to itself: with the builtin the compiler moves these
+      // small accumulators between registers inside the loop.
+      if constexpr (kInstruction == 1) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int ii = 0; ii < 8; ++ii) {
-          const int i = (j & 1) ? 7 - ii : ii;
-          // Accumulator tied to itself: with the builtin the compiler moves these
-          // small accumulators between registers inside the loop.
-          asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[i][j]) : "v"(a[0][i]), "v"(b[0][j]));
-          asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[i][j]) : "v"(a[1][i]), "v"(b[1][j]));
-        }
+          for (int ii = 0; ii < 8; ++ii) {
+            const int i = (j & 1) ? 7 - ii : ii;
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[i][j]) : "v"(a[0][i]), "v"(b[0][j]));
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[i][j]) : "v"(a[1][i]), "v"(b[1][j]));
+          }
+      } else {
+        // For comparison: one depth half after the other, every instruction
+        // on another accumulator than the one before it.
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int ii = 0; ii < 8; ++ii) {
+              const int i = (j & 1) ? 7 - ii : ii;
+              asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[i][j]) : "v"(a[ks][i]), "v"(b[ks][j]));
+            }
+      }
       if constexpr (kFromLds) __syncthreads();
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the last instructions finish before their results are read
@@ -146,6 +162,9 @@ hipError_t LaunchMfmaCeiling(hipStream_t stream, int instruction, bool from_lds,
   if (instruction == 1)
     return from_lds ? LaunchOne<1, true>(stream, operands, sink, iterations, workgroups)
                     : LaunchOne<1, false>(stream, operands, sink, iterations, workgroups);
+  if (instruction == 2)
+    return from_lds ? LaunchOne<2, true>(stream, operands, sink, iterations, workgroups)
+                    : LaunchOne<2, false>(stream, operands, sink, iterations, workgroups);
   return hipErrorInvalidValue;
 }
 
