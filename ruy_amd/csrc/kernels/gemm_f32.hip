@@ -37,29 +37,55 @@ struct F32Traits {
   static __device__ __forceinline__ int RawBits(float x) { return __float_as_int(x); }
   static __device__ __forceinline__ float FromRawBits(int w) { return __int_as_float(w); }
 
-  struct EdgeParams {};  // (kernels on 16x16 blocks only)
+  // Write-back parameters (the scheme of the int8 kernels): the bias of the
+  // wave's rows or columns, fetched by lane l for rows and columns l and
+  // l + 64 when the workgroup starts and handed round through LDS when the
+  // write-back starts.
+  static constexpr int kParamInts = 6 * 128;  // (the int8 kernels' area; rows at 0, columns at 3 * 128)
+  struct EdgeParams {
+    float bias[4];  // [0..1]: rows l, l + 64; [2..3]: columns l, l + 64
+  };
+  static __device__ __forceinline__ void LoadEdgeParams(const Epilogue& ep, const int (&row)[2], const int (&col)[2],
+                                                        EdgeParams& p) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) p.bias[k] = 0.f;
+    const float* bias = static_cast<const float*>(ep.bias);
+    if (bias && !ep.channel_is_col) {
+      p.bias[0] = bias[row[0]];
+      p.bias[1] = bias[row[1]];
+    }
+    if (bias && ep.channel_is_col) {
+      p.bias[2] = bias[col[0]];
+      p.bias[3] = bias[col[1]];
+    }
+  }
+  static __device__ __forceinline__ void Stage(const Epilogue&, const EdgeParams& p, int* area, int lane) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) area[(k < 2 ? 0 : 3 * 128) + lane + (k & 1) * 64] = __float_as_int(p.bias[k]);
+  }
   struct RowState {
     float bias[16];
-    __device__ __forceinline__ void Load(const Epilogue& ep, const int (&row_idx)[16]) {
+    __device__ __forceinline__ void Read(const int* area, int first) {
 #pragma unroll
-      for (int q = 0; q < 16; ++q) bias[q] = 0.f;
-      if (ep.bias && !ep.channel_is_col) {
-        const float* b = static_cast<const float*>(ep.bias);
+      for (int q = 0; q < 4; ++q) {
+        const v4i b = *reinterpret_cast<const v4i*>(area + first + 4 * q);
 #pragma unroll
-        for (int q = 0; q < 16; ++q) bias[q] = b[row_idx[q]];
+        for (int v = 0; v < 4; ++v) bias[4 * q + v] = __int_as_float(b[v]);
       }
     }
   };
+  struct ColState {
+    float bias;
+    __device__ __forceinline__ void Read(const int* area, int col) { bias = __int_as_float(area[3 * 128 + col]); }
+  };
 
-  static __device__ __forceinline__ void Finish(int32_t (&vals)[16], const RowState& rows, int j,
+  static __device__ __forceinline__ void Finish(int32_t (&vals)[16], const RowState& rows, const ColState& column,
                                                 const Epilogue& ep) {
     const bool has_bias = ep.bias != nullptr;
-    float col_bias = 0.f;
-    if (has_bias && ep.channel_is_col) col_bias = static_cast<const float*>(ep.bias)[j];
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
       float v = __int_as_float(vals[q]);
-      if (has_bias) v = v + (ep.channel_is_col ? col_bias : rows.bias[q]);
+      if (has_bias) v = v + (ep.channel_is_col ? column.bias : rows.bias[q]);
       v = ep.clamp_max_f < v ? ep.clamp_max_f : v;
       v = v < ep.clamp_min_f ? ep.clamp_min_f : v;
       vals[q] = __float_as_int(v);

@@ -50,125 +50,18 @@ struct Int8Traits {
   static __device__ __forceinline__ int RawBits(int x) { return x; }
   static __device__ __forceinline__ int FromRawBits(int w) { return w; }
 
-  struct EdgeParams {};  // (kernels on 16x16 blocks only)
-  struct RowState {
-    uint32_t add[16];
-    int32_t m[16];
-    int32_t e[16];
-    __device__ __forceinline__ void Load(const Epilogue& ep, const int (&row_idx)[16]) {
-      const bool row_channel = !ep.channel_is_col;
-#pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        add[q] = static_cast<uint32_t>(ep.zp_product_depth);
-        m[q] = ep.mult_fixedpoint_scalar;
-        e[q] = ep.mult_exponent_scalar;
-      }
-      if (ep.bias && row_channel) {
-        const int32_t* bias = static_cast<const int32_t*>(ep.bias);
-#pragma unroll
-        for (int q = 0; q < 16; ++q) add[q] += static_cast<uint32_t>(bias[row_idx[q]]);
-      }
-      if (ep.rhs_zero_point) {
-#pragma unroll
-        for (int q = 0; q < 16; ++q)
-          add[q] -= static_cast<uint32_t>(ep.rhs_zero_point) * static_cast<uint32_t>(ep.lhs_sums[row_idx[q]]);
-      }
-      if (ep.mult_fixedpoint && row_channel) {
-#pragma unroll
-        for (int q = 0; q < 16; ++q) {
-          m[q] = ep.mult_fixedpoint[row_idx[q]];
-          e[q] = ep.mult_exponent[row_idx[q]];
-        }
-      }
-    }
-  };
-
-  static __device__ __forceinline__ void Finish(int32_t (&vals)[16], const RowState& rows, int j,
-                                                const Epilogue& ep) {
-    const bool row_channel = !ep.channel_is_col;
-    const bool per_channel = ep.mult_fixedpoint != nullptr;
-    uint32_t col_add = 0;
-    int32_t col_m = 0, col_e = 0;
-    if (ep.bias && !row_channel) col_add += static_cast<uint32_t>(static_cast<const int32_t*>(ep.bias)[j]);
-    if (ep.lhs_zero_point)
-      col_add -= static_cast<uint32_t>(ep.lhs_zero_point) * static_cast<uint32_t>(ep.rhs_sums[j]);
-    if (per_channel && !row_channel) {
-      col_m = ep.mult_fixedpoint[j];
-      col_e = ep.mult_exponent[j];
-    }
-#pragma unroll
-    for (int q = 0; q < 16; ++q)
-      vals[q] = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + rows.add[q] + col_add);
-    // One wave-uniform branch per column, straight-line code per element.
-    // Fast path: scalar multiplier with exponent <= -2.
-    if (ep.requantize && !per_channel && ep.mult_exponent_scalar <= -2) {
-      const int32_t m = ep.mult_fixedpoint_scalar;
-      const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
-#pragma unroll
-      for (int q = 0; q < 16; ++q) vals[q] = RequantHigh(vals[q], m, high_shift);
-    } else if (ep.requantize) {
-      if (per_channel && !row_channel) {
-#pragma unroll
-        for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], col_m, col_e);
-      } else {
-#pragma unroll
-        for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], rows.m[q], rows.e[q]);
-      }
-    }
-    // The host hands over ordered clamp bounds (clamp_min <= clamp_max), for
-    // which min-then-max is the median of the three.
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
-      vals[q] = Median3(v, ep.clamp_min_i, ep.clamp_max_i);
-    }
-  }
-};
-
-// The same arithmetic on v_mfma_i32_16x16x64_i8: a quarter of the accumulator
-// registers read and written per instruction for half the operations, which on
-// random operand bytes, where the card runs into its power limit, costs about
-// a tenth less energy per operation than the 32x32x32 form; the fragment bytes
-// read from LDS per operation are the same. Used for the largest tile, whose
-// grids run long enough for the power limit to decide the clock.
-//
-// The instruction is written as inline assembly with the accumulator tied to
-// itself: given the builtin, the compiler's register allocator moves dozens of
-// these small accumulators between registers on every trip round the loop.
-// The compiler's hazard checks do not look inside inline assembly; the kernel
-// keeps what they would have ensured: an accumulator is only ever touched by
-// these instructions between the first one and DrainMma(), which stands
-// between the last one and the first ordinary read of an accumulator. Two of
-// them in a row on the same accumulator (the paired schedule) are the one
-// dependency the matrix pipe resolves itself, by handing the block from one
-// instruction to the next; any other accumulator is next touched 126
-// instructions later.
-struct Int8Traits16 : Int8Traits {
-  using Acc = v4i;
-  static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
-    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-  }
-  // The same with zero in place of the accumulator going in.
-  static __device__ __forceinline__ void MmaFromZero(const v4i& a, const v4i& b, Acc& acc) {
-    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
-  }
-  static __device__ __forceinline__ void DrainMma() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
-  static constexpr int kBlock = 16;
-  static constexpr bool kPaired = true;  // both depth halves of a ring step on one accumulator in a row (see the kernel)
-  using LargeTile = Int8Traits16;
-
-  // ---- write-back parameters of the 16x16-block kernel ----
-  // A wave's 128 rows and 128 columns each have three write-back parameters:
-  // what is added to the accumulator (bias, zero-point corrections; the
-  // constant part sits with the rows), and the multiplier and exponent that
-  // apply if the channels run along that dimension. Lane l fetches them for
-  // rows and columns l and l + 64 of the wave when the workgroup starts
-  // (EdgeParams: loads only, nothing computed, so nobody waits for them), and
-  // the wave puts them into an LDS area of its own when the write-back starts
-  // (Stage). From there every lane reads those of the rows and columns its
-  // accumulators belong to: LDS reads, so that inside the write-back loops
-  // nothing waits on the vector-memory counter, which would also mean waiting
-  // for the stores just issued.
+  // ---- write-back parameters ----
+  // A wave's rows and columns (up to 128 of each) have three write-back
+  // parameters each: what is added to the accumulator (bias, zero-point
+  // corrections; the constant part sits with the rows), and the multiplier and
+  // exponent that apply if the channels run along that dimension. Lane l
+  // fetches them for rows and columns l and l + 64 of the wave when the
+  // workgroup starts (EdgeParams: loads only, nothing computed, so nobody
+  // waits for them), and the wave puts them into an LDS area of its own when
+  // the write-back starts (Stage). From there every lane reads those of the
+  // rows and columns its accumulators belong to: LDS reads, so that inside the
+  // write-back loops nothing waits on the vector-memory counter, which would
+  // also mean waiting for the stores just issued.
   static constexpr int kParamInts = 6 * 128;  // per wave: row add, m, e; column add, m, e
   struct EdgeParams {
     int32_t bias[4], sums[4], m[4], e[4];  // [0..1]: rows l, l + 64; [2..3]: columns l, l + 64
@@ -227,6 +120,103 @@ struct Int8Traits16 : Int8Traits {
       base[256] = p.e[k];
     }
   }
+  // 32x32 blocks: the parameters of the 16 consecutive rows (from `first` on,
+  // counted inside the wave's rows) that a lane writes, and of one column.
+  struct RowState {
+    uint32_t add[16];
+    int32_t m[16];
+    int32_t e[16];
+    __device__ __forceinline__ void Read(const int* area, int first) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4i a = *reinterpret_cast<const v4i*>(area + first + 4 * q);
+        const v4i mm = *reinterpret_cast<const v4i*>(area + 128 + first + 4 * q);
+        const v4i ee = *reinterpret_cast<const v4i*>(area + 256 + first + 4 * q);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          add[4 * q + v] = static_cast<uint32_t>(a[v]);
+          m[4 * q + v] = mm[v];
+          e[4 * q + v] = ee[v];
+        }
+      }
+    }
+  };
+  struct ColState {
+    uint32_t add;
+    int32_t m, e;
+    __device__ __forceinline__ void Read(const int* area, int col) {
+      add = static_cast<uint32_t>(area[3 * 128 + col]);
+      m = area[4 * 128 + col];
+      e = area[5 * 128 + col];
+    }
+  };
+
+  static __device__ __forceinline__ void Finish(int32_t (&vals)[16], const RowState& rows, const ColState& column,
+                                                const Epilogue& ep) {
+    const bool row_channel = !ep.channel_is_col;
+    const bool per_channel = ep.mult_fixedpoint != nullptr;
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+      vals[q] = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + rows.add[q] + column.add);
+    // One wave-uniform branch per column, straight-line code per element.
+    // Fast path: scalar multiplier with exponent <= -2.
+    if (ep.requantize && !per_channel && ep.mult_exponent_scalar <= -2) {
+      const int32_t m = ep.mult_fixedpoint_scalar;
+      const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
+#pragma unroll
+      for (int q = 0; q < 16; ++q) vals[q] = RequantHigh(vals[q], m, high_shift);
+    } else if (ep.requantize) {
+      if (per_channel && !row_channel) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], column.m, column.e);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) vals[q] = MultiplyByQuantizedMultiplier(vals[q], rows.m[q], rows.e[q]);
+      }
+    }
+    // The host hands over ordered clamp bounds (clamp_min <= clamp_max), for
+    // which min-then-max is the median of the three.
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int32_t v = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(ep.dst_zero_point));
+      vals[q] = Median3(v, ep.clamp_min_i, ep.clamp_max_i);
+    }
+  }
+};
+
+// The same arithmetic on v_mfma_i32_16x16x64_i8: a quarter of the accumulator
+// registers read and written per instruction for half the operations, which on
+// random operand bytes, where the card runs into its power limit, costs about
+// a tenth less energy per operation than the 32x32x32 form; the fragment bytes
+// read from LDS per operation are the same. Used for the largest tile, whose
+// grids run long enough for the power limit to decide the clock.
+//
+// The instruction is written as inline assembly with the accumulator tied to
+// itself: given the builtin, the compiler's register allocator moves dozens of
+// these small accumulators between registers on every trip round the loop.
+// The compiler's hazard checks do not look inside inline assembly; the kernel
+// keeps what they would have ensured: an accumulator is only ever touched by
+// these instructions between the first one and DrainMma(), which stands
+// between the last one and the first ordinary read of an accumulator. Two of
+// them in a row on the same accumulator (the paired schedule) are the one
+// dependency the matrix pipe resolves itself, by handing the block from one
+// instruction to the next; any other accumulator is next touched 126
+// instructions later.
+struct Int8Traits16 : Int8Traits {
+  using Acc = v4i;
+  static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+  // The same with zero in place of the accumulator going in.
+  static __device__ __forceinline__ void MmaFromZero(const v4i& a, const v4i& b, Acc& acc) {
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void DrainMma() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+  static constexpr int kBlock = 16;
+  static constexpr bool kPaired = true;  // both depth halves of a ring step on one accumulator in a row (see the kernel)
+  using LargeTile = Int8Traits16;
+
+  // ---- the 16x16-block form of the write-back (parameters: Int8Traits::EdgeParams and Stage) ----
   // Which form of the arithmetic a launch needs, decided once so that the
   // write-back loops carry no branches on it: a lone wave pays for every
   // branch with an empty instruction buffer.

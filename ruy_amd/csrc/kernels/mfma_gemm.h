@@ -187,12 +187,16 @@ struct Cfg {
   static constexpr int kEpilogueBlockCols = kLogicalWN >= 2 ? kLogicalWN / 2 : 1;
   static constexpr int kEpiloguePitch = WM * 32 + 4;
   static constexpr int kEpilogueBytes = 4 * kEpilogueBlockCols * 32 * kEpiloguePitch * 4;
-  // 16x16 blocks: no staging (the write-back transposes between lanes), but
-  // 3 KiB of write-back parameters per wave behind the ring.
+  // 3 KiB of write-back parameters per wave (those of its rows and columns,
+  // fetched ahead of the main loop and handed round through LDS): behind the
+  // ring for 16x16 blocks, whose write-back has no staging area (it transposes
+  // between lanes); behind the staging area, inside the ring's memory where
+  // that is large enough, for 32x32 blocks.
   static constexpr int kParamBytes = 4 * 6 * 128 * 4;
   static constexpr int kLdsBytes = BLOCK == 16 ? kStages * kStageBytes + kParamBytes
-                                               : (kStages * kStageBytes > kEpilogueBytes ? kStages * kStageBytes
-                                                                                         : kEpilogueBytes);
+                                               : (kStages * kStageBytes > kEpilogueBytes + kParamBytes
+                                                      ? kStages * kStageBytes
+                                                      : kEpilogueBytes + kParamBytes);
 };
 
 // kFusedSums (64x64 tile of the int8 kernel only): the kernel also forms the
@@ -473,30 +477,21 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // ---- what the write-back needs per destination row ----
-  // 32x32 blocks: after the transposition (below) a lane owns 16 consecutive
-  // rows of one column at a time, the same rows for every column it writes:
-  // everything that depends only on the row is gathered once, when the
-  // write-back starts. Rows past the end are clamped to the last row (their
-  // results are never stored) so that the loads carry no per-lane branches and
-  // can all be in flight together.
+  // ---- what the write-back needs per destination row and column ----
+  // Bias, zero-point sums and per-channel multipliers of the wave's rows and
+  // columns: each lane fetches those of two rows and two columns here, ahead
+  // of the main loop (loads only, nothing computed on them, so nobody waits),
+  // and the write-back hands them round through LDS. Fetched when the
+  // write-back starts instead, they cost it a round trip to memory or two
+  // (1.4 us of a 7 us kernel on a 1024 x 1024 x 196 per-channel product).
+  // Rows and columns past the end are clamped to the last one (their results
+  // are never stored).
   constexpr int kChunksPerCol = WM * 32 / 16;
   const Epilogue& ep = args.ep;
-  typename Traits::RowState rows;
-  auto load_row_state = [&]() {
-    const int first_row = m0 + wave_m * (WM * 32) + (lane % kChunksPerCol) * 16;
-    int row_idx[16];
-#pragma unroll
-    for (int q = 0; q < 16; ++q) row_idx[q] = min(first_row + q, args.M - 1);
-    rows.Load(ep, row_idx);
-  };
-  // 16x16 blocks: each lane fetches the parameters of two of the wave's rows
-  // and two of its columns here, ahead of the main loop (loads only); the
-  // write-back hands them round through LDS.
   typename Traits::EdgeParams edge;
-  if constexpr (kB == 16) {
+  {
     const int row = m0 + wave_m * (WM * 32) + lane;
-    const int col = n0 + wave_n * (WN * 32) + lane;
+    const int col = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * (C::kLogicalWN * 32) + lane;
     const int row_idx[2] = {min(row, args.M - 1), min(row + 64, args.M - 1)};
     const int col_idx[2] = {min(col, args.n_logical - 1), min(col + 64, args.n_logical - 1)};
     Traits::LoadEdgeParams(ep, row_idx, col_idx, edge);
@@ -1171,7 +1166,15 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int64_t ldd = args.dst.cs;
   const int chunk = lane % kChunksPerCol;
   const int i0 = m0 + wave_m * kRows + chunk * 16;
-  load_row_state();
+  // The wave's parameter area: written and read by this wave only, and LDS
+  // operations of a wave complete in order. After the transposition (below) a
+  // lane owns 16 consecutive rows of one column at a time, the same rows for
+  // every column it writes: their parameters are read once, here.
+  static_assert(kDepthWaves ? 4 * 2 * 128 * BK >= C::kEpilogueBytes + C::kParamBytes : true, "");
+  int* const area = reinterpret_cast<int*>(lds + C::kEpilogueBytes) + wave * Traits::kParamInts;
+  Traits::Stage(ep, edge, area, lane);
+  typename Traits::RowState rows;
+  rows.Read(area, chunk * 16);
   const int64_t col_bytes = ldd * elt;  // from one destination column to the next
   const int j_first = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * C::kLogicalWN * 32 + lane / kChunksPerCol;
   char* const lane_out = dst_base + (int64_t(j_first) * ldd + i0) * elt;
@@ -1260,7 +1263,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         vals[4 * q + 2] = now.w[q][2];
         vals[4 * q + 3] = now.w[q][3];
       }
-      Traits::Finish(vals, rows, j, ep);
+      typename Traits::ColState column;
+      column.Read(area, half * kHalfCols + c);
+      Traits::Finish(vals, rows, column, ep);
       const bool full = i0 + 16 <= args.M;
       // This lane's address at the wave's first staged column, plus what the
       // pass adds (the same for every lane: scalar arithmetic).
