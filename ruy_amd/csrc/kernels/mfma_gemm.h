@@ -488,14 +488,18 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // are never stored).
   constexpr int kChunksPerCol = WM * 32 / 16;
   const Epilogue& ep = args.ep;
+  // (Issued right behind the first operand loads, which matter more. They are
+  // ordinary loads on the same counter as the direct-to-LDS loads: a wait that
+  // leaves the youngest N loads outstanding then waits for a few operand loads
+  // more than it meant to, never for fewer.)
   typename Traits::EdgeParams edge;
-  {
+  auto load_edge_params = [&]() {
     const int row = m0 + wave_m * (WM * 32) + lane;
     const int col = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * (C::kLogicalWN * 32) + lane;
     const int row_idx[2] = {min(row, args.M - 1), min(row + 64, args.M - 1)};
     const int col_idx[2] = {min(col, args.n_logical - 1), min(col + 64, args.n_logical - 1)};
     Traits::LoadEdgeParams(ep, row_idx, col_idx, edge);
-  }
+  };
 
   // ---- software pipeline ----
   // Fragments are double-buffered in registers: while the matrix instructions
@@ -652,6 +656,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     const int my_steps = k_tiles > depth_way ? (k_tiles - depth_way + kDepthWays - 1) / kDepthWays : 0;
     if (my_steps > 0) issue_step(depth_way, 0);
     if (my_steps > 1) issue_step(depth_way + kDepthWays, 1);
+    load_edge_params();
     Frags4 fr[2];
     for (int i = 0; i < my_steps; ++i) {
       if (i + 1 < my_steps)
@@ -768,6 +773,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
       for (int l = 0; l < C::kALoads; ++l) issue_one(st, l);
     }
+    load_edge_params();
     WaitVmcnt<C::kALoads + C::kBLoads>();
     __syncthreads();
 #pragma unroll
@@ -874,6 +880,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   } else {
 #pragma unroll
     for (int s = 0; s < C::kStages; ++s) issue(s);
+    load_edge_params();
     WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
     __syncthreads();
     Frags f[2];
