@@ -483,7 +483,14 @@ def bench_other_configs(ctx, args):
         dp = device_problem(problem)
         dp.run(ctx)
         kernel = ctx.last_kernel_name()
-        t = time_steps(lambda: dp.run(ctx), args.steps, args.warmup, ctx, settle=False, events_every=10)
+        # Settled like the headline workloads: a card that has idled through the
+        # previous configuration's CPU baseline needs some 50-100 ms of load before
+        # its clock is up, far more than --warmup calls of a few microseconds.
+        # These calls take microseconds: at least 400 of them are timed whatever
+        # --steps says (`calls_timed`), so that the time the first launch takes to
+        # reach an idle GPU does not weigh on the mean.
+        calls = max(args.steps, 400)
+        t = time_steps(lambda: dp.run(ctx), calls, args.warmup, ctx, settle=not args.no_settle, events_every=10)
         ops = float(problem.ops())
         fp = bound == "mfma-f32"
         peak = F32_MFMA_PEAK_TFLOPS if fp else INT8_MFMA_PEAK_TOPS
@@ -491,7 +498,8 @@ def bench_other_configs(ctx, args):
         # Back-to-back asynchronous calls: the events around the region see the
         # kernels (and, for a call of several launches, the gaps between them).
         achieved = ops / (t["region_ms"] * 1e-3) / 1e12
-        entry = {"config": name, "kernel": kernel, "us_per_step": t["step_s"] * 1e6,
+        entry = {"config": name, "kernel": kernel, "settle_ms": t["settle_ms"], "calls_timed": calls,
+                 "us_per_step": t["step_s"] * 1e6,
                  "us_per_step_min": t["step_min_s"] * 1e6, "us_per_step_median": t["step_median_s"] * 1e6,
                  unit: ops / t["step_s"] / 1e12,
                  "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": unit,
