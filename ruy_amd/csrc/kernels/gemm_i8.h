@@ -150,9 +150,27 @@ struct GemvI8Args {
   // (g * rotate_step) mod steps (odd strides between 3 and 17 measured within
   // 1 % of each other on the 16384^2 weights; 1 is 3 % slower).
   int32_t rotate_step = 7;
+  // Set by the launchers (GemvStreamsWide): the wide operand is too large to
+  // stay in the caches from one call to the next, so its loads carry the
+  // non-temporal hint (nothing is kept of a line that is read exactly once).
+  int32_t stream_wide = 0;
   Epilogue ep;
   DevMat dst;
 };
+
+// Whether the skinny kernels mark their loads of the wide operand
+// non-temporal. Every byte of it is read once per call, so the hint costs
+// nothing inside a call; what it gives up is finding the operand in the
+// 256 MB Infinity Cache on the next call. Measured on 16384 x 16384 int8
+// weights (256 MiB), one column: streaming through four such matrices in turn
+// 46.2 -> 41.1 us per call with the hint (5.8 -> 6.5 TB/s); the same matrix
+// again and again 37.7 -> 39.3 us. At 127 MiB the same matrix again and again
+// loses 7 %, at 31 MiB 25 %. Hence: from half the Infinity Cache upwards, where
+// an operand cannot stay resident next to anything else a caller touches.
+constexpr uint64_t kGemvStreamBytes = uint64_t(128) << 20;
+inline bool GemvStreamsWide(const GemvI8Args& args) {
+  return uint64_t(args.rows) * uint64_t(args.K) >= kGemvStreamBytes;
+}
 
 // Depth step of the skinny kernel that LaunchGemvI8 picks for this many
 // narrow vectors.

@@ -33,6 +33,11 @@ __device__ __forceinline__ v4f LoadF4(__amdgpu_buffer_rsrc_t rsrc, uint32_t off)
   const v4i raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
   return __builtin_bit_cast(v4f, raw);
 }
+// The same with the non-temporal hint (cache-policy operand 2).
+__device__ __forceinline__ v4f LoadF4Nt(__amdgpu_buffer_rsrc_t rsrc, uint32_t off) {
+  const v4i raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 2);
+  return __builtin_bit_cast(v4f, raw);
+}
 
 __device__ __forceinline__ float WaveSum(float v) {
 #pragma unroll
@@ -70,8 +75,13 @@ __global__ __launch_bounds__(64 * kWaves) void GemvF32Kernel(GemvI8Args args) {
 
   auto load_wide = [&](int k0, v4f (&w)[kRows]) {
     const bool in = k0 + lane * 16 < K;
+    if (args.stream_wide) {  // wave-uniform: a wide operand too large to stay cached between calls
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) w[r] = LoadF4(w_rsrc, in ? w_off[r] + k0 : kOutOfRange);
+      for (int r = 0; r < kRows; ++r) w[r] = LoadF4Nt(w_rsrc, in ? w_off[r] + k0 : kOutOfRange);
+    } else {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) w[r] = LoadF4(w_rsrc, in ? w_off[r] + k0 : kOutOfRange);
+    }
   };
   auto load_narrow = [&](int k0, v4f (&n)[NB]) {
     const bool in = k0 + lane * 16 < K;
@@ -135,7 +145,9 @@ void Launch(hipStream_t stream, const GemvI8Args& args) {
 
 }  // namespace
 
-hipError_t LaunchGemvF32(hipStream_t stream, const GemvI8Args& args) {
+hipError_t LaunchGemvF32(hipStream_t stream, const GemvI8Args& caller_args) {
+  GemvI8Args args = caller_args;
+  args.stream_wide = GemvStreamsWide(args);  // (K counts bytes here)
   if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
   // Two and more narrow vectors: the matrix-core streaming kernel.
   if (args.narrow_count >= 2) return LaunchGemvF32Mma(stream, args);

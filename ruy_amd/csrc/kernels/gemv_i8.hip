@@ -98,9 +98,16 @@ __global__ __launch_bounds__(64 * kWaves) void GemvI8Kernel(GemvI8Args args) {
   auto load_wide = [&](int k0, v4i (&w)[kRowsPerWave]) {
     const int kp = phys(k0);
     const bool in = kp + lane * 16 < K;
+    // (The cache-policy operand must be a constant: 2 = non-temporal.)
+    if (args.stream_wide) {  // wave-uniform
 #pragma unroll
-    for (int r = 0; r < kRowsPerWave; ++r)
-      w[r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, in ? w_off[r] + kp : kOutOfRange, 0, 0);
+      for (int r = 0; r < kRowsPerWave; ++r)
+        w[r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, in ? w_off[r] + kp : kOutOfRange, 0, 2);
+    } else {
+#pragma unroll
+      for (int r = 0; r < kRowsPerWave; ++r)
+        w[r] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, in ? w_off[r] + kp : kOutOfRange, 0, 0);
+    }
   };
   auto load_narrow = [&](int k0, v4i (&n)[NB]) {
     const int kp = phys(k0);
@@ -188,6 +195,17 @@ __device__ __forceinline__ void LoadToLds16(uint32_t lds_base, uint32_t voffset,
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
       "buffer_load_dwordx4 %1, %2, 0 offen lds"
+      :
+      : "s"(lds_base), "v"(voffset), "s"(rsrc)
+      : "memory");
+}
+
+// The same with the non-temporal hint (a wide operand that is streamed once).
+__device__ __forceinline__ void LoadToLds16Nt(uint32_t lds_base, uint32_t voffset, v4i rsrc) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, 0 offen nt lds"
       :
       : "s"(lds_base), "v"(voffset), "s"(rsrc)
       : "memory");
@@ -294,6 +312,7 @@ __global__ __launch_bounds__(64 * kSplit) void GemvMmaKernel(GemvI8Args args) {
   const v4i w_rsrc = RsrcWords(args.wide, args.wide_bytes);
   const v4i n_rsrc = RsrcWords(args.narrow, args.narrow_bytes);
   const int K = args.K;  // multiple of 16
+  const bool stream_wide = args.stream_wide != 0;  // wave-uniform
   const int row0 = blockIdx.x * kMmaRows;
   constexpr int kZeroSlot = kRing * kStage;
   if (lane < 4) reinterpret_cast<int*>(lds + kZeroSlot)[lane] = 0;
@@ -320,7 +339,15 @@ __global__ __launch_bounds__(64 * kSplit) void GemvMmaKernel(GemvI8Args args) {
   auto issue = [&](int s, int ring_slot) {
     const int k0 = s * kStep;
     const uint32_t base = lds_base + ring_slot * kStage;
-    if (k0 + kStep <= K) {
+    if (k0 + kStep <= K && stream_wide) {
+#pragma unroll
+      for (int i = 0; i < kLoadsPerStage; ++i) {
+        if (i < kWideLoads)
+          LoadToLds16Nt(base + i * 1024, v_off[i] + k0, w_rsrc);
+        else
+          LoadToLds16(base + i * 1024, v_off[i] + k0, n_rsrc);
+      }
+    } else if (k0 + kStep <= K) {
 #pragma unroll
       for (int i = 0; i < kLoadsPerStage; ++i)
         LoadToLds16(base + i * 1024, v_off[i] + k0, i < kWideLoads ? w_rsrc : n_rsrc);
@@ -470,7 +497,9 @@ int MmaDepthSplit(const GemvI8Args& args) {
 
 int GemvI8DepthStep(int narrow_count) { return narrow_count == 1 ? 1024 : 512; }
 
-hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
+hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& caller_args) {
+  GemvI8Args args = caller_args;
+  args.stream_wide = GemvStreamsWide(args);
   if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
   // What the kernels assume: at most 16 narrow vectors, 16-byte granularity of
   // the depth, of both pitches and of both base addresses; whole depth steps
@@ -504,7 +533,9 @@ hipError_t LaunchGemvI8(hipStream_t stream, const GemvI8Args& args) {
 
 // fp32 with 2..16 narrow vectors: the same streaming kernel on
 // v_mfma_f32_16x16x4f32 (arguments byte-addressed, see GemvMmaKernel).
-hipError_t LaunchGemvF32Mma(hipStream_t stream, const GemvI8Args& args) {
+hipError_t LaunchGemvF32Mma(hipStream_t stream, const GemvI8Args& caller_args) {
+  GemvI8Args args = caller_args;
+  args.stream_wide = GemvStreamsWide(args);
   if (args.rows == 0 || args.narrow_count == 0) return hipSuccess;
   if (args.narrow_count > 16 || args.K % 16 != 0 || args.ld_wide % 16 != 0 || args.ld_narrow % 16 != 0 ||
       (reinterpret_cast<uintptr_t>(args.wide) | reinterpret_cast<uintptr_t>(args.narrow)) % 16 != 0)
