@@ -376,6 +376,31 @@ def test_full_size_int8_gemv_16384(device_ctx, cols, requant):
         device_ctx.set_cache_max_bytes(1 << 28)
 
 
+@pytest.mark.parametrize("tup", [(S.F32, S.F32, S.F32, S.F32), (S.U8, S.I8, S.I32, S.I16)], ids=cases.tuple_name)
+def test_skinny_wide_operands_read_as_a_stream(device_ctx, tup):
+    """Wide operands of 128 MiB and more, whose loads carry the non-temporal
+    hint in every skinny kernel: fp32 (one narrow vector: the dot-product
+    kernel; three and nine: the matrix-core kernel with 8 and 16 staged) and
+    8-bit with the wide side as the RHS (swapped roles), next to the int8 cases
+    of test_full_size_int8_gemv_16384. Depth-contiguous wide operands used in
+    place, every element against the checker."""
+    rng = np.random.default_rng(99 + tup[0])
+    wide, depth = (8192, 4096) if tup[0] == S.F32 else (16384, 8192)   # 128 MiB either way
+    for narrow in (1, 3, 9):
+        for swapped in (False, True):
+            if swapped:   # the wide side is the RHS: K x wide, column-major = depth-contiguous
+                p = W.random_problem(rng, *tup, narrow, depth, wide, S.ORDER_ROW_MAJOR, S.ORDER_COL_MAJOR,
+                                     S.ORDER_COL_MAJOR, strided=False,
+                                     name="%s %dx%dx%d" % (cases.tuple_name(tup), narrow, depth, wide))
+            else:
+                p = W.random_problem(rng, *tup, wide, depth, narrow, *cases.RCC, strided=False,
+                                     name="%s %dx%dx%d" % (cases.tuple_name(tup), wide, depth, narrow))
+            announce(p.name)
+            got, want = run_both(device_ctx, p)
+            compare(p, got, want)
+            assert device_ctx.last_kernel_name() == ("f32_gemv" if tup[0] == S.F32 else "i8_gemv")
+
+
 def test_prepacked_cache_through_mul(device_ctx):
     """Cache behaviour seen through Mul: policies (ruy/prepare_packed_matrices.cc
     :38-66 with a kernel width of 8), byte accounting, distinct keys per source
