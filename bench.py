@@ -32,7 +32,9 @@ One JSON line is printed:
               back to the C restatement ("port") when that build is absent.
 
 Every entry of `other_configs` (and `gemv`) carries its own roofline and
-cpu_baseline objects.
+cpu_baseline objects. The calls of `other_configs` take microseconds: each is
+measured after its own settling period and over at least 400 calls
+(`calls_timed`), whatever --steps says.
 """
 import argparse
 import ctypes as C
