@@ -878,17 +878,13 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     }
     if (kt < k_tiles) paired_step(kt, Odd(), std::false_type(), std::false_type());
   } else {
-#pragma unroll
-    for (int s = 0; s < C::kStages; ++s) issue(s);
-    load_edge_params();
-    WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
-    __syncthreads();
     Frags f[2];
-    read_frags(0, 0, f[0]);
     // The fragments of consecutive sub-steps alternate between f[0] and f[1].
     // `parity`: which of the two the step's first sub-step finds its fragments
     // in (always 0 when a ring step has an even number of sub-steps).
-    auto ring_step = [&](int kt, auto dma_is_full_step, auto parity) {
+    // `refill`: the slot of step kt is refilled with step kt + kStages (false:
+    // the whole depth was in the ring from the start, see below).
+    auto ring_step = [&](int kt, auto dma_is_full_step, auto parity, auto refill) {
       constexpr int kParity = decltype(parity)::value;
 #pragma unroll
       for (int ks = 0; ks < C::kKSteps; ++ks) {
@@ -896,15 +892,39 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         Frags& next = f[(kParity + ks + 1) & 1];
         if (ks + 1 < C::kKSteps) {
           sub_step(cur, next, kt, ks + 1, -1, dma_is_full_step);
-        } else {
+        } else if constexpr (decltype(refill)::value) {
           WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
           __syncthreads();
           sub_step(cur, next, kt + 1, 0, kt + C::kStages, dma_is_full_step);
+        } else {
+          sub_step(cur, next, kt + 1, 0, -1, dma_is_full_step);
         }
       }
     };
     using Even = std::integral_constant<int, 0>;
     using Odd = std::integral_constant<int, 1>;
+    if (C::kKSteps % 2 == 0 && k_tiles <= C::kStages) {
+      // A depth that fits the ring as a whole (256 bytes on the 64x64 tile's
+      // four stages, say): only the steps that exist are fetched, everything is
+      // awaited once, and the loop carries neither loads nor waits nor
+      // barriers. (The general form below fetches kStages steps past the end
+      // of every depth, as zeros, to keep its load counts fixed: nothing for a
+      // long depth, a third of the kernel's loads for this one.)
+#pragma unroll
+      for (int s = 0; s < C::kStages; ++s)
+        if (s < k_tiles) issue(s);
+      WaitVmcnt<0>();
+      __syncthreads();
+      load_edge_params();
+      read_frags(0, 0, f[0]);
+      for (int kt = 0; kt < k_tiles; ++kt) ring_step(kt, std::false_type(), Even(), std::false_type());
+    } else {
+#pragma unroll
+    for (int s = 0; s < C::kStages; ++s) issue(s);
+    load_edge_params();
+    WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
+    __syncthreads();
+    read_frags(0, 0, f[0]);
     // While the step whose loads are being issued (kt + kStages) lies entirely
     // inside the depth, the cheap form of the loads is used; the last few steps
     // (a partial step and the ones past the end, which fetch zeros) take the
@@ -912,20 +932,21 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     int kt = 0;
     const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
     if constexpr (C::kKSteps % 2 == 0) {
-      for (; kt < full_end; ++kt) ring_step(kt, std::true_type(), Even());
-      for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type(), Even());
+      for (; kt < full_end; ++kt) ring_step(kt, std::true_type(), Even(), std::true_type());
+      for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type(), Even(), std::true_type());
     } else {
       // One sub-step per ring step: the steps are taken in pairs, so that each
       // finds its fragments in a buffer known at compile time.
       for (; kt + 1 < full_end; kt += 2) {
-        ring_step(kt, std::true_type(), Even());
-        ring_step(kt + 1, std::true_type(), Odd());
+        ring_step(kt, std::true_type(), Even(), std::true_type());
+        ring_step(kt + 1, std::true_type(), Odd(), std::true_type());
       }
       for (; kt + 1 < k_tiles; kt += 2) {
-        ring_step(kt, std::false_type(), Even());
-        ring_step(kt + 1, std::false_type(), Odd());
+        ring_step(kt, std::false_type(), Even(), std::true_type());
+        ring_step(kt + 1, std::false_type(), Odd(), std::true_type());
       }
-      if (kt < k_tiles) ring_step(kt, std::false_type(), Even());
+      if (kt < k_tiles) ring_step(kt, std::false_type(), Even(), std::true_type());
+    }
     }
   }
   Traits::DrainMma();  // (matrix instructions the compiler does not see: let the last ones finish)
