@@ -30,9 +30,6 @@ struct F32Traits {
   using LargeTile = F32Traits;
   static constexpr bool kSplitB = false;
   static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kF32;
-  // Time between two dependent launches (about 5 us) in depth steps of the
-  // 256x256 tile (32 floats deep, 7.8 us each).
-  static constexpr double kLaunchGapInDepthSteps = 0.65;
   static __device__ __forceinline__ int Bits(float x, float) { return __float_as_int(x); }
   static __device__ __forceinline__ int RawBits(float x) { return __float_as_int(x); }
   static __device__ __forceinline__ float FromRawBits(int w) { return __int_as_float(w); }

@@ -34,12 +34,15 @@ struct GemmArgs {
   int32_t n_logical = 0;
   Epilogue ep;
   // The destination must be column-major (dst.rs == 1): callers swap the
-  // operands for a row-major one. dst_elt is its element size; dst_vector_ok
-  // says that base and column pitch are 16-byte aligned so that 16-byte stores
-  // may be used.
+  // operands for a row-major one. dst_elt is its element size. Base and
+  // column pitch may have any alignment the element type allows.
   DevMat dst;
   int32_t dst_elt = 1;
-  int32_t dst_vector_ok = 0;
+  // Keeps the fields below where the kernels were compiled without scratch
+  // memory: with one word less here, the struct has a hole in front of its
+  // last pointers and the compiler copies that part of the kernel arguments
+  // through scratch in some kernels.
+  int32_t unused_padding = 0;
   // int8 kernel, small problems only (GemmI8CanFuseSums): when fuse_sums is
   // set the kernel forms the depth sums of a's rows and b's columns itself
   // and subtracts fused_a_factor * rowsum(i) + fused_b_factor * colsum(j)

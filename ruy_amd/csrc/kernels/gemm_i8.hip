@@ -43,9 +43,6 @@ struct Int8Traits {
   using LargeTile = Int8Traits16;
   static constexpr bool kSplitB = false;
   static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kInt8;
-  // Time between two dependent launches (about 5 us) in depth steps of the
-  // 256x256 tile (1.9 us each on int8).
-  static constexpr double kLaunchGapInDepthSteps = 2.6;
   static __device__ __forceinline__ int Bits(int x, int) { return x; }
   static __device__ __forceinline__ int RawBits(int x) { return x; }
   static __device__ __forceinline__ int FromRawBits(int w) { return w; }

@@ -58,6 +58,11 @@ namespace ruyamd {
 namespace mfma_gemm {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+// The same 16 bytes at an address of any alignment. Global memory instructions
+// of every width take any byte address on this target (the compiler emits the
+// one 16-byte store either way), so a destination whose base or column pitch
+// is not a multiple of 16 bytes is still written 16 bytes a lane.
+typedef v4i v4i_unaligned __attribute__((aligned(1)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -313,10 +318,15 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   constexpr bool kCanSplitDepth = WM * WN <= 2 && kB == 32;
   const int split = kCanSplitDepth ? args.split_k : 1;
   const int split_index = kCanSplitDepth ? blockIdx.y : 0;
-  const int kt_first = depth_split::FirstStep(k_tiles_all, split, split_index);
-  const int k_tiles = depth_split::StepCount(k_tiles_all, split, split_index);
+  // Divisions run on the vector unit: their results are read back into scalar
+  // registers here, so that what derives from them (a load's scalar offset
+  // operand among others) is scalar whatever the compiler makes of the
+  // expressions.
+  const int kt_first = __builtin_amdgcn_readfirstlane(depth_split::FirstStep(k_tiles_all, split, split_index));
+  const int k_tiles = __builtin_amdgcn_readfirstlane(depth_split::StepCount(k_tiles_all, split, split_index));
   constexpr bool kRotateDepth = WM * WN < 16;
-  const int rot = kRotateDepth && K % kBK == 0 && k_tiles > 0 ? (tile_m * 5 + split_index * 3) % k_tiles : 0;
+  const int rot = __builtin_amdgcn_readfirstlane(
+      kRotateDepth && K % kBK == 0 && k_tiles > 0 ? (tile_m * 5 + split_index * 3) % k_tiles : 0);
   auto phys = [&](int kt) {
     if constexpr (!kRotateDepth) return kt;
     const int p = kt + rot;
@@ -1127,14 +1137,14 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         for (int p = 0; p < kElt; ++p) transpose(w[p]);
         if (j < args.n_logical && row0 < args.M) {
           char* out = dst_base + (int64_t(j) * ldd + row0) * kElt;
-          if (rows_full && args.dst_vector_ok) {
+          if (rows_full) {
             // Memory order: rows 4k .. 4k+3 are words w[0][k] .. w[kElt-1][k].
 #pragma unroll
             for (int x = 0; x < kElt; ++x) {
               v4i o;
 #pragma unroll
               for (int y = 0; y < 4; ++y) o[y] = w[(4 * x + y) % kElt][(4 * x + y) / kElt];
-              reinterpret_cast<v4i*>(out)[x] = o;
+              reinterpret_cast<v4i_unaligned*>(out)[x] = o;
             }
           } else {
 #pragma unroll
@@ -1298,14 +1308,14 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       // This lane's address at the wave's first staged column, plus what the
       // pass adds (the same for every lane: scalar arithmetic).
       char* out = lane_out + int64_t(half * kHalfCols + pass * kColsPerPass) * col_bytes;
-      if (full && args.dst_vector_ok) {
+      if (full) {
         if (elt == 1) {
           v4i w;
 #pragma unroll
           for (int q = 0; q < 4; ++q)
             w[q] = (vals[4 * q] & 0xff) | ((vals[4 * q + 1] & 0xff) << 8) |
                    ((vals[4 * q + 2] & 0xff) << 16) | (vals[4 * q + 3] << 24);
-          *reinterpret_cast<v4i*>(out) = w;
+          *reinterpret_cast<v4i_unaligned*>(out) = w;
         } else if (elt == 2) {
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
@@ -1313,7 +1323,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
             for (int q = 0; q < 4; ++q)
               w[q] = (vals[8 * h + 2 * q] & 0xffff) | (vals[8 * h + 2 * q + 1] << 16);
-            reinterpret_cast<v4i*>(out)[h] = w;
+            reinterpret_cast<v4i_unaligned*>(out)[h] = w;
           }
         } else {
 #pragma unroll
@@ -1321,7 +1331,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
             v4i w;
 #pragma unroll
             for (int q = 0; q < 4; ++q) w[q] = vals[4 * h + q];
-            reinterpret_cast<v4i*>(out)[h] = w;
+            reinterpret_cast<v4i_unaligned*>(out)[h] = w;
           }
         }
       } else {
@@ -1417,184 +1427,178 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
   return ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
 }
 
-enum class Tile { k256x256, k256x128, k128x256, k128x128, k128x64, k64x128, k64x64 };
+enum class Tile { k256x256, k128x128, k128x64, k64x128, k64x64 };
 
-// Picks the tile by a small cost model: workgroups are dealt to the CUs in
-// rounds, a round of a given tile costs its area divided by how well that tile
-// feeds the matrix cores (measured on int8: 256x128 sustains about 0.75, the
-// 128x128 tile about 0.65 and the 64x64 tile, whose waves read one LDS
-// fragment pair per matrix instruction, about 0.45 of the 256x256 tile's
-// rate). Large tiles win when there are many rounds, small tiles when the last
-// (or only) round would leave most CUs idle. Model::kInt8PlaneSplit: the plane-split form
-// of the int16 kernel, which has the two square large tiles and a 64x128 one.
+// Which tile a problem runs on is decided by a timing model of every tile, in
+// microseconds, fitted to measurements of every tile on 134 shapes for int8,
+// 96 for fp32 and 48 for int8 x int16 (destinations of 128^2 to 12288^2
+// elements, square, oblong and ragged, depths of 2 to 64 steps). The fit is
+// within 3-12 % root mean square of the measurements. Picking by it costs 1 %
+// of time over always picking the fastest tile on the shapes it was fitted to
+// and about 4 % (int8), 2 % (fp32) on shapes held out of the fit: among the
+// 128x128, 128x64 and 64x128 tiles the times are often closer than the model
+// is good.
 //
+// Workgroups are dealt to the CUs in rounds, and a workgroup costs its ring
+// fill and write-back (`overhead`, in depth steps) plus its depth steps:
+//
+//   time = fixed + rounds * (overhead + depth steps) * step  [+ reduce]
+//
+// With q * CUs + r tiles there are q full rounds, and a last one on r CUs costs
+// last_round + (1 - last_round) * r / CUs of a full one: less, since the few
+// workgroups run at a higher clock and have the memory system to themselves,
+// but far from nothing. `fixed` is what does not grow with the tile count
+// (launch, first fetch). The smallest tile splits the depth when its tiles
+// leave CUs idle (DepthSplitParts): the parts count as tiles of a shorter depth
+// and adding them up costs `reduce`.
+//
+// The 128x128, 128x64 and 64x128 tiles run with two-stage rings when there are
+// more tiles than CUs (ShallowRing), and a CU then holds up to `occupancy` of
+// their workgroups side by side. A CU with n tiles runs them in groups of that
+// many; a group of j costs (overhead + depth steps) * shared_step[j - 1] (two
+// side by side cost less than twice one: they fill each other's waits), and
+// the r CUs that have one tile more than the others add the difference,
+// discounted as above with `shared_last_round`.
+//
+// What the fit says about the kernels: on int8 the 256x256 tile's depth step
+// (1.37 us) is a quarter of what the 64x64 tile needs for the same area (16 x
+// 0.200 us) and 60 % of the 128x128 tile's (4 x 1.08 us / 2 side by side), so it
+// wins whenever its tiles fill most of a round; fp32 is bound by its matrix
+// instructions at every tile size (7.85 us against 16 x 0.562 us) and the small
+// tiles, which fill the CUs more evenly, win up to destinations of 4096^2.
+// Tiles of 256x128 and 128x256 were built too, were the fastest at no shape
+// measured, and are not kept; neither is a second launch on a smaller tile for
+// the part of a 256x256 grid that does not fill its last round, which lost to
+// the single launch at every shape once that tile ran on 16x16 blocks.
+struct TileTiming {
+  Tile tile;
+  int bm, bn;
+  double fixed, overhead, step, last_round;
+  int occupancy;
+  double shared_step[3];
+  double shared_last_round;
+};
+enum class Model { kInt8, kInt8PlaneSplit, kF32 };
+struct TimingModel {
+  const TileTiming* tiles;
+  int count;
+  Tile smallest;           // the tile that has the depth split
+  int min_steps_per_part;  // of that split
+  double reduce;           // microseconds to add up the parts of a split
+};
+constexpr TileTiming kInt8Timings[] = {
+    {Tile::k256x256, 256, 256, 4.58, 7.20, 1.370, 0.68, 1, {}, 0},
+    {Tile::k128x128, 128, 128, 3.74, 4.36, 0.638, 0.74, 2, {0.755, 1.082}, 0.585},
+    {Tile::k128x64, 128, 64, 3.53, 4.21, 0.358, 0.87, 3, {0.257, 0.625, 1.073}, 0.78},
+    {Tile::k64x128, 64, 128, 4.43, 1.86, 0.354, 0.86, 3, {0.182, 0.777, 1.415}, 0.56},
+    {Tile::k64x64, 64, 64, 1.87, 13.6, 0.200, 0.93, 1, {}, 0},
+};
+constexpr TileTiming kF32Timings[] = {
+    {Tile::k256x256, 256, 256, 0.0, 2.21, 7.854, 0.88, 1, {}, 0},
+    {Tile::k128x128, 128, 128, 1.45, 3.02, 2.153, 0.85, 2, {1.751, 3.656}, 1.0},
+    {Tile::k128x64, 128, 64, 2.74, 2.74, 1.190, 0.83, 3, {1.037, 1.980, 2.722}, 0.91},
+    {Tile::k64x128, 64, 128, 3.03, 2.54, 1.152, 0.84, 3, {1.114, 1.977, 2.757}, 0.84},
+    {Tile::k64x64, 64, 64, 1.75, 6.46, 0.562, 0.86, 1, {}, 0},
+};
+// The plane-split form of the int16 kernel has the two square large tiles and
+// one of 64 rows x 128 plane columns (64 destination columns); `bn` counts
+// plane columns, as GemmArgs::N does there. `fixed` includes the launch that
+// splits the int16 operand, which the smallest tile does without.
+constexpr TileTiming kInt8PlaneSplitTimings[] = {
+    {Tile::k256x256, 256, 256, 10.7, 4.14, 2.00, 0.56, 1, {}, 0},
+    {Tile::k128x128, 128, 128, 8.48, 4.32, 0.727, 0.67, 1, {}, 0},
+    {Tile::k64x128, 64, 128, 2.08, 6.38, 0.504, 0.86, 1, {}, 0},
+};
+inline TimingModel TimingModelOf(Model model) {
+  switch (model) {
+    case Model::kF32:
+      return {kF32Timings, 5, Tile::k64x64, 16, 3.1};
+    case Model::kInt8PlaneSplit:
+      return {kInt8PlaneSplitTimings, 3, Tile::k64x128, 8, 3.6};
+    default:
+      return {kInt8Timings, 5, Tile::k64x64, 16, 2.1};
+  }
+}
+
+// Parts of the smallest tile's depth split: taken when the tiles alone leave
+// CUs idle, aims at one workgroup per CU (the rings take most of a CU's LDS),
+// and keeps at least `min_steps_per_part` depth steps in every part (16 for
+// the 64x64 tile: four steps for each of its waves) so that filling the ring
+// and adding up the parts stay small against the work shared out. One
+// workgroup streams operands that are not in L2 at 80-100 GB/s at best (what
+// its ring keeps in flight over a round trip to memory), so a problem with few
+// tiles and a long depth only gets faster by putting more workgroups on it.
+// Only the smallest tile has the split: adding up the parts costs time in
+// proportion to the tile's area, and with larger tiles that outweighed the
+// gain at every shape measured.
+inline int DepthSplitParts(int tiles, int k_steps, int num_cus, int min_steps_per_part) {
+  constexpr int kMaxParts = 32;
+  if (tiles <= 0 || tiles > kSplitCounters) return 1;
+  const int parts = std::min({num_cus / tiles, k_steps / min_steps_per_part, kMaxParts});
+  if (parts < 2) return 1;
+  return depth_split::PartsWithoutEmpty(k_steps, parts);
+}
+
+inline double ModelledMicroseconds(const GemmArgs& args, int num_cus, const TimingModel& model, const TileTiming& t) {
+  int tiles = TileCount(args, t.bm, t.bn);
+  int k_steps = std::max(1, (args.k_bytes + 127) / 128);
+  int parts = 1;
+  if (t.tile == model.smallest) {
+    parts = DepthSplitParts(tiles, k_steps, num_cus, model.min_steps_per_part);
+    tiles *= parts;
+    k_steps = depth_split::StepsPerPart(k_steps, parts);
+  }
+  const int q = tiles / num_cus, r = tiles % num_cus;
+  const double fraction = double(r) / num_cus;
+  double rounds;  // in units of one workgroup's (overhead + depth steps)
+  if (t.occupancy == 1 || tiles <= num_cus) {
+    rounds = (q + (r ? t.last_round + (1 - t.last_round) * fraction : 0.0)) * t.step;
+  } else {
+    auto cu_with = [&](int n) {
+      const int rest = n % t.occupancy;
+      return (n / t.occupancy) * t.shared_step[t.occupancy - 1] + (rest ? t.shared_step[rest - 1] : 0.0);
+    };
+    rounds = cu_with(q);
+    if (r) rounds += (cu_with(q + 1) - cu_with(q)) * (t.shared_last_round + (1 - t.shared_last_round) * fraction);
+  }
+  return t.fixed + rounds * (t.overhead + k_steps) + (parts > 1 ? model.reduce : 0.0);
+}
+
 // The 128x128, 128x64 and 64x128 tiles come with two ring depths. Four stages
 // when every tile has a CU to itself (a lone workgroup needs the deep prefetch:
 // 1280x1280 with K = 4096 runs in 24 us on 128x64 with four stages, 28 us with
 // two). Two stages when there are more tiles than CUs: two (three) workgroups
 // then fit a CU's LDS together, and a second wave on each SIMD fills the issue
 // slots and barrier waits of the first (4096x4096 with K = 2048 on 128x128:
-// 81 -> 58 us; 2560^3: 45 -> 34 us). The cost model knows the case of up to
-// two tiles per CU, where both run side by side as one shared round with a
-// measured efficiency of 0.85 (128x128) and 0.65 (128x64, 64x128); with more
-// tiles than that the large tiles win anyway and the rounds are counted as
-// before.
-//
-// fp32 is bound by its matrix instructions at every tile size (64 cycles of
-// matrix pipe per 32 bytes of fragment pair, eight times the int8 ratio), so
-// the small tiles lose little there and filling the CUs evenly matters more:
-// measured against the 256x256 tile, 256x128, 128x128 and 128x64 sustain
-// about 0.85 (0.9 in a shared round) and 64x64 0.75, which moves e.g.
-// 3072^3 from 256x256 (144 tiles, 723 us) to 128x64 (556 us) and 1536^3 from
-// 128x128 to 64x64 (114 -> 97 us).
-enum class Model { kInt8, kInt8PlaneSplit, kF32 };
-struct Efficiencies {
-  double t256x128, t128x128, t128x128_shared, t128x64, t128x64_shared, t64x64;
-};
-constexpr Efficiencies kInt8Efficiencies = {0.75, 0.65, 0.85, 0.55, 0.65, 0.45};
-constexpr Efficiencies kF32Efficiencies = {0.85, 0.85, 0.9, 0.85, 0.9, 0.75};
-struct TileChoice {
-  Tile tile;
-  double cost;  // rounds x tile area / efficiency
-};
+// 81 -> 58 us; 2560^3: 45 -> 34 us).
 inline bool ShallowRing(const GemmArgs& args, int num_cus, int bm, int bn) {
   return TileCount(args, bm, bn) > num_cus;
 }
-inline TileChoice BestTile(const GemmArgs& args, int num_cus, Model model) {
-  const bool split_b = model == Model::kInt8PlaneSplit;
-  const Efficiencies& eff = model == Model::kF32 ? kF32Efficiencies : kInt8Efficiencies;
-  auto cost = [&](int bm, int bn, double efficiency, double efficiency_shared = 0) {
-    const int tiles = TileCount(args, bm, bn);
-    if (efficiency_shared > 0 && tiles > num_cus && tiles <= 2 * num_cus)
-      return 2 * double(bm) * double(bn) / efficiency_shared;
-    const int rounds = (tiles + num_cus - 1) / num_cus;
-    return rounds * double(bm) * double(bn) / efficiency;
-  };
-  const double c256 = cost(256, 256, 1.0);
-  if (split_b) {
-    // Plane-split operand: the smallest tile is 64 rows x 128 plane columns (64 destination columns).
-    const double c128 = cost(128, 128, 0.65);
-    const double c64x128 = cost(64, 128, 0.5);
-    if (c256 <= c128 && c256 <= c64x128) return {Tile::k256x256, c256};
-    return c128 <= c64x128 ? TileChoice{Tile::k128x128, c128} : TileChoice{Tile::k64x128, c64x128};
-  }
-  const double c128 = cost(128, 128, eff.t128x128, eff.t128x128_shared);
-  const double c64 = cost(64, 64, eff.t64x64);
-  const double c256x128 = cost(256, 128, eff.t256x128);
-  const double c128x256 = cost(128, 256, eff.t256x128);
-  const double c128x64 = cost(128, 64, eff.t128x64, eff.t128x64_shared);
-  const double c64x128 = cost(64, 128, eff.t128x64, eff.t128x64_shared);
-  const double best = std::min({c256, c128, c64, c256x128, c128x256, c128x64, c64x128});
-  if (c256 == best) return {Tile::k256x256, best};
-  if (c256x128 == best) return {Tile::k256x128, best};
-  if (c128x256 == best) return {Tile::k128x256, best};
-  if (c128 == best) return {Tile::k128x128, best};
-  if (c128x64 == best) return {Tile::k128x64, best};
-  if (c64x128 == best) return {Tile::k64x128, best};
-  return {Tile::k64x64, best};
-}
-inline Tile PickTile(const GemmArgs& args, int num_cus, Model model) {
-  return BestTile(args, num_cus, model).tile;
-}
 
-// The sub-problem of `args` whose destination is rows [m_begin, m_begin +
-// m_count) x columns [n_begin, n_begin + n_count) of the original one: operand,
-// destination and per-row / per-column parameter pointers advanced, nothing
-// else changed. Not for the plane-split operand.
-inline GemmArgs SubProblem(const GemmArgs& args, int m_begin, int m_count, int n_begin, int n_count) {
-  GemmArgs sub = args;
-  const uint32_t a_skip = uint32_t(m_begin) * uint32_t(args.lda);
-  const uint32_t b_skip = uint32_t(n_begin) * uint32_t(args.ldb);
-  sub.a = static_cast<const char*>(args.a) + a_skip;
-  sub.b = static_cast<const char*>(args.b) + b_skip;
-  sub.a_bytes = args.a_bytes > a_skip ? args.a_bytes - a_skip : 0;
-  sub.b_bytes = args.b_bytes > b_skip ? args.b_bytes - b_skip : 0;
-  sub.M = m_count;
-  sub.N = n_count;
-  sub.n_logical = n_count;
-  sub.dst.rows = m_count;
-  sub.dst.cols = n_count;
-  sub.dst.data = static_cast<char*>(args.dst.data) +
-                 (int64_t(m_begin) * args.dst.rs + int64_t(n_begin) * args.dst.cs) * args.dst_elt;
-  sub.dst_vector_ok = (reinterpret_cast<uintptr_t>(sub.dst.data) & 15) == 0 && (args.dst.cs * args.dst_elt) % 16 == 0;
-  if (args.ep.lhs_sums) sub.ep.lhs_sums = args.ep.lhs_sums + m_begin;
-  if (args.ep.rhs_sums) sub.ep.rhs_sums = args.ep.rhs_sums + n_begin;
-  const int channel_begin = args.ep.channel_is_col ? n_begin : m_begin;
-  if (args.ep.bias) sub.ep.bias = static_cast<const char*>(args.ep.bias) + int64_t(channel_begin) * 4;  // int32 or fp32
-  if (args.ep.mult_fixedpoint) sub.ep.mult_fixedpoint = args.ep.mult_fixedpoint + channel_begin;
-  if (args.ep.mult_exponent) sub.ep.mult_exponent = args.ep.mult_exponent + channel_begin;
-  return sub;
-}
-
-// A grid of 256x256 tiles whose last round of workgroups would leave most CUs
-// idle (576 tiles on 256 CUs: three rounds for 2.25 rounds of work) is cut in
-// two launches: whole tile columns (or rows) that fill their rounds, and the
-// rest of the destination on whichever tile suits that strip best. The second
-// launch starts when the first has drained, which costs a few microseconds,
-// expressed here in depth steps of the large tile (`gap_steps`). The model
-// overstates the gain (a last round on a quarter of the CUs runs at a higher
-// clock than a full one; measured gains were about a third of the modelled
-// ones), so the cut is taken only for grids of at least 8 x 8 tiles and a
-// modelled saving of 12 % or more: 4608^3 135 -> 127 us, 7168^3 420 -> 396 us.
-struct TailPlan {
-  bool use = false;
-  bool along_n = false;  // the cut runs between tile columns (else between tile rows)
-  int main_tiles = 0;    // tile columns (rows) in the first launch
-};
-inline TailPlan PlanTail(const GemmArgs& args, int num_cus, double gap_steps, Model model) {
-  TailPlan plan;
-  const int tiles_m = (args.M + 255) / 256, tiles_n = (args.N + 255) / 256;
-  const int total = tiles_m * tiles_n;
-  if (total <= num_cus || total % num_cus == 0 || tiles_m < 8 || tiles_n < 8) return plan;
-  const double round_cost = 256.0 * 256.0;
-  const double single = double((total + num_cus - 1) / num_cus) * round_cost;
-  const int k_steps = std::max(1, (args.k_bytes + 127) / 128);
-  const double gap = gap_steps * round_cost / k_steps;
-  double best = single * 0.88;
-  for (int along_n = 0; along_n < 2; ++along_n) {
-    const int across = along_n ? tiles_m : tiles_n;  // tiles per column (row) of tiles
-    const int count = along_n ? tiles_n : tiles_m;
-    for (int c = 1; c < count; ++c) {
-      const int main_rounds = (across * c + num_cus - 1) / num_cus;
-      GemmArgs tail = args;
-      (along_n ? tail.N : tail.M) -= c * 256;
-      const double cost = main_rounds * round_cost + BestTile(tail, num_cus, model).cost + gap;
-      if (cost < best) {
-        best = cost;
-        plan.use = true;
-        plan.along_n = along_n != 0;
-        plan.main_tiles = c;
-      }
+inline Tile PickTile(const GemmArgs& args, int num_cus, Model which) {
+  const TimingModel model = TimingModelOf(which);
+  Tile best = model.tiles[0].tile;
+  double best_time = ModelledMicroseconds(args, num_cus, model, model.tiles[0]);
+  for (int i = 1; i < model.count; ++i) {
+    const double time = ModelledMicroseconds(args, num_cus, model, model.tiles[i]);
+    if (time < best_time) {
+      best_time = time;
+      best = model.tiles[i].tile;
     }
   }
-  return plan;
+  return best;
 }
 
-// Depth split for a launch of `args` (see GemmArgs::split_k). Only the
-// smallest tile has it (64x64, or 64 rows x 128 plane columns for the
-// plane-split operand): adding up the parts costs time in proportion to the
-// tile's area, and with larger tiles that outweighed the gain at every shape
-// measured. One workgroup streams operands that are not in L2 at 80-100 GB/s
-// at best (what its ring keeps in flight over a round trip to memory), so a
-// problem with few tiles and a long depth only gets faster by putting more
-// workgroups on it. The split is taken when the tiles alone leave CUs idle,
-// aims at one workgroup per CU (the rings take most of a CU's LDS), and keeps
-// at least kMinStepsPerPart depth steps in every part (16 for the 64x64 tile:
-// four steps for each of its waves) so that filling the ring and adding up the
-// parts stay small against the work shared out.
-inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, Model model) {
-  const bool split_b = model == Model::kInt8PlaneSplit;
-  const int kMinStepsPerPart = split_b ? 8 : 16;
-  constexpr int kMaxParts = 32;
-  const Tile tile = PickTile(args, num_cus, model);
-  if (tile != (split_b ? Tile::k64x128 : Tile::k64x64)) return DepthSplit();
+// Depth split for a launch of `args` (see GemmArgs::split_k and DepthSplitParts).
+inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, Model which) {
+  const TimingModel model = TimingModelOf(which);
+  if (PickTile(args, num_cus, which) != model.smallest) return DepthSplit();
+  const bool split_b = which == Model::kInt8PlaneSplit;
   const int bm = 64, bn = split_b ? 128 : 64;
   const int tiles = TileCount(args, bm, bn);
   const int k_tiles = (args.k_bytes + 127) / 128;
-  if (tiles == 0 || tiles > kSplitCounters) return DepthSplit();
-  int parts = std::min({num_cus / tiles, k_tiles / kMinStepsPerPart, kMaxParts});
+  const int parts = DepthSplitParts(tiles, k_tiles, num_cus, model.min_steps_per_part);
   if (parts < 2) return DepthSplit();
-  parts = depth_split::PartsWithoutEmpty(k_tiles, parts);
   DepthSplit split;
   split.parts = parts;
   split.partial_bytes = size_t(parts) * tiles * bm * bn * 4;
@@ -1643,10 +1647,6 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
   }
   if constexpr (!Traits::kSplitB) {
     switch (tile) {
-      case Tile::k256x128:
-        return Launch<Traits, 4, 2, 128, 3>(stream, args);
-      case Tile::k128x256:
-        return Launch<Traits, 2, 4, 128, 3>(stream, args);
       case Tile::k128x64:
         if (ShallowRing(args, num_cus, 128, 64)) return Launch<Traits, 2, 1, 128, 2>(stream, args);
         return Launch<Traits, 2, 1, 128, 4>(stream, args);
@@ -1659,22 +1659,7 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
 
 template <typename Traits>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
-  const Tile tile = PickTile(args, num_cus, Traits::kModel);
-  if constexpr (!Traits::kSplitB) {
-    if (tile == Tile::k256x256 && args.split_k == 1 && !args.fuse_sums) {
-      const TailPlan plan = PlanTail(args, num_cus, Traits::kLaunchGapInDepthSteps, Traits::kModel);
-      if (plan.use) {
-        const int cut = plan.main_tiles * 256;
-        const GemmArgs main = plan.along_n ? SubProblem(args, 0, args.M, 0, cut) : SubProblem(args, 0, cut, 0, args.N);
-        const GemmArgs tail = plan.along_n ? SubProblem(args, 0, args.M, cut, args.N - cut)
-                                           : SubProblem(args, cut, args.M - cut, 0, args.N);
-        const hipError_t first = Launch<typename Traits::LargeTile, 4, 4, 128, 2>(stream, main);
-        if (first != hipSuccess) return first;
-        return LaunchTile<Traits>(stream, tail, PickTile(tail, num_cus, Traits::kModel), num_cus);
-      }
-    }
-  }
-  return LaunchTile<Traits>(stream, args, tile, num_cus);
+  return LaunchTile<Traits>(stream, args, PickTile(args, num_cus, Traits::kModel), num_cus);
 }
 
 }  // namespace mfma_gemm

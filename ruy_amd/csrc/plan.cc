@@ -532,8 +532,6 @@ bool SetupDestination(const MulCall& call, GemmArgs* args) {
     args->dst.cs = dst.rs;
   }
   args->dst_elt = DtypeSize(dst.dtype);
-  args->dst_vector_ok = (reinterpret_cast<uintptr_t>(args->dst.data) & 15) == 0 &&
-                        (args->dst.cs * args->dst_elt) % 16 == 0;
   return swap;
 }
 
@@ -790,9 +788,6 @@ int RunMulBatch(ruyamd_ctx* ctx, const MulCall& first, const BatchBuffers* items
   GemmArgs args;
   const bool swap = SetupInt8Gemm(ctx, first, a, b, lzp, rzp, &args);
   if ((a.sums_pending || b.sums_pending) && !args.fuse_sums) return RUYAMD_OK;
-  // 16-byte stores need every product's destination aligned, not only the first one's.
-  for (int z = 0; z < n; ++z)
-    if (reinterpret_cast<uintptr_t>(items[z].dst) & 15) args.dst_vector_ok = 0;
   const bool timed = ctx->TimingBegin();
   hipError_t launched = hipSuccess;
   for (int z0 = 0; z0 < n && launched == hipSuccess; z0 += kGemmBatchMax) {

@@ -859,17 +859,20 @@ def test_largest_tile_over_depth_step_counts(device_ctx, tup):
     steps: depths of one to seven steps, whole and partial last steps, depths
     that are not a multiple of 16 (packed operands), ragged destination edges,
     per-channel parameters and zero points as the random problem draws them,
-    all three destination widths. Every element where the stock reference
+    all three destination widths, destinations whose column pitch or base
+    address is odd (the 16-byte stores then go to unaligned addresses). Every
+    element where the stock reference
     library is built (see test_full_size_int8_gemm_8192), a sample of rows and
     columns either side of every tile edge otherwise and in any case."""
     import device_runner as D
     rng = np.random.default_rng(4242 + tup[3])
-    for K, M, N in [(16, 4096, 4096), (112, 4096, 4096), (128, 4000, 4090), (144, 4096, 4096), (256, 4096, 3900),
-                    (300, 4096, 4096), (384, 4096, 4096), (500, 3850, 4096), (640, 4096, 4096), (896, 4096, 4096)]:
+    for K, M, N, misalign in [(16, 4096, 4096, 0), (112, 4096, 4096, 0), (128, 4000, 4090, 0), (144, 4096, 4096, 0),
+                              (256, 4096, 3900, 0), (300, 4096, 4096, 0), (384, 4096, 4096, 0), (500, 3850, 4096, 0),
+                              (640, 4096, 4096, 0), (896, 4096, 4096, 0), (256, 3001, 4096, 3), (128, 4095, 3003, 1)]:
         p = W.random_problem(rng, *tup, M, K, N, *cases.RCC, strided=False,
-                             name="%s %s" % (cases.tuple_name(tup), (M, K, N)))
+                             name="%s %s +%d" % (cases.tuple_name(tup), (M, K, N), misalign))
         announce(p.name)
-        got = D.device_mul(device_ctx, p, dst_fill=0)
+        got = D.device_mul(device_ctx, p, dst_fill=0, misalign=misalign)
         assert device_ctx.last_kernel_name() == "i8_mfma"
         rows, cols = _boundary_sample(rng, M), _boundary_sample(rng, N)
         g, w = _sample_block(p, got, rows, cols)
@@ -884,10 +887,11 @@ def test_largest_tile_over_depth_step_counts(device_ctx, tup):
                                  (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
 def test_base_addresses_that_are_not_aligned(device_ctx, tup):
     """Every buffer (operands, destination, bias, multipliers) starts 1 or 3
-    elements into its allocation: the kernels that read operands in place and
-    store 16 bytes at a time need aligned addresses, so these calls take the
-    packed route and the element-wise stores, on the tiled, the skinny and the
-    one-column kernels. The guard zones around the destination stay intact."""
+    elements into its allocation: the kernels that read operands in place
+    need aligned addresses, so these calls take the packed route, and the tiled
+    kernels' 16-byte stores go to unaligned addresses; on the tiled, the skinny
+    and the one-column kernels. The guard zones around the destination stay
+    intact."""
     import device_runner as D
     rng = np.random.default_rng(31337)
     for shape in [(200, 256, 300), (300, 1024, 7), (9, 512, 400), (500, 2048, 1), (64, 4096, 64), (130, 130, 130)]:
