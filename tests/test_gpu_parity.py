@@ -807,15 +807,13 @@ def _boundary_sample(rng, n, step=256, random_count=40):
                                        ((7000, 4096, 3000), (S.I8, S.U8, S.I32, S.U8)),
                                        ((4608, 1024, 4608), (S.F32, S.F32, S.F32, S.F32))],
                          ids=lambda v: "x".join(map(str, v)) if isinstance(v[0], int) and v[0] > 16 else cases.tuple_name(v))
-def test_grids_cut_into_two_launches(device_ctx, shape, tup):
+def test_grids_with_a_small_last_round(device_ctx, shape, tup):
     """Destinations whose 256x256 tiles make a whole number of rounds of
-    workgroups plus a small rest (324, 528, 336 tiles on 256 CUs): the
-    tiled kernel runs as two launches, whole tile rows or columns first and the
-    remaining strip on a smaller tile, with the per-row / per-column parameters
-    and the sums advanced to the strip. Both cut directions, ragged edges,
-    row-major and column-major destinations, per-channel parameters as the
-    random problem draws them. Too large for the checker as a whole:
-    requantized results are compared on a sample of rows and columns that
+    workgroups plus a small rest (324, 528, 336 tiles on 256 CUs): ragged
+    edges, row-major and column-major destinations, destination pitches that
+    are not a multiple of 16 bytes, per-channel parameters as the random
+    problem draws them, on whichever tile the timing model picks. Too large
+    for the checker as a whole: requantized results are compared on a sample of rows and columns that
     includes both sides of every tile edge, and for the integer cases every
     element of the raw int32 product enters a row/column checksum."""
     import device_runner as D
