@@ -1430,14 +1430,15 @@ inline int TileCount(const GemmArgs& args, int bm, int bn) {
 enum class Tile { k256x256, k128x128, k128x64, k64x128, k64x64 };
 
 // Which tile a problem runs on is decided by a timing model of every tile, in
-// microseconds, fitted to measurements of every tile on 134 shapes for int8,
-// 96 for fp32 and 48 for int8 x int16 (destinations of 128^2 to 12288^2
-// elements, square, oblong and ragged, depths of 2 to 64 steps). The fit is
-// within 3-12 % root mean square of the measurements. Picking by it costs 1 %
-// of time over always picking the fastest tile on the shapes it was fitted to
-// and about 4 % (int8), 2 % (fp32) on shapes held out of the fit: among the
-// 128x128, 128x64 and 64x128 tiles the times are often closer than the model
-// is good.
+// microseconds, fitted to measurements of every tile on 179 shapes for int8,
+// 96 for fp32 and 48 for int8 x int16 (destinations of 128^2 to 16384^2
+// elements, square, oblong and ragged, depths of 2 to 128 steps; each tile
+// timed over 200 calls after the clock had settled, twice, in mirrored order).
+// The fit is within 3-14 % root mean square of the measurements. Picking by
+// it costs 1.2 % of time over always picking the fastest tile on the shapes
+// it was fitted to and 2.2 % (int8), 2 % (fp32) on shapes held out of the fit:
+// among the 128x128, 128x64 and 64x128 tiles the times are often closer than
+// the model is good, and their order changes from card to card.
 //
 // Workgroups are dealt to the CUs in rounds, and a workgroup costs its ring
 // fill and write-back (`overhead`, in depth steps) plus its depth steps:
@@ -1461,8 +1462,8 @@ enum class Tile { k256x256, k128x128, k128x64, k64x128, k64x64 };
 // discounted as above with `shared_last_round`.
 //
 // What the fit says about the kernels: on int8 the 256x256 tile's depth step
-// (1.37 us) is a quarter of what the 64x64 tile needs for the same area (16 x
-// 0.200 us) and 60 % of the 128x128 tile's (4 x 1.08 us / 2 side by side), so it
+// (1.11 us) is a third of what the 64x64 tile needs for the same area (16 x
+// 0.190 us) and 58 % of the 128x128 tile's (4 x 0.96 us / 2 side by side), so it
 // wins whenever its tiles fill most of a round; fp32 is bound by its matrix
 // instructions at every tile size (7.85 us against 16 x 0.562 us) and the small
 // tiles, which fill the CUs more evenly, win up to destinations of 4096^2.
@@ -1487,11 +1488,11 @@ struct TimingModel {
   double reduce;           // microseconds to add up the parts of a split
 };
 constexpr TileTiming kInt8Timings[] = {
-    {Tile::k256x256, 256, 256, 4.58, 7.20, 1.370, 0.68, 1, {}, 0},
-    {Tile::k128x128, 128, 128, 3.74, 4.36, 0.638, 0.74, 2, {0.755, 1.082}, 0.585},
-    {Tile::k128x64, 128, 64, 3.53, 4.21, 0.358, 0.87, 3, {0.257, 0.625, 1.073}, 0.78},
-    {Tile::k64x128, 64, 128, 4.43, 1.86, 0.354, 0.86, 3, {0.182, 0.777, 1.415}, 0.56},
-    {Tile::k64x64, 64, 64, 1.87, 13.6, 0.200, 0.93, 1, {}, 0},
+    {Tile::k256x256, 256, 256, 3.05, 8.96, 1.111, 0.82, 1, {}, 0},
+    {Tile::k128x128, 128, 128, 3.93, 4.04, 0.517, 0.88, 2, {0.731, 0.956}, 0.67},
+    {Tile::k128x64, 128, 64, 3.19, 4.52, 0.330, 0.95, 3, {0.226, 0.587, 0.970}, 0.81},
+    {Tile::k64x128, 64, 128, 3.96, 1.98, 0.332, 0.93, 3, {0.249, 0.702, 1.349}, 0.60},
+    {Tile::k64x64, 64, 64, 1.46, 14.1, 0.190, 0.95, 1, {}, 0},
 };
 constexpr TileTiming kF32Timings[] = {
     {Tile::k256x256, 256, 256, 0.0, 2.21, 7.854, 0.88, 1, {}, 0},
@@ -1516,7 +1517,7 @@ inline TimingModel TimingModelOf(Model model) {
     case Model::kInt8PlaneSplit:
       return {kInt8PlaneSplitTimings, 3, Tile::k64x128, 8, 3.6};
     default:
-      return {kInt8Timings, 5, Tile::k64x64, 16, 2.1};
+      return {kInt8Timings, 5, Tile::k64x64, 16, 2.4};
   }
 }
 
