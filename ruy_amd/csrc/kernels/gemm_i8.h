@@ -51,8 +51,8 @@ struct GemmArgs {
   int32_t fuse_sums = 0;
   int32_t fused_a_factor = 0;
   int32_t fused_b_factor = 0;
-  // int8 kernel, smallest tile only (GemmI8CanFuseSums): kFlipU8 for an
-  // operand that is uint8 data used in place, else 0. Bytes that the kernel
+  // int8 kernel: kFlipU8 for an operand that is uint8 data used in place,
+  // else 0. Bytes that the kernel
   // reads as zero (past the depth) would turn into -128, so k_bytes must then
   // be a multiple of 128, the kernel's depth step.
   uint32_t a_flip = 0;

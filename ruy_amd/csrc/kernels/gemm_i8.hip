@@ -198,7 +198,14 @@ struct Int8Traits {
 // them in a row on the same accumulator (the paired schedule) are the one
 // dependency the matrix pipe resolves itself, by handing the block from one
 // instruction to the next; any other accumulator is next touched 126
-// instructions later.
+// instructions later. What may stand between the two instructions of a pair:
+// LDS reads, buffer loads, scalar instructions and vector-ALU instructions
+// that have nothing to do with the pair (the address arithmetic of the last
+// steps' loads) all do, and every-element comparisons pass. A vector-ALU
+// instruction that writes an operand of the second instruction must not: four
+// v_xor_b32 on its fragments between the two gave wrong sums in exactly the
+// blocks concerned (also with one wait state behind them, not with four), so
+// whatever the vector ALU does to a pair's operands is done ahead of the pair.
 struct Int8Traits16 : Int8Traits {
   using Acc = v4i;
   static __device__ __forceinline__ void Mma(const v4i& a, const v4i& b, Acc& acc) {
@@ -353,16 +360,16 @@ bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
   const bool flip = args.a_flip != 0 || args.b_flip != 0;
-  if (args.fuse_sums || flip) {
-    // Both exist for the smallest tile only; flipped bytes need a whole number of depth steps.
-    if (!GemmI8CanFuseSums(args, num_cus) || (flip && args.k_bytes % 128 != 0)) return hipErrorInvalidValue;
-    if (flip) {
-      return args.fuse_sums ? mfma_gemm::LaunchSmallestTile<Int8Traits, true, true>(stream, args)
-                            : mfma_gemm::LaunchSmallestTile<Int8Traits, false, true>(stream, args);
-    }
-    return mfma_gemm::LaunchSmallestTile<Int8Traits, true>(stream, args);
+  // Flipped bytes need a whole number of depth steps: bytes past the depth read as zero, which would turn into -128.
+  if (flip && args.k_bytes % 128 != 0) return hipErrorInvalidValue;
+  if (args.fuse_sums) {
+    // Exists for the smallest tile only.
+    if (!GemmI8CanFuseSums(args, num_cus)) return hipErrorInvalidValue;
+    return flip ? mfma_gemm::LaunchSmallestTile<Int8Traits, true, true>(stream, args)
+                : mfma_gemm::LaunchSmallestTile<Int8Traits, true>(stream, args);
   }
-  return mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);
+  return flip ? mfma_gemm::LaunchBest<Int8Traits, true>(stream, args, num_cus)
+              : mfma_gemm::LaunchBest<Int8Traits>(stream, args, num_cus);
 }
 
 hipError_t LaunchGemmI8Batch(hipStream_t stream, const GemmArgs& args, const GemmBatch& batch, int count,

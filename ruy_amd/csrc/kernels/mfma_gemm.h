@@ -213,7 +213,7 @@ struct Cfg {
 // problems so small that a second kernel launch would cost more than the
 // extra matrix instructions.
 //
-// kFlip (same tile only): args.a_flip / args.b_flip are applied to every
+// kFlip (int8 kernel): args.a_flip / args.b_flip are applied to every
 // fragment before use, which turns uint8 data used in place into the int8
 // values the arithmetic is defined on.
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
@@ -221,7 +221,7 @@ template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums =
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
                 "fused sums exist for the tiles with one block (one block per plane) per wave only");
-  static_assert(!kFlip || WM * WN == 1, "in-place uint8 operands exist for the single-block tile only");
+  static_assert(!kFlip || !Traits::kSplitB, "in-place uint8 operands exist for the int8 kernel only");
   static_assert(!kDepthWaves || (WM == 1 && WN == (Traits::kSplitB ? 2 : 1) && BK == 128),
                 "the depth-per-wave schedule exists for the smallest tile of each kernel");
   // Accumulator blocks: Traits::kBlock = 32 (one matrix instruction covers a
@@ -231,7 +231,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // blocks a wave holds kNB*WM x kNB*WN blocks of a quarter of the size.
   constexpr int kB = Traits::kBlock;
   static_assert(kB == 32 || kB == 16, "");
-  static_assert(kB == 32 || (!kFusedSums && !kFlip && !kDepthWaves && !Traits::kSplitB),
+  static_assert(kB == 32 || (!kFusedSums && !kDepthWaves && !Traits::kSplitB),
                 "the 16x16 block form exists for the plain schedule only");
   constexpr int kNB = 32 / kB;
   constexpr int kAB = WM * kNB;  // blocks of A rows per wave
@@ -441,8 +441,10 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
                       auto dma_is_full_step) {
     Frags flipped;
     if constexpr (kFlip) {
-      flipped.a[0] = cur_raw.a[0] ^ static_cast<int>(args.a_flip);
-      flipped.b[0] = cur_raw.b[0] ^ static_cast<int>(args.b_flip);
+#pragma unroll
+      for (int i = 0; i < kAB; ++i) flipped.a[i] = cur_raw.a[i] ^ static_cast<int>(args.a_flip);
+#pragma unroll
+      for (int j = 0; j < kBB; ++j) flipped.b[j] = cur_raw.b[j] ^ static_cast<int>(args.b_flip);
     }
     const Frags& cur = kFlip ? flipped : cur_raw;
     // Few matrix instructions per sub-step: their run time does not cover the
@@ -764,7 +766,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // for all its loads but the eight just issued, i.e. for everything of step
     // kt + 1, which the second half starts to read.
     static_assert(kB == 16 && C::kKSteps == 2 && C::kStages == 2 && kAB == 8 && kBB == 8 && C::kALoads == 8 &&
-                      C::kBLoads == 8 && !kFlip && !kFusedSums,
+                      C::kBLoads == 8 && !kFusedSums,
                   "the paired schedule is written for the 256x256 tile of 16x16 blocks");
     v4i fa[2][kAB];  // [depth half][block row]
     v4i fb[2][kBB];  // [depth half][block column]
@@ -827,6 +829,22 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         if constexpr (n == 64) {
           WaitVmcnt<8>();
           __syncthreads();
+        }
+        // uint8 data in place: a fragment is flipped where the step first uses
+        // it (A rows at the first column of their half, B columns at the first
+        // row of the first half), long after its read from LDS was issued;
+        // every fragment is read anew for every step. Both depth halves are
+        // flipped ahead of the pair: nothing may write an operand of a pair's
+        // second matrix instruction once the first is issued (Int8Traits16).
+        if constexpr (kFlip && ks == 0) {
+          if constexpr (cp == 0) {
+            fa[0][i] ^= static_cast<int>(args.a_flip);
+            fa[1][i] ^= static_cast<int>(args.a_flip);
+          }
+          if constexpr (h == 0 && rp == 0) {
+            fb[0][j] ^= static_cast<int>(args.b_flip);
+            fb[1][j] ^= static_cast<int>(args.b_flip);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (decltype(first)::value && ks == 0)
@@ -1631,36 +1649,37 @@ hipError_t LaunchSmallestTileBatch(hipStream_t stream, const GemmArgs& args, con
   return LaunchBatch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, true>(stream, args, batch, count);
 }
 
-template <typename Traits>
+template <typename Traits, bool kFlip = false>
 hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int num_cus) {
   switch (tile) {
     case Tile::k256x256:
-      return Launch<typename Traits::LargeTile, 4, 4, 128, 2>(stream, args);
+      return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip>(stream, args);
     case Tile::k128x128:
-      if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128)) return Launch<Traits, 2, 2, 128, 2>(stream, args);
-      return Launch<Traits, 2, 2, 128, 4>(stream, args);
+      if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128))
+        return Launch<Traits, 2, 2, 128, 2, false, kFlip>(stream, args);
+      return Launch<Traits, 2, 2, 128, 4, false, kFlip>(stream, args);
     case Tile::k64x128:
       if constexpr (Traits::kSplitB) return LaunchSmallestTile<Traits>(stream, args);
-      if (ShallowRing(args, num_cus, 64, 128)) return Launch<Traits, 1, 2, 128, 2>(stream, args);
-      return Launch<Traits, 1, 2, 128, 4>(stream, args);
+      if (ShallowRing(args, num_cus, 64, 128)) return Launch<Traits, 1, 2, 128, 2, false, kFlip>(stream, args);
+      return Launch<Traits, 1, 2, 128, 4, false, kFlip>(stream, args);
     default:
       break;
   }
   if constexpr (!Traits::kSplitB) {
     switch (tile) {
       case Tile::k128x64:
-        if (ShallowRing(args, num_cus, 128, 64)) return Launch<Traits, 2, 1, 128, 2>(stream, args);
-        return Launch<Traits, 2, 1, 128, 4>(stream, args);
+        if (ShallowRing(args, num_cus, 128, 64)) return Launch<Traits, 2, 1, 128, 2, false, kFlip>(stream, args);
+        return Launch<Traits, 2, 1, 128, 4, false, kFlip>(stream, args);
       default:
-        return LaunchSmallestTile<Traits>(stream, args);
+        return LaunchSmallestTile<Traits, false, kFlip>(stream, args);
     }
   }
   return hipErrorInvalidValue;
 }
 
-template <typename Traits>
+template <typename Traits, bool kFlip = false>
 hipError_t LaunchBest(hipStream_t stream, const GemmArgs& args, int num_cus) {
-  return LaunchTile<Traits>(stream, args, PickTile(args, num_cus, Traits::kModel), num_cus);
+  return LaunchTile<Traits, kFlip>(stream, args, PickTile(args, num_cus, Traits::kModel), num_cus);
 }
 
 }  // namespace mfma_gemm

@@ -306,19 +306,14 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const int32_t lzp = lhs.dtype == RUYAMD_DTYPE_U8 ? lhs.zero_point - 128 : lhs.zero_point;
   const int32_t rzp = rhs.dtype == RUYAMD_DTYPE_U8 ? rhs.zero_point - 128 : rhs.zero_point;
   Operand8 a, b;
-  // Which kernel will run decides whether uint8 storage can be used in place:
-  // the skinny kernels and the smallest tile of the tiled kernel flip bytes on
-  // the way in, provided the depth is a whole number of their depth steps.
+  // uint8 storage can be used in place: the kernels flip the top bit of every
+  // byte on the way in, provided the depth is a whole number of their depth
+  // steps (bytes past the depth read as zero, which must not be flipped).
   const bool skinny = N <= kSkinnyKernelWidth || M <= kSkinnyKernelWidth;
-  int u8_depth_step = 0;
+  int u8_depth_step = 128;
   if (skinny) {
     const bool swapped = !(N <= kSkinnyKernelWidth && (M > kSkinnyKernelWidth || M >= N));
     u8_depth_step = GemvI8DepthStep(swapped ? M : N);
-  } else {
-    GemmArgs shape;
-    shape.M = M;
-    shape.N = N;
-    if (GemmI8CanFuseSums(shape, ctx->multiprocessor_count)) u8_depth_step = 128;
   }
   // Row sums of one side are needed iff the other side's zero point is not 0
   // (ruy/kernel.h:219-232).

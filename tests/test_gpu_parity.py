@@ -881,6 +881,46 @@ def test_largest_tile_over_depth_step_counts(device_ctx, tup):
             assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
 
 
+@pytest.mark.parametrize("tup", [(S.U8, S.U8, S.I32, S.U8), (S.U8, S.I8, S.I32, S.I8), (S.I8, S.U8, S.I32, S.I32)],
+                         ids=cases.tuple_name)
+def test_uint8_operands_used_in_place_on_every_tile(device_ctx, tup):
+    """uint8 operands that are depth-contiguous, aligned and a whole number of
+    128-byte depth steps deep are read where they lie and turned into int8
+    (value - 128: the top bit flipped) by the kernel, fragment by fragment, on
+    every tile: shapes that the timing model puts on the 256x256 tile (one,
+    two, three and eight depth steps: its first / odd / even / last-steps
+    forms), on 128x128 alone on a CU and two to a CU, on 128x64 and 64x128
+    (two-stage rings) and on 64x64, with ragged edges (rows and columns past
+    the end read as zeros, which the flip turns into -128 in accumulators that
+    are never stored), both destination orders, zero points that need the
+    sums of both sides. Every element where the stock reference library is
+    built, a sample of rows and columns either side of every tile edge in any
+    case."""
+    import device_runner as D
+    rng = np.random.default_rng(8080 + tup[0] * 16 + tup[1])
+    for M, K, N, orders in [(3584, 128, 4096, cases.RCC), (3584, 256, 4090, cases.RCC), (2816, 384, 4096, (1, 0, 1)),
+                            (3000, 1024, 4096, cases.RCC), (1024, 512, 4096, cases.RCC), (1536, 512, 4000, (1, 0, 1)),
+                            (2048, 512, 2560, cases.RCC), (2040, 512, 2560, (1, 0, 1)), (1024, 256, 2048, cases.RCC),
+                            (1020, 512, 3072, cases.RCC), (1024, 1024, 1000, cases.RCC), (256, 256, 256, (1, 0, 1))]:
+        p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
+                             name="%s %s %s" % (cases.tuple_name(tup), (M, K, N), orders))
+        p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER  # a cached operand is a packed one
+        if p.lhs.zero_point in (0, 128):
+            p.lhs.zero_point = 121 if tup[0] == S.U8 else 9
+        if p.rhs.zero_point in (0, 128):
+            p.rhs.zero_point = 131 if tup[1] == S.U8 else -5
+        announce(p.name)
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        assert device_ctx.last_kernel_name() == "i8_mfma"
+        rows, cols = _boundary_sample(rng, M, step=64), _boundary_sample(rng, N, step=64)
+        g, w = _sample_block(p, got, rows, cols)
+        assert (g == w).all(), "%s: %d mismatches in the sampled block" % (p.name, (g != w).sum())
+        want = O.full_size_expected(p)
+        if want is not None:
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+
+
 @pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.I16), (S.I8, S.I16, S.I32, S.I16),
                                  (S.F32, S.F32, S.F32, S.F32)], ids=cases.tuple_name)
 def test_base_addresses_that_are_not_aligned(device_ctx, tup):
