@@ -16,6 +16,7 @@ namespace ruyamd {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef uint32_t UnalignedU32 __attribute__((aligned(1)));
 
 constexpr int kTileC = 64;  // vectors per block
 constexpr int kTileK = 64;  // depth bytes per step
@@ -200,8 +201,12 @@ __global__ __launch_bounds__(256) void PackI8PairKernel(PackPairI8 pair) {
   }
 }
 
-// Source contiguous along the vectors (the transposed case) with a 4-byte
-// aligned base and pitch: a block moves a 64-vector x 64-depth tile per step.
+// Source contiguous along the vectors (the transposed case), base and pitch
+// of any alignment (global loads take any byte address on this target; with
+// an odd pitch the dword loads are merely slower than aligned ones, not the
+// byte loads they would otherwise have to be: a 2048 x 2048 operand of pitch
+// 2049 packs in 8 us instead of 40): a block moves a 64-vector x 64-depth tile
+// per step.
 // Each thread loads four dwords (4 vectors x 4 consecutive depth positions),
 // transposes the 4x4 bytes in registers with v_perm_b32 and writes four
 // dwords to the LDS tile, from which the block writes depth-contiguous
@@ -226,9 +231,16 @@ __global__ __launch_bounds__(256) void PackI8TransposeKernel(PackSource src, int
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int k = k0 + kq * 4 + i;
-      r[i] = (cfirst < src.count && k < src.K)
-                 ? *reinterpret_cast<const uint32_t*>(s + int64_t(k) * src.stride_k + cfirst)
-                 : 0u;
+      r[i] = 0u;
+      if (k < src.K) {
+        const uint8_t* at = s + int64_t(k) * src.stride_k + cfirst;
+        if (cfirst + 4 <= src.count) {
+          r[i] = *reinterpret_cast<const UnalignedU32*>(at);
+        } else {
+          // The last vectors of a count that is not a multiple of four: nothing is read past the row's end.
+          for (int j = 0; cfirst + j < src.count; ++j) r[i] |= uint32_t(at[j]) << (8 * j);
+        }
+      }
     }
     // 4x4 byte transpose: t[j] = depth bytes k..k+3 of vector cfirst + j.
     const uint32_t x0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u);
@@ -539,13 +551,13 @@ hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, 
     return hipGetLastError();
   }
   const int blocks_c = (src.count + kTileC - 1) / kTileC;
-  // Split the depth when there are too few vector slabs to fill the device.
+  // Split the depth when there are too few vector slabs to fill the device: a
+  // block's steps are a chain of load, transposition through LDS and store
+  // (about a microsecond each), so a block gets as few of them as some two
+  // thousand blocks allow (a 2048 x 2048 operand: 7.2 -> 3.6 us).
   int k_split = 1;
   const int k_steps = (ld + kTileK - 1) / kTileK;
-  if (blocks_c < 512 && k_steps > 8) {
-    k_split = min((512 + blocks_c - 1) / blocks_c, k_steps / 8);
-    if (k_split < 1) k_split = 1;
-  }
+  if (blocks_c < 2048 && k_steps > 1) k_split = min((2048 + blocks_c - 1) / blocks_c, k_steps);
   const int steps_per = (k_steps + k_split - 1) / k_split;
   const int k_span = steps_per * kTileK;
   k_split = (k_steps + steps_per - 1) / steps_per;
@@ -553,10 +565,8 @@ hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, 
     hipLaunchKernelGGL(ZeroI32Kernel, dim3((src.count + 255) / 256), dim3(256), 0, stream, sums,
                        src.count);
   }
-  // The transposed case: dword loads if base and pitch allow, bytes otherwise.
-  const bool aligned = src.stride_c == 1 && (reinterpret_cast<uintptr_t>(src.data) & 3) == 0 &&
-                       src.stride_k % 4 == 0;
-  if (aligned) {
+  // The transposed case (vectors contiguous): dword loads; any other strides: bytes.
+  if (src.stride_c == 1) {
     hipLaunchKernelGGL(PackI8TransposeKernel, dim3(blocks_c, k_split), dim3(256), 0, stream, src, dst, ld,
                        sums, k_span);
   } else {

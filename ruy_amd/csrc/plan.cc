@@ -94,12 +94,19 @@ struct PendingPack8 {
   uint64_t bytes = 0;
 };
 // Packed operands up to this size are worth pairing (the launch saved costs
-// more than the slower generic pack kernel loses on them).
+// more than the paired kernel, in which a block walks the whole depth of its
+// vectors, loses on them): 256 KiB for a depth-contiguous source, 16 KiB for a
+// transposed one, which the paired kernel moves byte by byte (512^3 with both
+// operands transposed: 26.8 us paired, 11 us as two launches).
 constexpr uint64_t kPairedPackLimit = 256 * 1024;
+constexpr uint64_t kPairedTransposedPackLimit = 16 * 1024;
+bool WorthPairing(const PendingPack8& p) {
+  return p.bytes <= (p.src.stride_k == 1 ? kPairedPackLimit : kPairedTransposedPackLimit);
+}
 
 int LaunchPendingPacks8(ruyamd_ctx* ctx, PendingPack8* a, PendingPack8* b, std::string* err) {
   hipError_t status = hipSuccess;
-  if (a->pending && b->pending && a->bytes <= kPairedPackLimit && b->bytes <= kPairedPackLimit) {
+  if (a->pending && b->pending && WorthPairing(*a) && WorthPairing(*b)) {
     status = LaunchPackI8Pair(ctx->stream, a->src, a->dst, a->ld, a->sums, b->src, b->dst, b->ld, b->sums);
   } else {
     if (a->pending) status = LaunchPackI8(ctx->stream, a->src, a->dst, a->ld, a->sums);
