@@ -557,7 +557,8 @@ hipError_t LaunchPackI8(hipStream_t stream, const PackSource& src, int8_t* dst, 
   // thousand blocks allow (a 2048 x 2048 operand: 7.2 -> 3.6 us).
   int k_split = 1;
   const int k_steps = (ld + kTileK - 1) / kTileK;
-  if (blocks_c < 2048 && k_steps > 1) k_split = min((2048 + blocks_c - 1) / blocks_c, k_steps);
+  // (Not for one or two steps: the launch that clears the sums for the parts to add to would cost more.)
+  if (blocks_c < 2048 && k_steps > 2) k_split = min((2048 + blocks_c - 1) / blocks_c, k_steps);
   const int steps_per = (k_steps + k_split - 1) / k_split;
   const int k_span = steps_per * kTileK;
   k_split = (k_steps + steps_per - 1) / steps_per;
