@@ -303,6 +303,20 @@ RUYAMD_API int ruyamd_diag_mfma_ceiling(ruyamd_ctx* ctx, int instruction,
                                         double* tera_ops_per_second,
                                         double* ms_per_launch);
 
+/* Which tile of the tiled matrix-core kernels a product of `rows` x `depth` by
+ * `depth` x `cols` would run on with `compute_units` CUs, and into how many
+ * parts its depth would be split over workgroups: `kind` 0 = 8-bit operands,
+ * 1 = int8 x int16, 2 = fp32; `rows` and `cols` are those of the destination
+ * as the kernel sees it (column-major; swap them for a row-major one). Host
+ * arithmetic only, no device needed: the choice is made by a timing model of
+ * each tile fitted to measurements on an MI355X, where the reference looks up
+ * cache sizes and thread counts (MakeBlockMap, ruy/block_map.cc:339-496).
+ * Shapes with a destination dimension of 16 or less run on the skinny kernels
+ * instead. No counterpart in the reference. */
+RUYAMD_API int ruyamd_diag_tile_for(int kind, int rows, int depth, int cols,
+                                    int compute_units, int* tile_rows,
+                                    int* tile_cols, int* depth_parts);
+
 /* Library version string. */
 RUYAMD_API const char* ruyamd_version(void);
 

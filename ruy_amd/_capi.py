@@ -64,6 +64,8 @@ PROTOTYPES = {
     "ruyamd_ctx_kernel_timing": (C.c_int, [_ctx, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
     "ruyamd_diag_mfma_ceiling": (C.c_int, [_ctx, C.c_int, C.c_int, C.c_int, C.c_double,
                                            C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "ruyamd_diag_tile_for": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int),
+                                       C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "ruyamd_version": (C.c_char_p, []),
 }
 

@@ -342,6 +342,17 @@ class Context:
             self._h, _address(x), _address(m), _address(e), _address(out), n))
 
 
+def tile_for(kind, rows, depth, cols, compute_units=256):
+    """(tile rows, tile columns, depth parts) of the tiled kernels for a product
+    whose column-major destination is rows x cols; kind 0 = 8-bit, 1 = int8 x
+    int16, 2 = fp32. Host arithmetic, no device needed."""
+    tr, tc, parts = C.c_int(0), C.c_int(0), C.c_int(0)
+    rc = lib.ruyamd_diag_tile_for(kind, rows, depth, cols, compute_units, C.byref(tr), C.byref(tc), C.byref(parts))
+    if rc != 0:
+        raise ValueError("ruyamd_diag_tile_for: bad argument")
+    return tr.value, tc.value, parts.value
+
+
 def mul_batch(items, context):
     """`items`: a sequence of (lhs, rhs, mul_params, dst) as for mul(). One call
     of ruyamd_mul_batch; a CPU caller of the reference would loop over ruy::Mul."""

@@ -1,11 +1,13 @@
 // ruyamd_diag_mfma_ceiling: measures what the int8 matrix instructions sustain
 // on this card with nothing else running (see kernels/diag.hip).
+// ruyamd_diag_tile_for: which tile the tiled kernels would run a shape on.
 #include <chrono>
 #include <cstdint>
 #include <vector>
 
 #include "context.h"
 #include "kernels/diag.h"
+#include "kernels/gemm_i8.h"
 
 using namespace ruyamd;
 
@@ -71,5 +73,20 @@ extern "C" int ruyamd_diag_mfma_ceiling(ruyamd_ctx* ctx, int instruction, int op
   *ms_per_launch = double(ms) / kTimedLaunches;
   *tera_ops_per_second =
       kMfmaCeilingOpsPerWorkgroupIteration * kIterations * workgroups / (*ms_per_launch * 1e-3) / 1e12;
+  return RUYAMD_OK;
+}
+
+extern "C" int ruyamd_diag_tile_for(int kind, int rows, int depth, int cols, int compute_units, int* tile_rows,
+                                    int* tile_cols, int* depth_parts) {
+  if (kind < 0 || kind > 2 || rows < 1 || depth < 0 || cols < 1 || compute_units < 1 || !tile_rows || !tile_cols ||
+      !depth_parts)
+    return RUYAMD_E_INVALID;
+  GemmArgs args;
+  args.M = rows;
+  args.N = kind == 1 ? 2 * cols : cols;  // the int16 operand as two planes of int8 columns
+  args.k_bytes = ((kind == 2 ? 4 * depth : depth) + 15) / 16 * 16;
+  const GemmKind which = kind == 1 ? GemmKind::kInt8Int16 : kind == 2 ? GemmKind::kF32 : GemmKind::kInt8;
+  GemmTileFor(args, compute_units, which, tile_rows, tile_cols, depth_parts);
+  if (kind == 1) *tile_cols /= 2;  // destination columns
   return RUYAMD_OK;
 }

@@ -91,6 +91,10 @@ struct DepthSplit {
 DepthSplit GemmDepthSplit(const GemmArgs& args, int num_cus, GemmKind kind);
 // Number of 32-bit counters split_counters must hold.
 int GemmDepthSplitCounters();
+// The tile the launcher of `kind` picks for these arguments (M, N, k_bytes are
+// looked at; N counts plane vectors for GemmKind::kInt8Int16) and the number
+// of parts it would split the depth into. Host arithmetic only.
+void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_rows, int* tile_cols, int* depth_parts);
 
 // True if LaunchGemmI8 would run these arguments on its smallest tile, the
 // one that has a variant with the sums fused in.

@@ -354,6 +354,21 @@ DepthSplit GemmDepthSplit(const GemmArgs& args, int num_cus, GemmKind kind) {
 
 int GemmDepthSplitCounters() { return mfma_gemm::kSplitCounters; }
 
+void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_rows, int* tile_cols, int* depth_parts) {
+  const mfma_gemm::Model which = kind == GemmKind::kInt8Int16 ? mfma_gemm::Model::kInt8PlaneSplit
+                                 : kind == GemmKind::kF32     ? mfma_gemm::Model::kF32
+                                                              : mfma_gemm::Model::kInt8;
+  const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, which);
+  const mfma_gemm::TimingModel model = mfma_gemm::TimingModelOf(which);
+  for (int i = 0; i < model.count; ++i) {
+    if (model.tiles[i].tile == tile) {
+      *tile_rows = model.tiles[i].bm;
+      *tile_cols = model.tiles[i].bn;
+    }
+  }
+  *depth_parts = mfma_gemm::PlanDepthSplit(args, num_cus, which).parts;
+}
+
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
   return mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k64x64;
 }

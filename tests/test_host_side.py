@@ -164,3 +164,40 @@ def test_product_code_never_touches_the_checker():
                         if pattern.search(line):
                             offenders.append("%s:%d: %s" % (os.path.relpath(path, ROOT), number, line.strip()))
     assert not offenders, "\n".join(offenders)
+
+
+def test_tile_choice_of_the_timing_model():
+    """The tile the tiled kernels run a shape on is host arithmetic (a timing
+    model fitted to measurements, ruyamd_diag_tile_for): the benchmark
+    configurations that rely on the smallest tile (its fused sums, its batched
+    launch, the int16 operand read in place) get it, the 8192^3 product gets
+    the 256 x 256 tile, few tiles with a long depth split it over workgroups,
+    and the choice never splits the depth on a larger tile. Arguments that
+    make no sense are refused."""
+    from ruy_amd import api
+    assert api.tile_for(0, 256, 256, 256) == (64, 64, 1)        # C1
+    assert api.tile_for(2, 1024, 1024, 1024) == (64, 64, 1)     # C2
+    assert api.tile_for(0, 1024, 1024, 196) == (64, 64, 1)      # C3
+    assert api.tile_for(1, 2048, 2048, 512) == (64, 64, 1)      # C4: 64 rows x 128 plane columns
+    assert api.tile_for(0, 8192, 8192, 8192) == (256, 256, 1)   # the headline product
+    assert api.tile_for(0, 4096, 4096, 4096) == (256, 256, 1)   # exactly one round of large tiles
+    rows, cols, parts = api.tile_for(0, 128, 65536, 128)
+    assert (rows, cols) == (64, 64) and parts == 32
+    rows, cols, parts = api.tile_for(2, 64, 32768, 64)
+    assert (rows, cols) == (64, 64) and parts > 1
+    for kind in (0, 1, 2):
+        for m, k, n in [(300, 300, 300), (1536, 512, 4096), (2048, 2048, 2048), (5000, 5000, 5000), (16384, 16384, 256)]:
+            rows, cols, parts = api.tile_for(kind, m, k, n)
+            # (int8 x int16: a tile's plane columns are half as many destination columns)
+            tiles = ((256, 128), (128, 64), (64, 64)) if kind == 1 else \
+                ((256, 256), (128, 128), (128, 64), (64, 128), (64, 64))
+            assert (rows, cols) in tiles, (kind, m, k, n)
+            assert parts == 1 or (rows, cols) == (64, 64)
+    # Fewer compute units: a grid that fills 256 CUs once is four rounds on 64 and stays on the large tile.
+    assert api.tile_for(0, 4096, 4096, 4096, compute_units=64) == (256, 256, 1)
+    for bad in [(3, 64, 64, 64), (0, 0, 64, 64), (0, 64, -1, 64), (0, 64, 64, 0)]:
+        with pytest.raises(ValueError):
+            api.tile_for(*bad)
+    with pytest.raises(ValueError):
+        api.tile_for(0, 64, 64, 64, compute_units=0)
+
