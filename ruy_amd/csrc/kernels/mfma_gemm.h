@@ -1370,9 +1370,18 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   }
 }
 
+// The two-stage 128x64 and 64x128 tiles are meant to run three workgroups to a
+// CU (their rings take 48 KiB of LDS each): the second launch bound asks for
+// three waves per SIMD, for which the compiler keeps the accumulators in
+// ordinary registers (151-154 registers a lane instead of 170-183; 2048 x 512
+// x 2560 int8: 12.2 -> 10.6 us).
+template <int WM, int WN, int STAGES, bool kDepthWaves>
+constexpr int WavesPerSimdWanted() {
+  return (!kDepthWaves && STAGES == 2 && WM * WN == 2) ? 3 : 1;
+}
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false>
-__global__ __launch_bounds__(256) void MfmaGemmKernel(GemmArgs args) {
+__global__ __launch_bounds__(256, (WavesPerSimdWanted<WM, WN, STAGES, kDepthWaves>())) void MfmaGemmKernel(GemmArgs args) {
   MfmaGemmBody<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>(args);
 }
 
@@ -1453,7 +1462,7 @@ enum class Tile { k256x256, k128x128, k128x64, k64x128, k64x64 };
 // elements, square, oblong and ragged, depths of 2 to 128 steps; each tile
 // timed over 200 calls after the clock had settled, twice, in mirrored order).
 // The fit is within 3-14 % root mean square of the measurements. Picking by
-// it costs 1.2 % of time over always picking the fastest tile on the shapes
+// it costs 1.0 % of time over always picking the fastest tile on the shapes
 // it was fitted to and 2.2 % (int8), 2 % (fp32) on shapes held out of the fit:
 // among the 128x128, 128x64 and 64x128 tiles the times are often closer than
 // the model is good, and their order changes from card to card.
@@ -1480,8 +1489,8 @@ enum class Tile { k256x256, k128x128, k128x64, k64x128, k64x64 };
 // discounted as above with `shared_last_round`.
 //
 // What the fit says about the kernels: on int8 the 256x256 tile's depth step
-// (1.11 us) is a third of what the 64x64 tile needs for the same area (16 x
-// 0.190 us) and 58 % of the 128x128 tile's (4 x 0.96 us / 2 side by side), so it
+// (1.12 us) is a third of what the 64x64 tile needs for the same area (16 x
+// 0.191 us) and 58 % of the 128x128 tile's (4 x 0.96 us / 2 side by side), so it
 // wins whenever its tiles fill most of a round; fp32 is bound by its matrix
 // instructions at every tile size (7.85 us against 16 x 0.562 us) and the small
 // tiles, which fill the CUs more evenly, win up to destinations of 4096^2.
@@ -1506,11 +1515,11 @@ struct TimingModel {
   double reduce;           // microseconds to add up the parts of a split
 };
 constexpr TileTiming kInt8Timings[] = {
-    {Tile::k256x256, 256, 256, 3.05, 8.96, 1.111, 0.82, 1, {}, 0},
-    {Tile::k128x128, 128, 128, 3.93, 4.04, 0.517, 0.88, 2, {0.731, 0.956}, 0.67},
-    {Tile::k128x64, 128, 64, 3.19, 4.52, 0.330, 0.95, 3, {0.226, 0.587, 0.970}, 0.81},
-    {Tile::k64x128, 64, 128, 3.96, 1.98, 0.332, 0.93, 3, {0.249, 0.702, 1.349}, 0.60},
-    {Tile::k64x64, 64, 64, 1.46, 14.1, 0.190, 0.95, 1, {}, 0},
+    {Tile::k256x256, 256, 256, 3.17, 8.81, 1.120, 0.81, 1, {}, 0},
+    {Tile::k128x128, 128, 128, 3.99, 3.91, 0.514, 0.89, 2, {0.732, 0.962}, 0.67},
+    {Tile::k128x64, 128, 64, 3.66, 3.02, 0.328, 0.96, 3, {0.470, 0.582, 0.919}, 0.61},
+    {Tile::k64x128, 64, 128, 4.65, 0.06, 0.328, 0.93, 3, {0.503, 0.726, 1.558}, 0.12},
+    {Tile::k64x64, 64, 64, 1.51, 13.95, 0.191, 0.94, 1, {}, 0},
 };
 constexpr TileTiming kF32Timings[] = {
     {Tile::k256x256, 256, 256, 0.0, 2.21, 7.854, 0.88, 1, {}, 0},
