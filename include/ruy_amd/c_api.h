@@ -83,11 +83,15 @@ enum {
 enum {
   RUYAMD_KERNEL_NONE = 0,
   RUYAMD_KERNEL_GENERIC = 1,   /* one output per lane, any type/layout */
-  RUYAMD_KERNEL_I8_MFMA = 2,   /* v_mfma_i32_32x32x32_i8 GEMM */
-  RUYAMD_KERNEL_F32_MFMA = 3,  /* v_mfma_f32_32x32x2_f32 GEMM */
-  RUYAMD_KERNEL_I8_GEMV = 4,   /* wavefront-reduction skinny kernel, cols<=8 */
+  RUYAMD_KERNEL_I8_MFMA = 2,   /* tiled 8-bit GEMM on the int8 matrix cores:
+                                  v_mfma_i32_16x16x64_i8 (256x256 tile) or
+                                  v_mfma_i32_32x32x32_i8 (smaller tiles) */
+  RUYAMD_KERNEL_F32_MFMA = 3,  /* tiled fp32 GEMM, v_mfma_f32_32x32x2_f32 */
+  RUYAMD_KERNEL_I8_GEMV = 4,   /* 8-bit skinny kernels, narrow side <= 16
+                                  vectors: v_dot4 and a wavefront reduction for
+                                  one, v_mfma_i32_16x16x64_i8 for 2..16 */
   RUYAMD_KERNEL_I8I16_MFMA = 5,/* int8 x int16 as two int8 MFMA planes */
-  RUYAMD_KERNEL_F32_GEMV = 6,  /* fp32 skinny kernel */
+  RUYAMD_KERNEL_F32_GEMV = 6,  /* fp32 skinny kernels, narrow side <= 16 */
 };
 
 /* Type-erased, non-owning matrix view: the fields of ruy::Matrix<T>

@@ -50,6 +50,13 @@ void* Workspace::Alloc(std::size_t bytes) {
   return p;
 }
 
+void* Workspace::AllocOptional(std::size_t bytes) {
+  const bool was_exhausted = exhausted_;
+  void* p = Alloc(bytes);
+  if (!p) exhausted_ = was_exhausted;
+  return p;
+}
+
 void Workspace::Reset() {
   exhausted_ = false;
   if (blocks_.size() > 1 && !pinned_ && growth_allowed_ && !fixed_) {

@@ -31,6 +31,9 @@ class Workspace {
   // 256-byte aligned device memory valid until the next Reset; nullptr on
   // allocation failure.
   void* Alloc(std::size_t bytes);
+  // The same for memory the caller can do without (it runs another way when
+  // there is none): a failure is not recorded by exhausted().
+  void* AllocOptional(std::size_t bytes);
   // Call only when no kernel still uses the previous call's scratch.
   void Reset();
   std::size_t capacity() const;

@@ -845,6 +845,14 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
             fb[0][j] ^= static_cast<int>(args.b_flip);
             fb[1][j] ^= static_cast<int>(args.b_flip);
           }
+          // The matrix instructions are inline assembly, which the compiler's
+          // hazard checks do not see: the distance between the last write of
+          // an operand and the pair is kept here, by hand, whatever order the
+          // compiler gives the flips above (five wait states).
+          if constexpr (cp == 0 || (h == 0 && rp == 0)) {
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_nop 4" ::: "memory");
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (decltype(first)::value && ks == 0)

@@ -247,7 +247,7 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
 void PlanDepthSplit(ruyamd_ctx* ctx, GemmKind kind, GemmArgs* args) {
   const DepthSplit split = GemmDepthSplit(*args, ctx->multiprocessor_count, kind);
   if (split.parts < 2) return;
-  void* partials = ctx->ws->Alloc(split.partial_bytes);
+  void* partials = ctx->ws->AllocOptional(split.partial_bytes);
   if (!partials) return;
   uint32_t* counters = ctx->split_counters;
   if (ctx->no_alloc) {
@@ -764,6 +764,7 @@ int RunMulBatch(ruyamd_ctx* ctx, const MulCall& first, const BatchBuffers* items
   GemmArgs shape;
   shape.M = M;
   shape.N = N;
+  shape.k_bytes = RoundUp(K, 16);  // the depth the launcher will see: both must pick the same tile
   if (!GemmI8CanFuseSums(shape, ctx->multiprocessor_count)) return RUYAMD_OK;  // not the smallest tile
   const int u8_depth_step = 128;
   const int32_t lzp = lhs.dtype == RUYAMD_DTYPE_U8 ? lhs.zero_point - 128 : lhs.zero_point;
@@ -864,6 +865,11 @@ uint64_t VectorsThatFit(const DevMat& m, int depth) {
 // type, with the int32 sums buffer the reference's packed matrices carry for
 // integer types (ruy/prepacked_cache.cc:33-37), so that entry counts and byte
 // accounting behave as in the reference. The kernel then reads the copy.
+// (Beyond the copy kernel's grid limit an operand is used where it lies.)
+bool GenericOperandIsCacheable(int64_t count, int64_t depth) {
+  return (count + 31) / 32 <= 65535 && (depth + 31) / 32 <= 65535;
+}
+
 int CacheGenericOperand(ruyamd_ctx* ctx, MulCall* call, int side, std::string* err) {
   DevMat& m = side == 0 ? call->lhs : call->rhs;
   const int policy = side == 0 ? call->lhs_cache_policy : call->rhs_cache_policy;
@@ -872,7 +878,7 @@ int CacheGenericOperand(ruyamd_ctx* ctx, MulCall* call, int side, std::string* e
   const int depth = side == 0 ? m.cols : m.rows;
   const int other_width = side == 0 ? call->rhs.cols : call->lhs.rows;
   if (!ShouldCache(policy, other_width)) return RUYAMD_OK;
-  if ((int64_t(count) + 31) / 32 > 65535 || (int64_t(depth) + 31) / 32 > 65535) return RUYAMD_OK;  // copy kernel's grid
+  if (!GenericOperandIsCacheable(count, depth)) return RUYAMD_OK;
   PackedMatrix pm;
   pm.element_size = DtypeSize(m.dtype);
   pm.is_floating_point = IsFloating(m.dtype);
@@ -969,24 +975,31 @@ const void* Advance(const void* p, int64_t elements, int element_size) {
 }  // namespace
 
 int RunMul(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
-  if (ctx->capturing && !ctx->no_alloc) {
+  const TunedPath path = ctx->force_generic ? TunedPath::kNone : TunedPathFor(*call);
+  const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
+  const uint64_t rows_fit = VectorsThatFit(call->lhs, K);
+  const uint64_t cols_fit = VectorsThatFit(call->rhs, K);
+  const bool generic = path == TunedPath::kNone || rows_fit == 0 || cols_fit == 0;  // (0: a single vector of 2 GiB)
+  const bool blocked = !generic && (uint64_t(M) > rows_fit || uint64_t(N) > cols_fit);
+  if (ctx->capturing && !ctx->no_alloc && !blocked) {
     // A call that cannot be recorded should record nothing: an operand with a
     // cache policy that was never packed is found out here, before the other
-    // side's pack or sums kernel has gone into the caller's graph.
-    const bool lhs_missing = ShouldCache(call->lhs_cache_policy, call->rhs.cols) && !ctx->cache->HasSource(call->lhs_src_key);
-    const bool rhs_missing = ShouldCache(call->rhs_cache_policy, call->lhs.rows) && !ctx->cache->HasSource(call->rhs_src_key);
+    // side's pack or sums kernel has gone into the caller's graph. Only where
+    // the path below would look the operand up under this key: the blocked
+    // path keys its entries by the sub-views' addresses (and reports a miss
+    // itself), and the generic kernel does not cache an operand beyond its
+    // copy kernel's grid.
+    const bool lhs_cached = ShouldCache(call->lhs_cache_policy, N) && (!generic || GenericOperandIsCacheable(M, K));
+    const bool rhs_cached = ShouldCache(call->rhs_cache_policy, M) && (!generic || GenericOperandIsCacheable(N, K));
+    const bool lhs_missing = lhs_cached && !ctx->cache->HasSource(call->lhs_src_key);
+    const bool rhs_missing = rhs_cached && !ctx->cache->HasSource(call->rhs_src_key);
     if (lhs_missing || rhs_missing) {
       *err = kCaptureCacheMiss;
       return RUYAMD_E_UNSUPPORTED;
     }
   }
-  const TunedPath path = ctx->force_generic ? TunedPath::kNone : TunedPathFor(*call);
-  if (path == TunedPath::kNone) return RunGeneric(ctx, call, err);
-  const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
-  const uint64_t rows_fit = VectorsThatFit(call->lhs, K);
-  const uint64_t cols_fit = VectorsThatFit(call->rhs, K);
-  if (rows_fit == 0 || cols_fit == 0) return RunGeneric(ctx, call, err);  // a single vector of 2 GiB
-  if (uint64_t(M) <= rows_fit && uint64_t(N) <= cols_fit) return RunTuned(ctx, call, path, err);
+  if (generic) return RunGeneric(ctx, call, err);
+  if (!blocked) return RunTuned(ctx, call, path, err);
 
   // An operand of 2 GiB or more: the destination is computed in blocks of
   // rows and columns whose operands fit. Each block is an ordinary call on

@@ -61,7 +61,7 @@ def _refill_rhs(problem, dp, rng):
 
 def test_captured_calls_replay_correctly():
     import torch
-    import device_runner as D
+    from ruy_amd import device_problem as D
     from ruy_amd import api
 
     ctx = api.Context()
@@ -142,7 +142,7 @@ def test_captured_cache_entries_survive_ejection():
     """A cache entry that a recorded call reads stays put when newer entries
     overflow the budget; the replay after that still gives the right answer."""
     import torch
-    import device_runner as D
+    from ruy_amd import device_problem as D
     from ruy_amd import api
 
     ctx = api.Context()

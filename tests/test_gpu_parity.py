@@ -34,8 +34,17 @@ def compare(problem, got, want, exact_fp=False):
         denom = max(np.linalg.norm(w), 1e-30)
         err = np.linalg.norm(g - w) / denom
         assert err <= REL_FROBENIUS_TOL, (problem.name, err)
-        # and padding untouched
-        mask = np.ones(got.shape, bool)
+        # and the padding between the columns / rows of a strided destination
+        # untouched: byte for byte what the checker's storage holds there.
+        d = problem.dst
+        valid = np.zeros(got.shape, bool)
+        if d.rows and d.cols:
+            strides = (1, d.stride) if d.order == S.ORDER_COL_MAJOR else (d.stride, 1)
+            np.lib.stride_tricks.as_strided(valid, (d.rows, d.cols), strides)[...] = True
+        it = got.itemsize
+        got_pad = got.view(np.uint8).reshape(-1, it)[~valid]
+        want_pad = want.view(np.uint8).reshape(-1, it)[~valid]
+        assert (got_pad == want_pad).all(), "%s: padding of the destination was written" % problem.name
     else:
         bad = np.nonzero(got != want)[0]
         assert bad.size == 0, "%s: %d mismatches, first at %d: got %r want %r" % (
@@ -58,7 +67,7 @@ def expected(problem, fill=0x5A):
 
 
 def run_both(ctx, problem, fill=0x5A):
-    import device_runner as D
+    from ruy_amd import device_problem as D
     return D.device_mul(ctx, problem, fill), expected(problem, fill)
 
 
@@ -83,14 +92,14 @@ def test_requantizer_known_answers_on_device(device_ctx):
 
 @pytest.mark.parametrize("dst_dtype,cols,zp", SATURATION_CASES)
 def test_saturation_known_answers_on_device(device_ctx, dst_dtype, cols, zp):
-    import device_runner as D
+    from ruy_amd import device_problem as D
     p, want = saturation_problem(dst_dtype, cols, zp)
     got = D.device_mul(device_ctx, p)
     assert (got[:cols] == want).all()
 
 
 def test_example_cases_on_device(device_ctx):
-    import device_runner as D
+    from ruy_amd import device_problem as D
     for p, want in example_problems():
         announce("example", p.name)
         got = O.dense_of(p, D.device_mul(device_ctx, p))
@@ -146,7 +155,7 @@ def test_all_orders_with_padded_strides(device_ctx, tup):
 def test_host_pointer_operands(device_ctx):
     """Host pointers for every buffer (what a drop-in caller of the reference
     passes): staged by the library, padding of a strided dst left alone."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     rng = np.random.default_rng(5)
     for tup in [(S.I8, S.I8, S.I32, S.I8), (S.F32, S.F32, S.F32, S.F32), (S.U8, S.U8, S.I32, S.I16)]:
         p = W.random_problem(rng, *tup, 37, 91, 23, 1, 0, 0, strided=True)
@@ -163,7 +172,7 @@ def test_large_host_pointer_operands_and_the_staging_advisory(device_ctx):
     """Host operands larger than one pinned staging chunk (4 MiB) on both the
     way in and the way out, a strided destination whose padding must survive,
     and the advisory bit that tells a caller its data crossed PCIe in the call."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     rng = np.random.default_rng(55)
     big = W.random_problem(rng, S.I8, S.I8, S.I32, S.I32, 1500, 5000, 1100, *cases.RCC, strided=True, name="big host")
     want = expected(big, fill=0x33)
@@ -194,7 +203,7 @@ def test_large_host_pointer_operands_and_the_staging_advisory(device_ctx):
 
 
 def test_empty_and_degenerate_shapes(device_ctx):
-    import device_runner as D
+    from ruy_amd import device_problem as D
     rng = np.random.default_rng(6)
     for shape in [(0, 5, 3), (4, 5, 0), (4, 0, 3), (1, 1, 1)]:
         p = W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, *shape, 1, 0, 0)
@@ -214,7 +223,7 @@ def test_empty_and_degenerate_shapes(device_ctx):
 
 
 def test_rejects_what_the_reference_forbids(device_ctx):
-    import device_runner as D
+    from ruy_amd import device_problem as D
     from ruy_amd import api
     p = W.config_int8_gemm(8)
     p.lhs.zero_point, p.rhs.zero_point = -128, -128
@@ -239,7 +248,7 @@ def test_rejects_what_the_reference_forbids(device_ctx):
 def test_golden_fixture_on_device(device_ctx):
     """Device results against the committed outputs of the stock reference
     library (tests/golden/stock_ruy_golden.npz)."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     import golden_cases
     for p, want in golden_cases.load():
         got = D.device_mul(device_ctx, p, dst_fill=0)
@@ -311,7 +320,7 @@ def test_full_size_int8_gemm_8192(device_ctx):
     rhs and lhs x (sum of rhs columns), exact modulo 2^32; (2) the requantized
     int8 result is compared bit for bit with the checker on a random 192 x 192
     sample of rows and columns plus the four tile-corner regions."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     n = 8192
     p = W.config_int8_gemm(n, config_id=6)
     announce("T requantized", n)
@@ -354,7 +363,7 @@ def test_full_size_int8_gemv_16384(device_ctx, cols, requant):
     (called twice: the second call is served from the cache and must agree, the
     reference's own caching check, ruy/test.h:733-737). Compared bit for bit
     with the checker on every element."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     n = 16384
     p = W.config_int8_gemv(n, cols, requant=requant)
     announce("GEMV", n, cols, requant)
@@ -405,7 +414,7 @@ def test_prepacked_cache_through_mul(device_ctx):
     """Cache behaviour seen through Mul: policies (ruy/prepare_packed_matrices.cc
     :38-66 with a kernel width of 8), byte accounting, distinct keys per source
     pointer and zero point, least-recently-used ejection, clear."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     from ruy_amd import api
     ctx = device_ctx
     ctx.clear_prepacked_cache()
@@ -468,7 +477,7 @@ def test_cache_policy_on_generic_tuples_and_int16_operands(device_ctx):
     as ruy/prepacked_cache.cc:33-37 counts them); the int16 operand of the
     int8 x int16 kernel keeps its two int8 planes. Entry counts and bytes are
     checked, the second call is a hit, results stay those of the checker."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     ctx = device_ctx
     ctx.clear_prepacked_cache()
     rng = np.random.default_rng(2718)
@@ -527,7 +536,7 @@ def test_cache_policy_on_generic_tuples_and_int16_operands(device_ctx):
 def test_tuned_kernels_are_the_ones_that_run(device_ctx):
     """Each benchmark configuration must be served by its tuned kernel, not by
     the generic one."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     expect = [(W.config_int8_gemm(256), "i8_mfma"), (W.config_f32_gemm(256), "f32_mfma"),
               (W.config_int8_perchannel_conv(256, 256, 196), "i8_mfma"),
               (W.config_int8_int16(256, 256, 64), "i8i16_mfma"), (W.config_int8_gemv(512, 4), "i8_gemv")]
@@ -581,7 +590,7 @@ def test_two_contexts_on_two_threads():
     concurrent Mul calls need distinct Contexts. Two threads, each with its own
     context (hence its own stream, scratch and cache), multiply concurrently."""
     import threading
-    import device_runner as D
+    from ruy_amd import device_problem as D
     from ruy_amd import api
     rng = np.random.default_rng(99)
     jobs = []
@@ -635,7 +644,7 @@ def test_caller_stream_asynchronous_calls_and_kernel_timing(device_ctx):
     """Device-side controls without a counterpart in the reference: launching on
     a caller-owned stream, returning before completion, per-kernel timing."""
     import torch
-    import device_runner as D
+    from ruy_amd import device_problem as D
     from ruy_amd import api
     ctx = api.Context()
     try:
@@ -787,7 +796,7 @@ def test_deep_shapes_that_split_the_depth(device_ctx, tup):
                 p.lhs.zero_point = 119 if tup[0] == S.U8 else -7
                 p.rhs.zero_point = 133 if tup[1] == S.U8 else 11
             announce(p.name)
-            import device_runner as D
+            from ruy_amd import device_problem as D
             want = expected(p)
             for _ in range(3):
                 compare(p, D.device_mul(device_ctx, p), want)
@@ -816,7 +825,7 @@ def test_grids_with_a_small_last_round(device_ctx, shape, tup):
     for the checker as a whole: requantized results are compared on a sample of rows and columns that
     includes both sides of every tile edge, and for the integer cases every
     element of the raw int32 product enters a row/column checksum."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     M, K, N = shape
     rng = np.random.default_rng(5150 + M)
     for orders in (cases.RCC, (1, 0, 1)):
@@ -862,7 +871,7 @@ def test_largest_tile_over_depth_step_counts(device_ctx, tup):
     element where the stock reference
     library is built (see test_full_size_int8_gemm_8192), a sample of rows and
     columns either side of every tile edge otherwise and in any case."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     rng = np.random.default_rng(4242 + tup[3])
     for K, M, N, misalign in [(16, 4096, 4096, 0), (112, 4096, 4096, 0), (128, 4000, 4090, 0), (144, 4096, 4096, 0),
                               (256, 4096, 3900, 0), (300, 4096, 4096, 0), (384, 4096, 4096, 0), (500, 3850, 4096, 0),
@@ -896,7 +905,7 @@ def test_uint8_operands_used_in_place_on_every_tile(device_ctx, tup):
     sums of both sides. Every element where the stock reference library is
     built, a sample of rows and columns either side of every tile edge in any
     case."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     rng = np.random.default_rng(8080 + tup[0] * 16 + tup[1])
     for M, K, N, orders in [(3584, 128, 4096, cases.RCC), (3584, 256, 4090, cases.RCC), (2816, 384, 4096, (1, 0, 1)),
                             (3000, 1024, 4096, cases.RCC), (1024, 512, 4096, cases.RCC), (1536, 512, 4000, (1, 0, 1)),
@@ -930,7 +939,7 @@ def test_base_addresses_that_are_not_aligned(device_ctx, tup):
     kernels' 16-byte stores go to unaligned addresses; on the tiled, the skinny
     and the one-column kernels. The guard zones around the destination stay
     intact."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     rng = np.random.default_rng(31337)
     for shape in [(200, 256, 300), (300, 1024, 7), (9, 512, 400), (500, 2048, 1), (64, 4096, 64), (130, 130, 130)]:
         for misalign in (1, 3):
@@ -947,7 +956,7 @@ def test_operand_of_more_than_2_gib(device_ctx):
     row blocks whose operands fit (here 65472 + 1088 rows), each an ordinary
     call on a sub-view; bias and per-channel multipliers follow the rows. One,
     three and seventeen columns: both skinny kernels and the tiled kernel."""
-    import device_runner as D
+    from ruy_amd import device_problem as D
     rng = np.random.default_rng(2024)
     K, rows = 32768, 66560
     block = rng.integers(-127, 128, (1024, K), dtype=np.int8)

@@ -126,3 +126,49 @@ def test_refuses_what_does_not_fit_or_is_host_memory(device_ctx):
     # The context is still good for ordinary calls afterwards.
     small = W.config_int8_gemm(256)
     compare(small, D.device_mul(device_ctx, small, entry=no_alloc), expected(small))
+
+
+def test_recorded_into_a_graph_and_replayed():
+    """The call needs no memory, so it may be recorded into a HIP graph without
+    ever having run eagerly: a product that packs both operands into the static
+    area and splits its depth over workgroups (partials and counters there
+    too) is captured, then replayed with fresh right-hand values, with eager
+    work between the replays, each replay checked against the allocating entry
+    point and the CPU checker."""
+    import torch
+    from test_gpu_graph import _refill_rhs
+    no_alloc = api.lib.ruyamd_mul_no_alloc
+    ctx = api.Context()
+    try:
+        stream = torch.cuda.Stream()
+        ctx.set_stream(stream.cuda_stream)
+        ctx.set_synchronous(False)
+        tup = (S.I8, S.I8, S.I32, S.I8)
+        p, q = _problems(tup, [(100, 5016, 70), (64, 4096, 64)], 99)
+        announce("no-alloc graph", p.name, q.name)
+        dp, dq = D.DeviceProblem(p, dst_fill=0), D.DeviceProblem(q, dst_fill=0)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            dp.run(ctx, no_alloc)
+            dq.run(ctx, no_alloc)
+        rng = np.random.default_rng(5)
+        for replay in range(3):
+            for prob, d in ((p, dp), (q, dq)):
+                _refill_rhs(prob, d, rng)
+                d.dst_all.zero_()
+            torch.cuda.synchronize()
+            with torch.cuda.stream(stream):
+                graph.replay()
+            torch.cuda.synchronize()
+            for prob, d in ((p, dp), (q, dq)):
+                got = d.dst_t.cpu().numpy().copy()
+                assert (got == O.oracle_mul(prob)).all(), (prob.name, replay)
+                # the allocating entry point, eagerly, between the replays
+                d.dst_all.zero_()
+                with torch.cuda.stream(stream):
+                    d.run(ctx)
+                torch.cuda.synchronize()
+                assert (d.dst_t.cpu().numpy() == got).all(), (prob.name, replay)
+        del graph
+    finally:
+        ctx.close()
