@@ -66,6 +66,9 @@ def parse_args():
     ap.add_argument("--zero-operands", action="store_true",
                     help="diagnostic for --workload gemm / shape: all-zero operand values, on which the card "
                          "does not run into its power limit (not a valid benchmark figure)")
+    ap.add_argument("--separate-sums-kernel", action="store_true",
+                    help="diagnostic: the operand sums of the large int8 tile by a kernel of their own in front "
+                         "of the product, as before they were formed inside its launch")
     ap.add_argument("--no-settle", action="store_true",
                     help="time the K steps right after the W warm-up steps (no settling period)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -575,6 +578,8 @@ def main():
     ctx.set_stream(torch.cuda.current_stream().cuda_stream)
     ctx.set_synchronous(False)
     ctx.set_kernel_timing(True)
+    if args.separate_sums_kernel:
+        ctx.set_sums_in_launch(0)
 
     line = {
         "metric": "int8 TOPS @%d^3 (+ GEMV HBM GB/s in 'gemv'), vs MI355X roofline and host-CPU ruy" % args.size,

@@ -268,6 +268,21 @@ RUYAMD_API int ruyamd_ctx_last_kernel(const ruyamd_ctx* ctx);
  * role of ruy's kInternalStandardCppVariant paths, ruy/kernel.h:150-169). */
 RUYAMD_API void ruyamd_ctx_force_generic_kernel(ruyamd_ctx* ctx, int force);
 
+/* Operand sums formed inside the launch of the largest int8 tile (no
+ * counterpart in the reference, whose Pack forms them in the pass that already
+ * touches the data, ruy/pack.h:105-132). On by default: a large 8-bit product
+ * whose left-hand rows (as the kernel sees them) need their depth sums is then
+ * one launch instead of a sums kernel followed by the product. `enable` 0
+ * restores the separate kernel; 2 is 1 with no wave fetching the sums ahead of
+ * the end of its main loop. `spin_limit`: how often a wave that finds the sums
+ * unfinished after its main loop looks again before it forms the sums of its
+ * rows itself (negative: keep the current value; 0: it never looks). The
+ * last two exist so that tests reach those paths. */
+RUYAMD_API int ruyamd_ctx_set_sums_in_launch(ruyamd_ctx* ctx, int enable, int spin_limit);
+/* The number of calls on this context so far whose launch formed operand sums
+ * this way (diagnostics/tests). */
+RUYAMD_API int64_t ruyamd_ctx_sums_in_launch_calls(const ruyamd_ctx* ctx);
+
 /* Timing of the main device kernel of each call, for roofline measurements.
  * While enabled, every ruyamd_mul brackets the launch of its dominant kernel
  * (the GEMM / GEMV kernel, not the pack or sums helpers) with HIP events on

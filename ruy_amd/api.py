@@ -320,6 +320,12 @@ class Context:
     def force_generic_kernel(self, flag):
         lib.ruyamd_ctx_force_generic_kernel(self._h, int(flag))
 
+    def set_sums_in_launch(self, enable, spin_limit=-1):
+        self._check(lib.ruyamd_ctx_set_sums_in_launch(self._h, int(enable), int(spin_limit)))
+
+    def sums_in_launch_calls(self):
+        return int(lib.ruyamd_ctx_sums_in_launch_calls(self._h))
+
     def set_kernel_timing(self, flag):
         self._check(lib.ruyamd_ctx_set_kernel_timing(self._h, int(flag)))
 

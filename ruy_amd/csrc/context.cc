@@ -4,6 +4,7 @@
 #include <cstdlib>
 #include <cstring>
 
+#include "kernels/fused_sums.h"
 #include "kernels/gemm_i8.h"
 #include "kernels/static_scratch.h"
 
@@ -295,11 +296,20 @@ int ruyamd_ctx_create(ruyamd_ctx** out) {
     return RUYAMD_E_HIP;
   }
   ctx->stream = ctx->own_stream;
-  const std::size_t counter_bytes = std::size_t(ruyamd::GemmDepthSplitCounters()) * sizeof(uint32_t);
-  ctx->split_counters = static_cast<uint32_t*>(DeviceAlloc(counter_bytes));
-  if (!ctx->split_counters || hipMemsetAsync(ctx->split_counters, 0, counter_bytes, ctx->own_stream) != hipSuccess ||
+  // One zeroed allocation: the two sets of words of the row sums formed
+  // inside a launch, then the depth split's counters.
+  const std::size_t split_words = std::size_t(ruyamd::GemmDepthSplitCounters());
+  const std::size_t set_words = std::size_t(ruyamd::fused_sums::kMaxRows);
+  const std::size_t counter_bytes = 2 * set_words * sizeof(long long) + split_words * sizeof(uint32_t);
+  void* const zeroed = DeviceAlloc(counter_bytes);
+  if (zeroed) {
+    ctx->row_sums_sets[0] = static_cast<long long*>(zeroed);
+    ctx->row_sums_sets[1] = ctx->row_sums_sets[0] + set_words;
+    ctx->split_counters = reinterpret_cast<uint32_t*>(ctx->row_sums_sets[1] + set_words);
+  }
+  if (!zeroed || hipMemsetAsync(zeroed, 0, counter_bytes, ctx->own_stream) != hipSuccess ||
       hipStreamSynchronize(ctx->own_stream) != hipSuccess) {
-    DeviceFree(ctx->split_counters);
+    DeviceFree(zeroed);
     (void)hipStreamDestroy(ctx->own_stream);
     delete ctx;
     return RUYAMD_E_HIP;
@@ -309,7 +319,7 @@ int ruyamd_ctx_create(ruyamd_ctx** out) {
   void* static_scratch = nullptr;
   if (ruyamd::StaticScratchOfCurrentDevice(&static_scratch) != hipSuccess) {
     (void)hipGetLastError();
-    DeviceFree(ctx->split_counters);
+    DeviceFree(ctx->row_sums_sets[0]);
     (void)hipStreamDestroy(ctx->own_stream);
     delete ctx;
     return RUYAMD_E_HIP;
@@ -327,7 +337,7 @@ void ruyamd_ctx_destroy(ruyamd_ctx* ctx) {
   if (!ctx) return;
   (void)hipStreamSynchronize(ctx->stream);
   ctx->cache.reset();
-  DeviceFree(ctx->split_counters);
+  DeviceFree(ctx->row_sums_sets[0]);  // (the depth split's counters lie behind the two sets)
   for (auto* v : {&ctx->timing_pending, &ctx->timing_pool})
     for (auto& ev : *v) {
       (void)hipEventDestroy(ev.first);
@@ -406,6 +416,16 @@ void ruyamd_ctx_set_cache_max_bytes(ruyamd_ctx* ctx, int64_t max_bytes) {
   (void)hipStreamSynchronize(ctx->stream);
   ctx->cache->SetMaxBuffersBytes(static_cast<std::ptrdiff_t>(max_bytes));
 }
+
+int ruyamd_ctx_set_sums_in_launch(ruyamd_ctx* ctx, int enable, int spin_limit) {
+  if (!ctx) return RUYAMD_E_INVALID;
+  ctx->row_sums_in_launch = enable != 0;
+  ctx->row_sums_fetch_late = enable == 2;
+  if (spin_limit >= 0) ctx->row_sums_spin_limit = spin_limit;
+  return RUYAMD_OK;
+}
+
+int64_t ruyamd_ctx_sums_in_launch_calls(const ruyamd_ctx* ctx) { return ctx ? ctx->row_sums_calls : 0; }
 
 int ruyamd_ctx_set_kernel_timing(ruyamd_ctx* ctx, int enable) {
   if (!ctx) return RUYAMD_E_INVALID;

@@ -125,6 +125,17 @@ struct ruyamd_ctx {
   uint32_t* split_counters = nullptr;
   // The same in this GPU's static scratch area, for calls that may not allocate.
   uint32_t* static_split_counters = nullptr;
+  // Row sums formed inside the launch of the largest int8 tile
+  // (kernels/fused_sums.h): two sets of 64-bit words, one per row, all zero
+  // when a launch starts. A launch uses set `row_sums_next` and clears what
+  // the launch before it left in the other one (`row_sums_dirty_rows`).
+  long long* row_sums_sets[2] = {nullptr, nullptr};
+  int row_sums_dirty_rows[2] = {0, 0};
+  int row_sums_next = 0;
+  bool row_sums_in_launch = true;
+  bool row_sums_fetch_late = false;
+  int64_t row_sums_calls = 0;
+  int row_sums_spin_limit = 1 << 14;
   // Optional timing of the dominant kernel of each call.
   bool kernel_timing = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pending;

@@ -65,6 +65,24 @@ struct GemmArgs {
   int32_t split_k = 1;
   void* split_partials = nullptr;
   uint32_t* split_counters = nullptr;
+  // int8 kernel, largest tile only (GemmI8CanFormRowSums): with row_sums set
+  // the kernel forms the depth sums of a's rows itself (fused_sums.h), in
+  // row_sums (one 64-bit word per row, rounded up to whole tiles: sum and
+  // number of contributions), zero when the launch starts, and reads them
+  // back for its write-back in place of ep.lhs_sums. It also zeroes the first
+  // row_sums_zero_rows words of row_sums_to_zero (the set the next launch uses).
+  // row_sums_spin_limit: how often a wave that finds the sums unfinished after
+  // its main loop looks again before it forms its rows' sums itself (0: it
+  // does not look at all). row_sums_fetch_late: no wave fetches the sums
+  // ahead of the end of its main loop (both for tests of those paths).
+  long long* row_sums = nullptr;
+  long long* row_sums_to_zero = nullptr;
+  int32_t row_sums_zero_rows = 0;
+  int32_t row_sums_spin_limit = 0;
+  int32_t row_sums_fetch_late = 0;
+  // The contributors of every tile row start at tile column 0
+  // (fused_sums::FirstContributorIsZero): the kernel need not look for them.
+  int32_t row_sums_first_is_zero = 0;
 };
 
 // Buffers of the products of a batched launch (GemmArgs holds what they have
@@ -99,6 +117,10 @@ void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_row
 // True if LaunchGemmI8 would run these arguments on its smallest tile, the
 // one that has a variant with the sums fused in.
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus);
+// True if LaunchGemmI8 would run these arguments (M, N, k_bytes, a_flip,
+// b_flip are looked at) on its largest tile in the form that can also produce
+// the depth sums of a's rows (GemmArgs::row_sums).
+bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
 // `count` <= kGemmBatchMax products of the shape and parameters of `args`, each
 // on its own buffers, in one launch. Only for arguments that run on the

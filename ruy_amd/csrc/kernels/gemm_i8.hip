@@ -63,6 +63,9 @@ struct Int8Traits {
   struct EdgeParams {
     int32_t bias[4], sums[4], m[4], e[4];  // [0..1]: rows l, l + 64; [2..3]: columns l, l + 64
   };
+  // kSkipRowSums: the sums of the rows are not in ep.lhs_sums (the kernel
+  // forms them itself and puts them into p.sums[0..1] later).
+  template <bool kSkipRowSums = false>
   static __device__ __forceinline__ void LoadEdgeParams(const Epilogue& ep, const int (&row)[2], const int (&col)[2],
                                                         EdgeParams& p) {
     const bool row_channel = !ep.channel_is_col;
@@ -83,7 +86,7 @@ struct Int8Traits {
       p.bias[2] = bias[col[0]];
       p.bias[3] = bias[col[1]];
     }
-    if (ep.rhs_zero_point) {
+    if (ep.rhs_zero_point && !kSkipRowSums) {
       p.sums[0] = ep.lhs_sums[row[0]];
       p.sums[1] = ep.lhs_sums[row[1]];
     }
@@ -371,6 +374,14 @@ void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_row
 
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
   return mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k64x64;
+}
+
+bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
+  const bool flip = args.a_flip != 0 || args.b_flip != 0;
+  const int tiles_m = (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
+  return !flip && args.k_bytes / 128 >= fused_sums::kMinDepthSteps &&
+         tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows &&
+         mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k256x256;
 }
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {

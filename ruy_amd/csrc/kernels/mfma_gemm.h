@@ -52,6 +52,7 @@
 #include "../epilogue.h"
 #include "../internal.h"
 #include "depth_split.h"
+#include "fused_sums.h"
 #include "gemm_i8.h"
 
 namespace ruyamd {
@@ -128,6 +129,12 @@ __device__ __forceinline__ uint32_t MulLo(uint32_t a, uint32_t b) {
 // that uses it; here that slot does useful work instead of a no-op).
 __device__ __forceinline__ void SetLdsTarget(uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0" : : "s"(lds_base));
+}
+// The same for a target that is a wave-uniform base plus a compile-time
+// constant: one instruction instead of an add and a move.
+template <uint32_t kOffset>
+__device__ __forceinline__ void SetLdsTargetAt(uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_base), "n"(kOffset) : "scc");
 }
 __device__ __forceinline__ void LoadToLdsTarget16(uint32_t voffset, uint32_t soffset, v4i rsrc) {
   asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
@@ -216,9 +223,15 @@ struct Cfg {
 // kFlip (int8 kernel): args.a_flip / args.b_flip are applied to every
 // fragment before use, which turns uint8 data used in place into the int8
 // values the arithmetic is defined on.
+//
+// kRowSums (largest int8 tile only): the launch also forms the depth sums of
+// the rows of `a`, dealt out over the first workgroups of every tile row, and
+// every workgroup fetches them shortly before its write-back (fused_sums.h).
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
-          bool kDepthWaves = false>
+          bool kDepthWaves = false, bool kRowSums = false>
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
+  static_assert(!kRowSums || (Traits::kPaired && !kFlip && !kFusedSums),
+                "row sums in passing exist for the paired schedule on int8 data");
   static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
                 "fused sums exist for the tiles with one block (one block per plane) per wave only");
   static_assert(!kFlip || !Traits::kSplitB, "in-place uint8 operands exist for the int8 kernel only");
@@ -252,6 +265,16 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int total = tiles_m * tiles_n;
   const int per_xcd = (total + 7) / 8;
   const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if constexpr (kRowSums) {
+    // The sums of the launch after this one: every workgroup clears its share
+    // (nothing in this launch looks at them).
+    const int per_group = (args.row_sums_zero_rows + int(gridDim.x) - 1) / int(gridDim.x);
+    for (int i = threadIdx.x; i < per_group; i += C::kThreads) {
+      const int at = int(blockIdx.x) * per_group + i;
+      if (at < args.row_sums_zero_rows)
+        __hip_atomic_store(args.row_sums_to_zero + at, 0ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
   if (t >= total) return;
   constexpr int kGroupM = 4;
   const int band = t / (kGroupM * tiles_n);
@@ -327,6 +350,16 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   constexpr bool kRotateDepth = WM * WN < 16;
   const int rot = __builtin_amdgcn_readfirstlane(
       kRotateDepth && K % kBK == 0 && k_tiles > 0 ? (tile_m * 5 + split_index * 3) % k_tiles : 0);
+  // kRowSums: what this wave does for the sums of its rows.
+  fused_sums::WaveShare share = {};
+  if constexpr (kRowSums) {
+    const fused_sums::WaveShare s =
+        fused_sums::ShareOfWave(tiles_m, tiles_n, tile_m, tile_n, wave_n, k_tiles, args.row_sums_first_is_zero != 0);
+    share.contributes = __builtin_amdgcn_readfirstlane(s.contributes);
+    share.first_step = __builtin_amdgcn_readfirstlane(s.first_step);
+    share.end_step = __builtin_amdgcn_readfirstlane(s.end_step);
+    share.expected = __builtin_amdgcn_readfirstlane(s.expected);
+  }
   auto phys = [&](int kt) {
     if constexpr (!kRotateDepth) return kt;
     const int p = kt + rot;
@@ -510,7 +543,10 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     const int col = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * (C::kLogicalWN * 32) + lane;
     const int row_idx[2] = {min(row, args.M - 1), min(row + 64, args.M - 1)};
     const int col_idx[2] = {min(col, args.n_logical - 1), min(col + 64, args.n_logical - 1)};
-    Traits::LoadEdgeParams(ep, row_idx, col_idx, edge);
+    if constexpr (kRowSums)
+      Traits::template LoadEdgeParams<true>(ep, row_idx, col_idx, edge);  // the sums of the rows come later
+    else
+      Traits::LoadEdgeParams(ep, row_idx, col_idx, edge);
   };
 
   // ---- software pipeline ----
@@ -804,7 +840,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // instead of the sixteen of a_k / b_k, in code that has none to spare.
     const int tail_k[2] = {a_k[0], a_k[1]};
     auto issue_tail = [&](int kt_load, auto is_b, int l) {
-      const int kbase = kt_load * kBK;
+      const int kbase = phys(kt_load) * kBK;
       const uint32_t stage = lds_base + (kt_load % C::kStages) * C::kStageBytes;
       const uint32_t goff = decltype(is_b)::value ? b_goff[l] : a_goff[l];
       const uint32_t off = kbase + tail_k[l & 1] < K ? goff + kbase : kOutOfRange;
@@ -814,8 +850,14 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // Barrier 1 stands in front of this instruction; the eight B loads follow it.
     constexpr int kBarrier1 = 24, kLoadB0 = 26, kLoadBStride = 5;
     static_assert(kLoadB0 > kBarrier1 && kLoadB0 + 7 * kLoadBStride < 64, "");
+    // Where this wave's eight loads of an operand go inside a ring slot's half.
+    const uint32_t wave_targets = lds_base + wave * C::kALoads * 1024;
     auto paired_step = [&](int kt, auto parity_constant, auto full, auto first) {
-      constexpr int kParity = decltype(parity_constant)::value;
+      constexpr int kParity = decltype(parity_constant)::value;  // of kt, hence the ring slot
+      // The depth offset of the loads of step kt + 2 (inside the depth): held
+      // in one scalar register for the whole step.
+      uint32_t refill_offset = uint32_t(phys(kt + C::kStages)) * kBK;
+      if constexpr (decltype(full)::value) asm volatile("" : "+s"(refill_offset));
       StaticFor<2 * kMmas>([&](auto n_constant) {
         constexpr int n = decltype(n_constant)::value;
         constexpr int pair = n / 2;
@@ -878,23 +920,88 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         constexpr bool kTargetA = n + 1 >= 66 && n + 1 < 112 && (n + 1 - 66) % 6 == 0;
         if constexpr (decltype(full)::value && (kTargetA || kTargetB)) {
           constexpr int l = kTargetB ? (n + 1 - kLoadB0) / kLoadBStride : (n + 1 - 66) / 6;
-          const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
-          SetLdsTarget(stage + (kTargetB ? C::kBM * kBK : 0) + (wave * C::kALoads + l) * 1024);
+          SetLdsTargetAt<uint32_t(kParity * C::kStageBytes + (kTargetB ? C::kBM * kBK : 0) + l * 1024)>(wave_targets);
         }
         if constexpr (kLoadA || kLoadB) {
           constexpr int l = kLoadB ? (n - kLoadB0) / kLoadBStride : (n - 66) / 6;
           if constexpr (decltype(full)::value)
-            LoadToLdsTarget16(kLoadB ? b_goff[l] : a_goff[l], uint32_t(kt + C::kStages) * kBK, kLoadB ? b_rsrc : a_rsrc);
+            LoadToLdsTarget16(kLoadB ? b_goff[l] : a_goff[l], refill_offset, kLoadB ? b_rsrc : a_rsrc);
           else
             issue_tail(kt + C::kStages, std::integral_constant<bool, kLoadB>(), l);
         }
       });
       __builtin_amdgcn_sched_barrier(0);
     };
+    // ---- the sums of the rows of `a`, formed in passing (kRowSums; fused_sums.h) ----
+    // Between two ring steps fragment rows 0-3 hold the step to come and rows
+    // 4-7 the step just done. A contributing wave adds up the registers of the
+    // walk steps of its share there: lane l holds, of block row i, depth
+    // granules l / 16 (and 4 + l / 16) of row 16 i + l % 16.
+    int32_t row_sum[kAB];
+    // The share is a run of walk steps [first_step, end_step): something to do
+    // between ring steps first_step .. last_event, where the share's sums go
+    // out: one 64-bit atomic add per row that carries the sum and counts the
+    // contribution (fused_sums::Contribution).
+    const int last_event = min(share.end_step + 1, k_tiles);
+    if constexpr (kRowSums) {
+#pragma unroll
+      for (int i = 0; i < kAB; ++i) row_sum[i] = 0;
+    }
+    auto add_rows = [&](auto first_block_constant) {
+      constexpr int kFirst = decltype(first_block_constant)::value;
+#pragma unroll
+      for (int i = kFirst; i < kFirst + kAB / 2; ++i)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) row_sum[i] = __builtin_amdgcn_sdot4(fa[ks][i][d], 0x01010101, row_sum[i], false);
+    };
+    auto publish = [&]() {
+      long long* out = args.row_sums + m0 + wave_m * (WM * 32) + (lane & 15);
+#pragma unroll
+      for (int i = 0; i < kAB; ++i) {
+        // The four lanes that share a row: lane rows 0-3 of the wave.
+        const auto halves = __builtin_amdgcn_permlane32_swap(row_sum[i], row_sum[i], false, false);
+        const int two = halves[0] + halves[1];
+        const auto quarters = __builtin_amdgcn_permlane16_swap(two, two, false, false);
+        const int all = quarters[0] + quarters[1];
+        if (lane < 16)
+          __hip_atomic_fetch_add(out + 16 * i, fused_sums::Contribution(all), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    };
+    // The sums of the wave's 128 rows, 16 bytes (two rows) a lane, into the
+    // wave's parameter area in LDS.
+    constexpr int kSumsArea = C::kStages * C::kStageBytes;  // + wave * Traits::kParamInts * 4
+    auto fetch_sums = [&]() {
+      const v4i sums_rsrc = MakeRsrc(args.row_sums, uint32_t(tiles_m * C::kBM) * 8u);
+      asm volatile(
+          "s_mov_b32 m0, %0\n\t"
+          "s_nop 0\n\t"
+          "buffer_load_dwordx4 %1, %2, 0 offen sc1 lds"
+          :
+          : "s"(lds_base + kSumsArea + wave * Traits::kParamInts * 4),
+            "v"(uint32_t(m0 + wave_m * (WM * 32) + 2 * lane) * 8u), "s"(sums_rsrc)
+          : "memory");
+    };
+    // `beta`: the number of ring steps done so far. Called only where a
+    // contributor may have something to do (and at the last steps): a lone
+    // wave on its SIMD pays for every instruction between two ring steps with
+    // idle matrix cores. Between two ring steps fragment rows 0-3 hold the
+    // step to come and rows 4-7 the step just done.
+    auto between = [&](int beta) {
+      if constexpr (kRowSums) {
+        if (__builtin_expect(!share.contributes || beta < share.first_step || beta > last_event, 1)) return;
+        if (beta < share.end_step) add_rows(std::integral_constant<int, 0>());
+        if (beta > share.first_step && beta <= share.end_step) add_rows(std::integral_constant<int, kAB / 2>());
+        if (beta == last_event) publish();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
     const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
     using Even = std::integral_constant<int, 0>;
     using Odd = std::integral_constant<int, 1>;
     int kt = 1;
+    between(0);
     if (full_end > 0) {
       paired_step(0, Even(), std::true_type(), std::true_type());
     } else if (k_tiles > 0) {
@@ -902,17 +1009,88 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     } else {
       clear_accumulators();
     }
-    for (; kt + 1 < full_end; kt += 2) {
-      paired_step(kt, Odd(), std::true_type(), std::false_type());
-      paired_step(kt + 1, Even(), std::true_type(), std::false_type());
-    }
+    between(1);
     // (Straight-line loop bodies only: with a branch on the step's parity in
-    // the loop the register allocator moves accumulators through scratch memory.)
-    for (; kt + 1 < k_tiles; kt += 2) {
-      paired_step(kt, Odd(), std::false_type(), std::false_type());
-      paired_step(kt + 1, Even(), std::false_type(), std::false_type());
+    // the loop the register allocator moves accumulators through scratch
+    // memory; so it does with a second copy of the loop below.)
+    //
+    // The steps whose loads lie inside the depth run two at a time in a loop
+    // that does nothing else. A contributor leaves it for the pair of steps
+    // with its next event, which runs in the loop of the last steps (that one
+    // looks up between any two steps, and its loads are good for any step),
+    // and comes back. Everybody else never leaves it.
+    bool sums_asked_for = false;
+    for (;;) {
+      // The next event, if any: between steps 2 j - 1 and 2 j or behind step
+      // 2 j, i.e. in the pair that starts with step 2 j - 1.
+      const int next_event = max(share.first_step, kt + 1);
+      const int fast_until =
+          kRowSums && share.contributes && next_event <= last_event ? min(full_end, (next_event & ~1) - 1) : full_end;
+      for (; kt + 1 < fast_until; kt += 2) {
+        paired_step(kt, Odd(), std::true_type(), std::false_type());
+        paired_step(kt + 1, Even(), std::true_type(), std::false_type());
+      }
+      const bool last_steps = !kRowSums || kt + 1 >= full_end;
+      if constexpr (kRowSums) {
+        // Two or three steps before the end: the sums are asked for (they land
+        // in LDS while the last steps run; whether they were complete is
+        // looked at after the loop).
+        if (last_steps && !sums_asked_for && !args.row_sums_fetch_late) fetch_sums();
+        sums_asked_for = sums_asked_for || last_steps;
+      }
+      const int checked_until = last_steps ? k_tiles : kt + 2;
+      for (; kt + 1 < checked_until; kt += 2) {
+        paired_step(kt, Odd(), std::false_type(), std::false_type());
+        between(kt + 1);
+        paired_step(kt + 1, Even(), std::false_type(), std::false_type());
+        between(kt + 2);
+      }
+      if (last_steps) break;
     }
-    if (kt < k_tiles) paired_step(kt, Odd(), std::false_type(), std::false_type());
+    if (kt < k_tiles) {
+      paired_step(kt, Odd(), std::false_type(), std::false_type());
+      between(kt + 1);
+    }
+    if constexpr (kRowSums) {
+      Traits::DrainMma();
+      WaitVmcnt<0>();
+      const int first_row = m0 + wave_m * (WM * 32);
+      const long long* fetched =
+          reinterpret_cast<const long long*>(lds + kSumsArea + wave * Traits::kParamInts * 4);
+      long long word[2] = {fetched[lane], fetched[64 + lane]};
+      bool ready = !args.row_sums_fetch_late &&
+                   __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
+                         fused_sums::ContributionsIn(word[1]) == share.expected);
+      // Not complete when they were asked for: look again, a bounded number
+      // of times. Contributors that never got to run (a device shared with
+      // somebody else's work) must not be waited for without end: then this
+      // wave forms the sums of its rows itself, from global memory.
+      for (int spins = 0; !ready && spins < args.row_sums_spin_limit; ++spins) {
+        if (spins) __builtin_amdgcn_s_sleep(8);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          word[h] = __hip_atomic_load(args.row_sums + first_row + 64 * h + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ready = __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
+                      fused_sums::ContributionsIn(word[1]) == share.expected);
+      }
+      if (ready) {
+        edge.sums[0] = fused_sums::SumIn(word[0]);
+        edge.sums[1] = fused_sums::SumIn(word[1]);
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int row = min(first_row + 64 * h + lane, args.M - 1);
+          const char* from = static_cast<const char*>(args.a) + size_t(row) * size_t(args.lda);
+          int sum = 0;
+          for (int k = 0; k < K; k += kGranule) {
+            const v4i x = *reinterpret_cast<const v4i*>(from + k);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) sum = __builtin_amdgcn_sdot4(x[d], 0x01010101, sum, false);
+          }
+          edge.sums[h] = sum;
+        }
+      }
+    }
   } else {
     Frags f[2];
     // The fragments of consecutive sub-steps alternate between f[0] and f[1].
@@ -1388,9 +1566,9 @@ constexpr int WavesPerSimdWanted() {
   return (!kDepthWaves && STAGES == 2 && WM * WN == 2) ? 3 : 1;
 }
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
-          bool kDepthWaves = false>
+          bool kDepthWaves = false, bool kRowSums = false>
 __global__ __launch_bounds__(256, (WavesPerSimdWanted<WM, WN, STAGES, kDepthWaves>())) void MfmaGemmKernel(GemmArgs args) {
-  MfmaGemmBody<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>(args);
+  MfmaGemmBody<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves, kRowSums>(args);
 }
 
 // Several products of one shape in one launch: grid.z counts the products,
@@ -1429,7 +1607,7 @@ hipError_t LaunchBatch(hipStream_t stream, const GemmArgs& args, const GemmBatch
 }
 
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
-          bool kDepthWaves = false>
+          bool kDepthWaves = false, bool kRowSums = false>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB, Traits::kBlock>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
@@ -1438,7 +1616,11 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int grid = ((total + 7) / 8) * 8;
   // The depth-per-wave schedule: two ring slots of 16 KiB for each of four waves.
   const size_t lds_bytes = kDepthWaves ? size_t(4 * 2 * 128 * BK) : size_t(C::kLdsBytes);
-  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves>;
+  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves, kRowSums>;
+  if (kRowSums != (args.row_sums != nullptr)) return hipErrorInvalidValue;
+  if (kRowSums && (!args.row_sums_to_zero || tiles_m * C::kBM > fused_sums::kMaxRows ||
+                   args.row_sums_zero_rows > fused_sums::kMaxRows))
+    return hipErrorInvalidValue;
   if (lds_bytes > 48 * 1024) {
     // Once per process; static initialisation is safe against concurrent callers.
     static const hipError_t attr = hipFuncSetAttribute(
@@ -1670,6 +1852,10 @@ template <typename Traits, bool kFlip = false>
 hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int num_cus) {
   switch (tile) {
     case Tile::k256x256:
+      if constexpr (Traits::LargeTile::kPaired && !kFlip) {
+        if (args.row_sums)
+          return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, false, false, true>(stream, args);
+      }
       return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip>(stream, args);
     case Tile::k128x128:
       if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128))

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdint>
 
+#include "kernels/fused_sums.h"
 #include "kernels/gemm_i8.h"
 #include "kernels/static_scratch.h"
 
@@ -381,12 +382,33 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   }
   GemmArgs args;
   const bool swap = SetupInt8Gemm(ctx, *call, a, b, lzp, rzp, &args);
+  // The largest tile can form the sums of the rows of its `a` operand in
+  // passing (kernels/fused_sums.h): one launch instead of a sums kernel and
+  // the product. Not for a call that is being recorded (a replayed launch
+  // would meet the sums its last run left behind) and not for a call that
+  // shares the GPU's static scratch area with other contexts.
+  Operand8& kernel_a = swap ? b : a;
+  bool row_sums_in_launch = false;
+  if (!args.fuse_sums && kernel_a.sums_pending && ctx->row_sums_in_launch && !ctx->capturing && !ctx->no_alloc &&
+      GemmI8CanFormRowSums(args, ctx->multiprocessor_count)) {
+    const int set = ctx->row_sums_next;
+    args.row_sums = ctx->row_sums_sets[set];
+    args.row_sums_to_zero = ctx->row_sums_sets[set ^ 1];
+    args.row_sums_zero_rows = ctx->row_sums_dirty_rows[set ^ 1];
+    args.row_sums_spin_limit = ctx->row_sums_spin_limit;
+    args.row_sums_fetch_late = ctx->row_sums_fetch_late;
+    args.row_sums_first_is_zero = fused_sums::FirstContributorIsZero(
+        (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows, (args.N + fused_sums::kTileRows - 1) / fused_sums::kTileRows);
+    kernel_a.sums_pending = false;
+    row_sums_in_launch = true;
+  }
   if (!args.fuse_sums) {
     if (int rc = MaterializeSums(ctx, &a, K, err)) return rc;
     if (int rc = MaterializeSums(ctx, &b, K, err)) return rc;
   }
   args.ep.lhs_sums = (swap ? b : a).sums;
   args.ep.rhs_sums = (swap ? a : b).sums;
+  if (row_sums_in_launch) args.ep.lhs_sums = nullptr;  // the kernel does not look there
   PlanDepthSplit(ctx, GemmKind::kInt8, &args);
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
@@ -394,6 +416,14 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   if (launched != hipSuccess) {
     *err = "int8 MFMA kernel launch failed";
     return RUYAMD_E_HIP;
+  }
+  if (row_sums_in_launch) {
+    // The launch is on the stream: it leaves its own set dirty and the other one clean.
+    const int set = ctx->row_sums_next;
+    ctx->row_sums_dirty_rows[set ^ 1] = 0;
+    ctx->row_sums_dirty_rows[set] = RoundUp(args.M, fused_sums::kTileRows);
+    ctx->row_sums_next = set ^ 1;
+    ++ctx->row_sums_calls;
   }
   ctx->last_kernel = RUYAMD_KERNEL_I8_MFMA;
   return RUYAMD_OK;

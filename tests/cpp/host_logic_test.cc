@@ -12,6 +12,16 @@
 // once whatever the remainder, exactly one workgroup per tile elects itself,
 // it sees every part, the sum is taken in part order, and the counters are
 // back at zero for the next launch.
+//
+// Row sums formed inside the launch of the largest int8 tile: which
+// workgroups of a tile row add up which depth steps (kernels/fused_sums.h).
+// Checked for every grid up to 48 x 48 tiles and several depths: the shares of
+// a row's contributing waves cover every depth step exactly once for each of
+// the two groups of 128 rows, the number of contributions everybody waits for
+// is the number of contributing waves, and the contributors are among the
+// tiles of their row that the hardware starts first; and a row's 64-bit word
+// gives back the sum and the number of contributions whatever the signs and
+// the order of the shares.
 #include <atomic>
 #include <cstdint>
 #include <cstdio>
@@ -19,6 +29,7 @@
 #include <vector>
 
 #include "kernels/depth_split.h"
+#include "kernels/fused_sums.h"
 #include "kernels/launch_geometry.h"
 
 static int g_failures = 0;
@@ -158,7 +169,90 @@ static void TestDepthSplitArrivalProtocol() {
   }
 }
 
+namespace fs = ruyamd::fused_sums;
+
+static void CheckRowSumShares(int tiles_m, int tiles_n, int depth_steps) {
+  for (int tile_m = 0; tile_m < tiles_m; ++tile_m) {
+    const fs::Contributors c = fs::ContributorsOfRow(tiles_m, tiles_n, tile_m);
+    EXPECT(c.count >= 1 && c.count <= fs::kMaxContributorTiles);
+    EXPECT(c.first_tile_n >= 0 && c.first_tile_n + c.count <= tiles_n);
+    // The first contributor is in the round of workgroups (32 to an XCD) in
+    // which the first tile of the row is started, and the contributors follow
+    // each other in the tile order.
+    int first_place = 1 << 30;
+    for (int n = 0; n < tiles_n; ++n) {
+      const int place = fs::PlaceInQueue(tiles_m, tiles_n, fs::TileOrder(tiles_m, tiles_n, tile_m, n));
+      if (place < first_place) first_place = place;
+    }
+    const int order0 = fs::TileOrder(tiles_m, tiles_n, tile_m, c.first_tile_n);
+    EXPECT(fs::PlaceInQueue(tiles_m, tiles_n, order0) / 32 == first_place / 32);
+    const int order_last = fs::TileOrder(tiles_m, tiles_n, tile_m, c.first_tile_n + c.count - 1);
+    EXPECT(order_last - order0 <= (fs::kMaxContributorTiles - 1) * fs::kBandRows);
+    // Coverage: every depth step once, by the waves that hold the same rows
+    // (wave_n 0 and 1 of every contributing workgroup).
+    std::vector<int> seen(depth_steps, 0);
+    int contributing = 0, expected = -1;
+    for (int n = 0; n < tiles_n; ++n) {
+      for (int wave_n = 0; wave_n < 2; ++wave_n) {
+        const fs::WaveShare s = fs::ShareOfWave(tiles_m, tiles_n, tile_m, n, wave_n, depth_steps);
+        EXPECT(expected < 0 || expected == s.expected);
+        expected = s.expected;
+        EXPECT(s.contributes == (n >= c.first_tile_n && n < c.first_tile_n + c.count));
+        // The same with the hint that saves the search for the contributors.
+        if (fs::FirstContributorIsZero(tiles_m, tiles_n)) {
+          const fs::WaveShare h = fs::ShareOfWave(tiles_m, tiles_n, tile_m, n, wave_n, depth_steps, true);
+          EXPECT(h.contributes == s.contributes && h.first_step == s.first_step && h.end_step == s.end_step &&
+                 h.expected == s.expected);
+        }
+        if (!s.contributes) continue;
+        ++contributing;
+        EXPECT(s.first_step >= 0 && s.first_step <= s.end_step && s.end_step <= depth_steps);
+        for (int step = s.first_step; step < s.end_step; ++step) ++seen[step];
+      }
+    }
+    EXPECT(contributing == expected);
+    for (int k = 0; k < depth_steps; ++k) EXPECT(seen[k] == 1);
+  }
+}
+
+static void TestRowSumWords() {
+  // Shares of every sign and size that a depth of up to 2^23 bytes can
+  // produce, added in any order, 1 to 16 of them.
+  uint64_t state = 12345;
+  auto next = [&]() {
+    state = state * 6364136223846793005ull + 1442695040888963407ull;
+    return state >> 33;
+  };
+  const int extremes[] = {0, 1, -1, 127 * (1 << 23), -128 * (1 << 23), 2147483647, -2147483647 - 1};
+  for (int trial = 0; trial < 20000; ++trial) {
+    const int n = 1 + int(next() % 16);
+    long long word = 0;
+    int64_t sum = 0;
+    for (int i = 0; i < n; ++i) {
+      int share = trial < 2000 ? extremes[next() % 7] / n : int(int64_t(next() % (1ull << 31)) - (1ll << 30)) / n;
+      word += fs::Contribution(share);
+      sum += share;
+      EXPECT(fs::ContributionsIn(word) == i + 1);
+      EXPECT(fs::SumIn(word) == int(sum));
+    }
+  }
+  EXPECT(fs::ContributionsIn(0) == 0 && fs::SumIn(0) == 0);
+}
+
+static void TestRowSumShares() {
+  const int before = g_failures;
+  for (int tiles_m = 1; tiles_m <= 48 && g_failures == before; ++tiles_m)
+    for (int tiles_n = 1; tiles_n <= 48 && g_failures == before; ++tiles_n)
+      for (int depth_steps : {16, 17, 33, 64}) CheckRowSumShares(tiles_m, tiles_n, depth_steps);
+  CheckRowSumShares(32, 32, 64);   // 8192^3
+  CheckRowSumShares(256, 3, 128);  // the most rows a launch may have
+  CheckRowSumShares(5, 200, 20);
+  if (g_failures != before) std::fprintf(stderr, "(row-sum shares: stopped at the first failing grid)\n");
+}
+
 int main() {
+  TestRowSumWords();
+  TestRowSumShares();
   TestGenericGrid();
   TestElementwiseBlocks();
   TestDepthPartsCoverEveryStepOnce();

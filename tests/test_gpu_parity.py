@@ -857,6 +857,68 @@ def test_grids_with_a_small_last_round(device_ctx, shape, tup):
         assert ((got.sum(axis=1) % 2**32) == (L @ R.sum(axis=1)) % 2**32).all()
 
 
+@pytest.mark.parametrize("mode", ["ahead", "late", "own", "separate"])
+def test_operand_sums_formed_inside_the_launch(mode):
+    """The 256x256 tile of the int8 kernel forms the depth sums of its `a`
+    operand's rows in passing, dealt out over the first workgroups of every
+    tile row (one launch where a sums kernel used to run in front). Shapes:
+    one round of tiles at the shortest depth that takes this route; ragged
+    edges with a depth of 17 steps and a bit; grids whose bands of four tile rows begin in the middle of an XCD's
+    queue (10 x 20 and 11 x 16 tiles), a last band of two tile rows; both
+    destination orders (the row-major one swaps the operands, so the sums are
+    then those of the right-hand side); zero points that need the sums of both
+    sides. Three calls in a row on one context, of different heights, so that
+    each launch meets the counters and sums that the launch before cleared for
+    it. Modes: the sums fetched three depth steps ahead of the write-back (the
+    default), only after the main loop (polling the arrival counter), formed by
+    every wave for its own rows from global memory (what a wave does when the
+    contributions do not arrive), and the separate kernel. Every element where
+    the stock reference library is built, a sample of rows and columns either
+    side of every tile edge in any case."""
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    ctx = api.Context()
+    try:
+        ctx.set_sums_in_launch({"ahead": 1, "late": 2, "own": 1, "separate": 0}[mode], 0 if mode == "own" else -1)
+        if mode == "own":
+            ctx.set_sums_in_launch(2, 0)  # no fetch ahead either: every wave forms its rows' sums itself
+        rng = np.random.default_rng(60606)
+        tup = (S.I8, S.I8, S.I32, S.I8)
+        expected_calls = 0
+        for (M, K, N), orders in [((4096, 2048, 4096), cases.RCC), ((4000, 2192, 3900), (1, 0, 1)),
+                                  ((2560, 2048, 5120), cases.RCC), ((4096, 2048, 2816), (1, 0, 1)),
+                                  ((3072, 4096, 3072), cases.RCC)]:
+            p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
+                                 name="%s %s %s %s" % (cases.tuple_name(tup), (M, K, N), orders, mode))
+            p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+            p.lhs.zero_point, p.rhs.zero_point = (9, -5) if M != 2560 else (0, -3)
+            assert api.tile_for(0, *((M, K, N) if orders[2] == S.ORDER_COL_MAJOR else (N, K, M))) == (256, 256, 1)
+            announce(p.name)
+            got = D.device_mul(ctx, p, dst_fill=0)
+            assert ctx.last_kernel_name() == "i8_mfma"
+            expected_calls += mode != "separate"
+            assert ctx.sums_in_launch_calls() == expected_calls
+            rows, cols = _boundary_sample(rng, M, step=128), _boundary_sample(rng, N, step=128)
+            g, w = _sample_block(p, got, rows, cols)
+            assert (g == w).all(), "%s: %d mismatches in the sampled block" % (p.name, (g != w).sum())
+            want = O.full_size_expected(p)
+            if want is not None:
+                bad = np.nonzero(got != want)[0]
+                assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+        # Not while a graph is being recorded and not for uint8 data used in place: the separate kernel.
+        u8 = W.random_problem(rng, S.U8, S.I8, S.I32, S.I8, 4096, 2048, 4096, *cases.RCC, strided=False, name="u8 lhs")
+        u8.lhs.cache_policy = u8.rhs.cache_policy = S.CACHE_NEVER
+        u8.lhs.zero_point, u8.rhs.zero_point = 121, -5
+        announce(u8.name)
+        got = D.device_mul(ctx, u8, dst_fill=0)
+        assert ctx.sums_in_launch_calls() == expected_calls
+        rows, cols = _boundary_sample(rng, 4096, step=128), _boundary_sample(rng, 4096, step=128)
+        g, w = _sample_block(u8, got, rows, cols)
+        assert (g == w).all()
+    finally:
+        ctx.close()
+
+
 @pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I16), (S.I8, S.U8, S.I32, S.I32)],
                          ids=cases.tuple_name)
 def test_largest_tile_over_depth_step_counts(device_ctx, tup):
