@@ -129,24 +129,29 @@ struct WaveShare {
   int expected;      // contributions a row's word shows when its sum is complete
 };
 
+// Depth steps per contributing wave when `contributor_tiles` workgroups of a
+// tile row contribute.
+RUYAMD_HOST_DEVICE inline int StepsPerWave(int depth_steps, int contributor_tiles) {
+  return (depth_steps + 2 * contributor_tiles - 1) / (2 * contributor_tiles);
+}
+
 // `wave_n`: which of the workgroup's two waves that hold the same rows.
-// `depth_steps`: ring steps of the whole depth. `first_is_zero`: the caller
-// knows that the contributors of every tile row of this grid start at tile
-// column 0 (FirstContributorIsZero), which saves the divisions that finding
-// them takes. The contributing waves take consecutive runs of the depth
+// `depth_steps`: ring steps of the whole depth. `uniform_run`: not 0 if the
+// caller knows that the contributors of every tile row of this grid start at
+// tile column 0 (FirstContributorIsZero), and then StepsPerWave of the grid,
+// which saves the divisions that finding both takes. The contributing waves take consecutive runs of the depth
 // steps, the two waves of a workgroup neighbouring runs: a workgroup is busy
 // with the sums during one short stretch of its main loop.
 RUYAMD_HOST_DEVICE inline WaveShare ShareOfWave(int tiles_m, int tiles_n, int tile_m, int tile_n, int wave_n,
-                                               int depth_steps, bool first_is_zero = false) {
+                                               int depth_steps, int uniform_run = 0) {
   const Contributors c =
-      first_is_zero ? Contributors{0, tiles_n < kMaxContributorTiles ? tiles_n : kMaxContributorTiles}
-                    : ContributorsOfRow(tiles_m, tiles_n, tile_m);
+      uniform_run ? Contributors{0, tiles_n < kMaxContributorTiles ? tiles_n : kMaxContributorTiles}
+                  : ContributorsOfRow(tiles_m, tiles_n, tile_m);
   WaveShare s;
   const int index = tile_n - c.first_tile_n;
   s.contributes = index >= 0 && index < c.count;
   s.expected = 2 * c.count;
-  const int waves = 2 * c.count;
-  const int run = (depth_steps + waves - 1) / waves;
+  const int run = uniform_run ? uniform_run : StepsPerWave(depth_steps, c.count);
   const int first = (2 * index + wave_n) * run;
   const int end = first + run;
   s.first_step = first < depth_steps ? first : depth_steps;

@@ -80,9 +80,11 @@ struct GemmArgs {
   int32_t row_sums_zero_rows = 0;
   int32_t row_sums_spin_limit = 0;
   int32_t row_sums_fetch_late = 0;
-  // The contributors of every tile row start at tile column 0
-  // (fused_sums::FirstContributorIsZero): the kernel need not look for them.
-  int32_t row_sums_first_is_zero = 0;
+  // Not 0: the contributors of every tile row start at tile column 0
+  // (fused_sums::FirstContributorIsZero) and each of their waves takes this
+  // many depth steps (fused_sums::StepsPerWave): the kernel need not work
+  // either out.
+  int32_t row_sums_uniform_run = 0;
 };
 
 // Buffers of the products of a batched launch (GemmArgs holds what they have

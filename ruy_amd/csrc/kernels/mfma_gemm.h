@@ -354,7 +354,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   fused_sums::WaveShare share = {};
   if constexpr (kRowSums) {
     const fused_sums::WaveShare s =
-        fused_sums::ShareOfWave(tiles_m, tiles_n, tile_m, tile_n, wave_n, k_tiles, args.row_sums_first_is_zero != 0);
+        fused_sums::ShareOfWave(tiles_m, tiles_n, tile_m, tile_n, wave_n, k_tiles, args.row_sums_uniform_run);
     share.contributes = __builtin_amdgcn_readfirstlane(s.contributes);
     share.first_step = __builtin_amdgcn_readfirstlane(s.first_step);
     share.end_step = __builtin_amdgcn_readfirstlane(s.end_step);
@@ -806,12 +806,14 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
                   "the paired schedule is written for the 256x256 tile of 16x16 blocks");
     v4i fa[2][kAB];  // [depth half][block row]
     v4i fb[2][kBB];  // [depth half][block column]
-    auto read_a = [&](int kt, int ks, int i) {
-      const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
+    // `slot`: the ring slot of the step whose fragments are read (its parity:
+    // a compile-time constant wherever these are called).
+    auto read_a = [&](int slot, int ks, int i) {
+      const char* stage = lds + slot * C::kStageBytes;
       fa[ks][i] = *reinterpret_cast<const v4i*>(stage + a_foff[ks] + i * kB * kBK);
     };
-    auto read_b = [&](int kt, int ks, int j) {
-      const char* stage = lds + (kt % C::kStages) * C::kStageBytes;
+    auto read_b = [&](int slot, int ks, int j) {
+      const char* stage = lds + slot * C::kStageBytes;
       fb[ks][j] = *reinterpret_cast<const v4i*>(stage + b_foff[ks] + j * kB * kBK);
     };
 #pragma unroll
@@ -841,7 +843,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     const int tail_k[2] = {a_k[0], a_k[1]};
     auto issue_tail = [&](int kt_load, auto is_b, int l) {
       const int kbase = phys(kt_load) * kBK;
-      const uint32_t stage = lds_base + (kt_load % C::kStages) * C::kStageBytes;
+      const uint32_t stage = lds_base + (uint32_t(kt_load) & (C::kStages - 1)) * C::kStageBytes;
       const uint32_t goff = decltype(is_b)::value ? b_goff[l] : a_goff[l];
       const uint32_t off = kbase + tail_k[l & 1] < K ? goff + kbase : kOutOfRange;
       LoadToLds16(stage + (decltype(is_b)::value ? C::kBM * kBK : 0) + (wave * C::kALoads + l) * 1024, off,
@@ -903,15 +905,15 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           Traits::Mma(fa[ks][i], fb[ks][j], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         // The last four columns of this step's first half (needed from instruction 32 on).
-        if constexpr (n < 16 && n % 2 == 0) read_b(kt, n / 2 % 2, PairedColumnAt(kParity, 0, 4 + n / 4));
+        if constexpr (n < 16 && n % 2 == 0) read_b(kParity, n / 2 % 2, PairedColumnAt(kParity, 0, 4 + n / 4));
         // A rows 4-7 of this step.
         if constexpr (n >= kBarrier1 + 1 && n < kBarrier1 + 25 && (n - kBarrier1) % 3 == 1)
-          read_a(kt, (n - kBarrier1 - 1) / 3 % 2, 4 + (n - kBarrier1 - 1) / 6);
+          read_a(kParity, (n - kBarrier1 - 1) / 3 % 2, 4 + (n - kBarrier1 - 1) / 6);
         // A rows 0-3 of the next step.
-        if constexpr (n >= 65 && n < 81 && n % 2 == 1) read_a(kt + 1, (n - 65) / 2 % 2, (n - 65) / 4);
+        if constexpr (n >= 65 && n < 81 && n % 2 == 1) read_a(kParity ^ 1, (n - 65) / 2 % 2, (n - 65) / 4);
         // The first four columns of the second half, as they come free.
         if constexpr (n >= 72 && n < 104 && (n % 8 == 0 || n % 8 == 2))
-          read_b(kt + 1, n % 8 / 2, PairedColumnAt(kParity, 1, (n - 72) / 8));
+          read_b(kParity ^ 1, n % 8 / 2, PairedColumnAt(kParity, 1, (n - 72) / 8));
         // The loads of ring step kt + 2: B behind barrier 1, A behind barrier 2.
         // Inside the depth the LDS address goes to M0 behind the instruction before.
         constexpr bool kLoadB = n >= kLoadB0 && n < 64 && (n - kLoadB0) % kLoadBStride == 0;
@@ -1050,46 +1052,6 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     if (kt < k_tiles) {
       paired_step(kt, Odd(), std::false_type(), std::false_type());
       between(kt + 1);
-    }
-    if constexpr (kRowSums) {
-      Traits::DrainMma();
-      WaitVmcnt<0>();
-      const int first_row = m0 + wave_m * (WM * 32);
-      const long long* fetched =
-          reinterpret_cast<const long long*>(lds + kSumsArea + wave * Traits::kParamInts * 4);
-      long long word[2] = {fetched[lane], fetched[64 + lane]};
-      bool ready = !args.row_sums_fetch_late &&
-                   __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
-                         fused_sums::ContributionsIn(word[1]) == share.expected);
-      // Not complete when they were asked for: look again, a bounded number
-      // of times. Contributors that never got to run (a device shared with
-      // somebody else's work) must not be waited for without end: then this
-      // wave forms the sums of its rows itself, from global memory.
-      for (int spins = 0; !ready && spins < args.row_sums_spin_limit; ++spins) {
-        if (spins) __builtin_amdgcn_s_sleep(8);
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-          word[h] = __hip_atomic_load(args.row_sums + first_row + 64 * h + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ready = __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
-                      fused_sums::ContributionsIn(word[1]) == share.expected);
-      }
-      if (ready) {
-        edge.sums[0] = fused_sums::SumIn(word[0]);
-        edge.sums[1] = fused_sums::SumIn(word[1]);
-      } else {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int row = min(first_row + 64 * h + lane, args.M - 1);
-          const char* from = static_cast<const char*>(args.a) + size_t(row) * size_t(args.lda);
-          int sum = 0;
-          for (int k = 0; k < K; k += kGranule) {
-            const v4i x = *reinterpret_cast<const v4i*>(from + k);
-#pragma unroll
-            for (int d = 0; d < 4; ++d) sum = __builtin_amdgcn_sdot4(x[d], 0x01010101, sum, false);
-          }
-          edge.sums[h] = sum;
-        }
-      }
     }
   } else {
     Frags f[2];
@@ -1268,6 +1230,45 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // The wave's parameter area (behind the ring): written and read by this
     // wave only, and LDS operations of a wave complete in order.
     int* const area = reinterpret_cast<int*>(lds + C::kStages * C::kStageBytes) + wave * Traits::kParamInts;
+    // kRowSums: the sums of this wave's rows, two rows a lane, complete or not.
+    if constexpr (kRowSums) {
+      const int first_row = m0 + wave_m * (WM * 32);
+      // (Fetched into this wave's parameter area while the last ring steps ran.)
+      const long long* fetched = reinterpret_cast<const long long*>(area);
+      long long word[2] = {fetched[lane], fetched[64 + lane]};
+      bool ready = !args.row_sums_fetch_late &&
+                   __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
+                         fused_sums::ContributionsIn(word[1]) == share.expected);
+      // Not complete when they were asked for: look again, a bounded number
+      // of times. Contributors that never got to run (a device shared with
+      // somebody else's work) must not be waited for without end: then this
+      // wave forms the sums of its rows itself, from global memory.
+      for (int spins = 0; !ready && spins < args.row_sums_spin_limit; ++spins) {
+        if (spins) __builtin_amdgcn_s_sleep(8);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          word[h] = __hip_atomic_load(args.row_sums + first_row + 64 * h + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ready = __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
+                      fused_sums::ContributionsIn(word[1]) == share.expected);
+      }
+      if (ready) {
+        edge.sums[0] = fused_sums::SumIn(word[0]);
+        edge.sums[1] = fused_sums::SumIn(word[1]);
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int row = min(first_row + 64 * h + lane, args.M - 1);
+          const char* from = static_cast<const char*>(args.a) + size_t(row) * size_t(args.lda);
+          int sum = 0;
+          for (int k = 0; k < K; k += kGranule) {
+            const v4i x = *reinterpret_cast<const v4i*>(from + k);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) sum = __builtin_amdgcn_sdot4(x[d], 0x01010101, sum, false);
+          }
+          edge.sums[h] = sum;
+        }
+      }
+    }
     Traits::Stage(ep, edge, area, lane);
     const int col0 = n0 + wave_n * (WN * 32) + (lane & 15);
     // reg k of lane row q  <->  reg q of lane row k (lane rows: 16 lanes each).

@@ -397,8 +397,11 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     args.row_sums_zero_rows = ctx->row_sums_dirty_rows[set ^ 1];
     args.row_sums_spin_limit = ctx->row_sums_spin_limit;
     args.row_sums_fetch_late = ctx->row_sums_fetch_late;
-    args.row_sums_first_is_zero = fused_sums::FirstContributorIsZero(
-        (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows, (args.N + fused_sums::kTileRows - 1) / fused_sums::kTileRows);
+    const int tiles_m = (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
+    const int tiles_n = (args.N + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
+    if (fused_sums::FirstContributorIsZero(tiles_m, tiles_n))
+      args.row_sums_uniform_run = fused_sums::StepsPerWave(
+          (args.k_bytes + 127) / 128, std::min(tiles_n, fused_sums::kMaxContributorTiles));
     kernel_a.sums_pending = false;
     row_sums_in_launch = true;
   }

@@ -200,7 +200,8 @@ static void CheckRowSumShares(int tiles_m, int tiles_n, int depth_steps) {
         EXPECT(s.contributes == (n >= c.first_tile_n && n < c.first_tile_n + c.count));
         // The same with the hint that saves the search for the contributors.
         if (fs::FirstContributorIsZero(tiles_m, tiles_n)) {
-          const fs::WaveShare h = fs::ShareOfWave(tiles_m, tiles_n, tile_m, n, wave_n, depth_steps, true);
+          const int run = fs::StepsPerWave(depth_steps, tiles_n < fs::kMaxContributorTiles ? tiles_n : fs::kMaxContributorTiles);
+          const fs::WaveShare h = fs::ShareOfWave(tiles_m, tiles_n, tile_m, n, wave_n, depth_steps, run);
           EXPECT(h.contributes == s.contributes && h.first_step == s.first_step && h.end_step == s.end_step &&
                  h.expected == s.expected);
         }
