@@ -268,6 +268,15 @@ RUYAMD_API int ruyamd_ctx_last_kernel(const ruyamd_ctx* ctx);
  * role of ruy's kInternalStandardCppVariant paths, ruy/kernel.h:150-169). */
 RUYAMD_API void ruyamd_ctx_force_generic_kernel(ruyamd_ctx* ctx, int force);
 
+/* Makes the tiled matrix-core kernels run on the tile of tile_rows x
+ * tile_cols destination elements (256x256, 128x128, 128x64, 64x128 or 64x64;
+ * plane columns count for int8 x int16) instead of the one their timing model
+ * picks, where the kernel has that tile; 0, 0 restores the model's choice.
+ * For tests that must reach a particular tile whatever the model was last
+ * fitted to, and for measuring every tile on one shape. No counterpart in the
+ * reference (its kernel shape is fixed per path, ruy/kernel_x86.h:62-90). */
+RUYAMD_API int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_cols);
+
 /* Operand sums formed inside the launch of the largest int8 tile (no
  * counterpart in the reference, whose Pack forms them in the pass that already
  * touches the data, ruy/pack.h:105-132). On by default: a large 8-bit product

@@ -417,6 +417,13 @@ void ruyamd_ctx_set_cache_max_bytes(ruyamd_ctx* ctx, int64_t max_bytes) {
   ctx->cache->SetMaxBuffersBytes(static_cast<std::ptrdiff_t>(max_bytes));
 }
 
+int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_cols) {
+  if (!ctx || tile_rows < 0 || tile_cols < 0) return RUYAMD_E_INVALID;
+  ctx->forced_tile_rows = tile_rows;
+  ctx->forced_tile_cols = tile_cols;
+  return RUYAMD_OK;
+}
+
 int ruyamd_ctx_set_sums_in_launch(ruyamd_ctx* ctx, int enable, int spin_limit) {
   if (!ctx) return RUYAMD_E_INVALID;
   ctx->row_sums_in_launch = enable != 0;

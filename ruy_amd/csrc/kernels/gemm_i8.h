@@ -85,6 +85,11 @@ struct GemmArgs {
   // many depth steps (fused_sums::StepsPerWave): the kernel need not work
   // either out.
   int32_t row_sums_uniform_run = 0;
+  // Diagnostics/tests: not 0 = run on the tile of (forced_tile_rows x
+  // forced_tile_cols) whatever the timing model says, if the kernel has it.
+  int32_t forced_tile_rows = 0;
+  int32_t forced_tile_cols = 0;
+  int32_t unused_padding_2 = 0;
 };
 
 // Buffers of the products of a batched launch (GemmArgs holds what they have

@@ -227,11 +227,23 @@ struct Int8Traits16 : Int8Traits {
   // Which form of the arithmetic a launch needs, decided once so that the
   // write-back loops carry no branches on it: a lone wave pays for every
   // branch with an empty instruction buffer.
-  enum FinishMode { kRaw = 0, kScalarHigh, kScalar, kPerRow, kPerColumn, kFinishModes };
+  enum FinishMode { kRaw = 0, kScalarHighMerged, kScalarHigh, kScalar, kPerRow, kPerColumn, kFinishModes };
+  // kScalarHighMerged: RequantHigh with the destination zero point folded into
+  // its rounding term, (hi + 2^(s-1) + zp * 2^s) >> s, one addition less per
+  // value. The same number as ((hi + 2^(s-1)) >> s) + zp as long as the sum
+  // cannot leave 32 bits: hi lies in [-2^30, 2^30) (a 32-bit value times a
+  // multiplier below 2^31, high word), so that is asked of the rest.
+  static __device__ __forceinline__ bool CanMergeZeroPoint(const Epilogue& ep) {
+    const int s = -1 - ep.mult_exponent_scalar;
+    if (s < 1 || s > 30) return false;
+    const long long zp = ep.dst_zero_point < 0 ? -static_cast<long long>(ep.dst_zero_point) : ep.dst_zero_point;
+    return (zp << s) + (1ll << (s - 1)) < (1ll << 30);
+  }
   static __device__ __forceinline__ int ModeOf(const Epilogue& ep) {
     if (!ep.requantize) return kRaw;
     if (ep.mult_fixedpoint) return ep.channel_is_col ? kPerColumn : kPerRow;
-    return ep.mult_exponent_scalar <= -2 ? kScalarHigh : kScalar;
+    if (ep.mult_exponent_scalar > -2) return kScalar;
+    return CanMergeZeroPoint(ep) ? kScalarHighMerged : kScalarHigh;
   }
   struct RowParams {
     v4i add[4], m[4], e[4];
@@ -270,7 +282,16 @@ struct Int8Traits16 : Int8Traits {
     for (int q = 0; q < 16; ++q)
       vals[q] = static_cast<int32_t>(static_cast<uint32_t>(vals[q]) + static_cast<uint32_t>(r.add[q / 4][q % 4]) +
                                      static_cast<uint32_t>(c.add));
-    if constexpr (kMode == kScalarHigh) {
+    if constexpr (kMode == kScalarHighMerged) {
+      const int32_t m = ep.mult_fixedpoint_scalar;
+      const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
+      const int32_t rounding_and_zero_point =
+          (1 << (high_shift - 1)) + static_cast<int32_t>(static_cast<uint32_t>(ep.dst_zero_point) << high_shift);
+#pragma unroll
+      for (int q = 0; q < 16; ++q)
+        vals[q] = Median3((__mulhi(vals[q], m) + rounding_and_zero_point) >> high_shift, ep.clamp_min_i, ep.clamp_max_i);
+      return;
+    } else if constexpr (kMode == kScalarHigh) {
       const int32_t m = ep.mult_fixedpoint_scalar;
       const int high_shift = -1 - ep.mult_exponent_scalar;  // (31 - e) - 32
 #pragma unroll

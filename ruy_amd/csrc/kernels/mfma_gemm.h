@@ -1321,16 +1321,22 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         // rows 4k .. 4k+3 of the lane's block. Every lane takes part in the
         // swaps; columns and rows past the end are left out when storing.
         int w[kElt][4];
+        // (The values lie inside the destination type's range by now, so the
+        // saturation of v_cvt_pk_i16_i32 does nothing: it is the two-in-one
+        // instruction that puts a pair into one register.)
         if constexpr (kElt == 1) {
 #pragma unroll
-          for (int b = 0; b < 4; ++b)
-            w[0][b] = (vals[4 * b] & 0xff) | ((vals[4 * b + 1] & 0xff) << 8) | ((vals[4 * b + 2] & 0xff) << 16) |
-                      (vals[4 * b + 3] << 24);
+          for (int b = 0; b < 4; ++b) {
+            const auto low = __builtin_amdgcn_cvt_pk_i16(vals[4 * b], vals[4 * b + 1]);
+            const auto high = __builtin_amdgcn_cvt_pk_i16(vals[4 * b + 2], vals[4 * b + 3]);
+            // The low bytes of the four 16-bit halves.
+            w[0][b] = __builtin_amdgcn_perm(__builtin_bit_cast(int, high), __builtin_bit_cast(int, low), 0x06040200);
+          }
         } else if constexpr (kElt == 2) {
 #pragma unroll
           for (int b = 0; b < 4; ++b) {
-            w[0][b] = (vals[4 * b] & 0xffff) | (vals[4 * b + 1] << 16);
-            w[1][b] = (vals[4 * b + 2] & 0xffff) | (vals[4 * b + 3] << 16);
+            w[0][b] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(vals[4 * b], vals[4 * b + 1]));
+            w[1][b] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(vals[4 * b + 2], vals[4 * b + 3]));
           }
         } else {
 #pragma unroll
@@ -1796,6 +1802,9 @@ inline bool ShallowRing(const GemmArgs& args, int num_cus, int bm, int bn) {
 
 inline Tile PickTile(const GemmArgs& args, int num_cus, Model which) {
   const TimingModel model = TimingModelOf(which);
+  for (int i = 0; i < model.count; ++i)
+    if (model.tiles[i].bm == args.forced_tile_rows && model.tiles[i].bn == args.forced_tile_cols)
+      return model.tiles[i].tile;
   Tile best = model.tiles[0].tile;
   double best_time = ModelledMicroseconds(args, num_cus, model, model.tiles[0]);
   for (int i = 1; i < model.count; ++i) {

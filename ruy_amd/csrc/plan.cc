@@ -273,6 +273,8 @@ void PlanDepthSplit(ruyamd_ctx* ctx, GemmKind kind, GemmArgs* args) {
 bool SetupInt8Gemm(ruyamd_ctx* ctx, const MulCall& call, const Operand8& a, const Operand8& b, int32_t lzp,
                    int32_t rzp, GemmArgs* out) {
   GemmArgs& args = *out;
+  args.forced_tile_rows = ctx->forced_tile_rows;
+  args.forced_tile_cols = ctx->forced_tile_cols;
   const int M = call.lhs.rows, K = call.lhs.cols, N = call.rhs.cols;
   args.k_bytes = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
   const bool swap = SetupDestination(call, &args);
@@ -607,6 +609,8 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     return RUYAMD_OK;
   }
   GemmArgs args;
+  args.forced_tile_rows = ctx->forced_tile_rows;
+  args.forced_tile_cols = ctx->forced_tile_cols;
   args.k_bytes = RoundUp(K, 4) * 4;
   const bool swap = SetupDestination(*call, &args);
   const OperandF32& x = swap ? b : a;
@@ -637,6 +641,8 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
 int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
   GemmArgs args;
+  args.forced_tile_rows = ctx->forced_tile_rows;
+  args.forced_tile_cols = ctx->forced_tile_cols;
   const bool swap = SetupDestination(*call, &args);  // true: A side = rhs
   const int side8 = swap ? 1 : 0;
   const int side16 = 1 - side8;
@@ -795,6 +801,8 @@ int RunMulBatch(ruyamd_ctx* ctx, const MulCall& first, const BatchBuffers* items
   if (M <= kSkinnyKernelWidth || N <= kSkinnyKernelWidth || K <= 0) return RUYAMD_OK;
   if (ShouldCache(first.lhs_cache_policy, N) || ShouldCache(first.rhs_cache_policy, M)) return RUYAMD_OK;
   GemmArgs shape;
+  shape.forced_tile_rows = ctx->forced_tile_rows;
+  shape.forced_tile_cols = ctx->forced_tile_cols;
   shape.M = M;
   shape.N = N;
   shape.k_bytes = RoundUp(K, 16);  // the depth the launcher will see: both must pick the same tile

@@ -27,6 +27,11 @@ def announce(*what):
     sys.stdout.flush()
 
 
+def api_tile(M, K, N):
+    from ruy_amd import api
+    return api.tile_for(0, M, K, N)
+
+
 def compare(problem, got, want, exact_fp=False):
     if problem.dst.dtype in (S.F32, S.F64) and not exact_fp:
         g = O.dense_of(problem, got).astype(np.float64)
@@ -857,6 +862,59 @@ def test_grids_with_a_small_last_round(device_ctx, shape, tup):
         assert ((got.sum(axis=1) % 2**32) == (L @ R.sum(axis=1)) % 2**32).all()
 
 
+@pytest.mark.parametrize("dst_dtype", [S.I8, S.U8, S.I16], ids=lambda d: S.NUMPY_NAMES[d] if hasattr(S, "NUMPY_NAMES") else str(d))
+def test_largest_tile_requantization_corner_cases(device_ctx, dst_dtype):
+    """The write-back of the 256x256 tile has a form of its own for a scalar
+    multiplier with an exponent of -2 or less (the high word of the product,
+    rounded and shifted), in which the destination zero point rides on the
+    rounding term where that cannot overflow, and falls back to the separate
+    addition or to the 64-bit form otherwise: exponents on both sides of every
+    switch (-1, -2, -8, -15, -22, -23, -24, -31), zero points at both ends of the
+    destination type and in the middle, a bias that takes the accumulators over
+    the whole 32-bit range (where the exponent lets them through: results at
+    the clamps and between them), narrowed clamp bounds, multipliers at both ends of [2^30, 2^31). Every element against the
+    checker (the depth is short enough for it)."""
+    from ruy_amd import device_problem as D
+    rng = np.random.default_rng(515 + dst_dtype)
+    lo, hi = S.INT_RANGES[dst_dtype]
+    M, K, N = 4096, 32, 4096
+    device_ctx.force_tile(256, 256)  # (the timing model would put so short a depth on a smaller tile)
+    try:
+        _requantization_corner_cases(device_ctx, rng, dst_dtype, M, K, N, lo, hi)
+    finally:
+        device_ctx.force_tile(0, 0)
+
+
+def _requantization_corner_cases(device_ctx, rng, dst_dtype, M, K, N, lo, hi):
+    from ruy_amd import device_problem as D
+    for exponent, zero_point, multiplier, narrow in [
+            (-1, lo, 1 << 30, False), (-2, hi, (1 << 31) - 1, False), (-8, (lo + hi) // 2, 1395864371, True),
+            (-15, hi, 1518500250, False), (-22, lo, (1 << 31) - 1, False), (-23, hi, 1 << 30, True),
+            (-24, lo, 1234567891, False), (-31, hi, (1 << 31) - 1, False), (-10, lo, 1 << 30, True)]:
+        lhs = W.HostMatrix(S.I8, M, K, S.ORDER_ROW_MAJOR, zero_point=0)
+        lhs.storage[:] = rng.integers(-127, 128, lhs.storage.size).astype(np.int8)
+        rhs = W.HostMatrix(S.I8, K, N, S.ORDER_COL_MAJOR, zero_point=-3)
+        rhs.storage[:] = rng.integers(-128, 128, rhs.storage.size).astype(np.int8)
+        dst = W.HostMatrix(dst_dtype, M, N, S.ORDER_COL_MAJOR, zero_point=zero_point)
+        # Accumulators all over the 32-bit range: what reaches the destination type's
+        # range after the shift depends on the exponent, so the bias is scaled to it.
+        spread = min(2**31 - 2**20, (hi - lo + 64) << (-exponent))
+        bias = rng.integers(-spread, spread + 1, M).astype(np.int32)
+        bias[:8] = [2**31 - 2**20, -(2**31 - 2**20), 0, 1, -1, spread, -spread, spread // 2]
+        cmin, cmax = (lo + (hi - lo) // 5, hi - (hi - lo) // 7) if narrow else (lo, hi)
+        p = W.Problem("requant e=%d zp=%d m=%d %s" % (exponent, zero_point, multiplier, S.NUMPY_NAMES[dst_dtype]),
+                      lhs, rhs, dst, S.I32, bias=bias, multiplier_fixedpoint=multiplier,
+                      multiplier_exponent=exponent, clamp_min=cmin, clamp_max=cmax,
+                      channel_dimension=S.CHANNEL_ROW)
+        announce(p.name)
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        assert device_ctx.last_kernel_name() == "i8_mfma"
+        want = O.oracle_mul(p)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "%s: %d of %d elements differ, first at %d: got %r want %r" % (
+            p.name, bad.size, got.size, bad[0], got[bad[0]], want[bad[0]])
+
+
 @pytest.mark.parametrize("mode", ["ahead", "late", "own", "separate"])
 def test_operand_sums_formed_inside_the_launch(mode):
     """The 256x256 tile of the int8 kernel forms the depth sums of its `a`
@@ -935,6 +993,15 @@ def test_largest_tile_over_depth_step_counts(device_ctx, tup):
     columns either side of every tile edge otherwise and in any case."""
     from ruy_amd import device_problem as D
     rng = np.random.default_rng(4242 + tup[3])
+    device_ctx.force_tile(256, 256)  # (the timing model puts the shortest of these depths on smaller tiles)
+    try:
+        _largest_tile_depth_step_counts(device_ctx, rng, tup)
+    finally:
+        device_ctx.force_tile(0, 0)
+
+
+def _largest_tile_depth_step_counts(device_ctx, rng, tup):
+    from ruy_amd import device_problem as D
     for K, M, N, misalign in [(16, 4096, 4096, 0), (112, 4096, 4096, 0), (128, 4000, 4090, 0), (144, 4096, 4096, 0),
                               (256, 4096, 3900, 0), (300, 4096, 4096, 0), (384, 4096, 4096, 0), (500, 3850, 4096, 0),
                               (640, 4096, 4096, 0), (896, 4096, 4096, 0), (256, 3001, 4096, 3), (128, 4095, 3003, 1)]:
