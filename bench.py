@@ -442,7 +442,7 @@ def bench_gemv(ctx, args):
         entry = {"run": label, "N": cols, "kernel": kernel_wider, "ms_per_step": tw["step_s"] * 1e3,
                  "ms_per_step_min": tw["step_min_s"] * 1e3, "algorithmic_bytes": nbytes_w,
                  "roofline": hbm_roofline(nbytes_w, tw["region_ms"],
-                                          None if kw.get("requant") else load_traffic("int8_gemv_%d_n%d" % (n, cols)))}
+                                          load_traffic("int8_gemv_%d_n%d%s" % (n, cols, "_requant" if kw.get("requant") else "")))}
         if not args.no_cpu_baseline:
             entry["cpu_baseline"] = cpu_baseline(
                 wider[0].problem, nbytes_w, "GB/s",

@@ -56,7 +56,7 @@ namespace fused_sums {
 constexpr int kTileRows = 256;          // of the tile that forms sums this way
 constexpr int kMaxRows = 65536;         // rows of `a` a launch may have
 constexpr int kMaxContributorTiles = 8;
-constexpr int kMinDepthSteps = 16;      // fewer ring steps than this: not worth it
+constexpr int kMinDepthSteps = 8;       // fewer ring steps than this: not worth it
 constexpr int kBandRows = 4;            // tile rows per band of the kernel's tile order
 constexpr int kXcds = 8;
 

@@ -920,8 +920,8 @@ def test_operand_sums_formed_inside_the_launch(mode):
     """The 256x256 tile of the int8 kernel forms the depth sums of its `a`
     operand's rows in passing, dealt out over the first workgroups of every
     tile row (one launch where a sums kernel used to run in front). Shapes:
-    one round of tiles at the shortest depth that takes this route; ragged
-    edges with a depth of 17 steps and a bit; grids whose bands of four tile rows begin in the middle of an XCD's
+    one round of tiles at a short depth; ragged edges with a depth of 17 steps
+    and a bit; grids whose bands of four tile rows begin in the middle of an XCD's
     queue (10 x 20 and 11 x 16 tiles), a last band of two tile rows; both
     destination orders (the row-major one swaps the operands, so the sums are
     then those of the right-hand side); zero points that need the sums of both
@@ -945,7 +945,7 @@ def test_operand_sums_formed_inside_the_launch(mode):
         expected_calls = 0
         for (M, K, N), orders in [((4096, 2048, 4096), cases.RCC), ((4000, 2192, 3900), (1, 0, 1)),
                                   ((2560, 2048, 5120), cases.RCC), ((4096, 2048, 2816), (1, 0, 1)),
-                                  ((3072, 4096, 3072), cases.RCC)]:
+                                  ((3072, 4096, 3072), cases.RCC), ((4096, 1024, 4096), cases.RCC)]:
             p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
                                  name="%s %s %s %s" % (cases.tuple_name(tup), (M, K, N), orders, mode))
             p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
