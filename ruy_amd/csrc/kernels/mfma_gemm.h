@@ -54,6 +54,7 @@
 #include "depth_split.h"
 #include "fused_sums.h"
 #include "gemm_i8.h"
+#include "paired_schedule.h"
 
 namespace ruyamd {
 namespace mfma_gemm {
@@ -169,10 +170,6 @@ template <int BK>
 __device__ __forceinline__ int LdsOffset(int r, int g) {
   return r * BK + ((g ^ Swizzle<BK>(r)) << 4);
 }
-
-// The paired schedule of the largest int8 tile (see the kernel): the block
-// column (of eight) at position `cp` of half `h` of a ring step of the given parity.
-constexpr int PairedColumnAt(int parity, int h, int cp) { return (parity ^ h) == 0 ? cp : 7 - cp; }
 
 template <int WM, int WN, int BK, int STAGES, bool SPLIT_B = false, int BLOCK = 32>
 struct Cfg {
@@ -795,12 +792,13 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     //     next ring step. The first four are read as they come free, the last
     //     four during the first instructions of the next ring step.
     // Ring: two slots. The B half of slot kt % 2 has been read by every wave
-    // once the "last four" reads of step kt are done (barrier 1, in front of
-    // instruction 16), the A half once rows 4-7 have been read (barrier 2, in
-    // front of instruction 64); the loads of step kt + 2 follow each barrier,
-    // one every sixth instruction. Barrier 2 is also where every wave has waited
-    // for all its loads but the eight just issued, i.e. for everything of step
-    // kt + 1, which the second half starts to read.
+    // once the "last four" reads of step kt are done (barrier 1), the A half
+    // once rows 4-7 have been read (barrier 2, in front of the second half);
+    // the loads of step kt + 2 follow each barrier, one every fifth or sixth
+    // instruction. Barrier 2 is also where every wave has waited for all its
+    // loads but the eight just issued, i.e. for everything of step kt + 1,
+    // which the second half starts to read. The instruction numbers of all of
+    // this are in paired_schedule.h.
     static_assert(kB == 16 && C::kKSteps == 2 && C::kStages == 2 && kAB == 8 && kBB == 8 && C::kALoads == 8 &&
                       C::kBLoads == 8 && !kFusedSums,
                   "the paired schedule is written for the 256x256 tile of 16x16 blocks");
@@ -824,17 +822,17 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       for (int l = 0; l < C::kALoads; ++l) issue_one(st, l);
     }
     load_edge_params();
-    WaitVmcnt<C::kALoads + C::kBLoads>();
+    WaitVmcnt<paired_schedule::kLoadsLeftBeforeFirstStep>();
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < kAB / 2; ++i) {
+    for (int i = 0; i < paired_schedule::kRowsReadAhead; ++i) {
       read_a(0, 0, i);
       read_a(0, 1, i);
     }
 #pragma unroll
-    for (int cp = 0; cp < kBB / 2; ++cp) {
-      read_b(0, 0, cp);
-      read_b(0, 1, cp);
+    for (int cp = 0; cp < paired_schedule::kColumnsReadAhead; ++cp) {
+      read_b(0, 0, paired_schedule::ColumnAt(0, 0, cp));
+      read_b(0, 1, paired_schedule::ColumnAt(0, 0, cp));
     }
     // The bounds-tested form of a load for the last ring steps. The depth
     // granule a lane fetches (after the swizzle) depends on the parity of the
@@ -849,29 +847,32 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       LoadToLds16(stage + (decltype(is_b)::value ? C::kBM * kBK : 0) + (wave * C::kALoads + l) * 1024, off,
                   decltype(is_b)::value ? b_rsrc : a_rsrc);
     };
-    // Barrier 1 stands in front of this instruction; the eight B loads follow it.
-    constexpr int kBarrier1 = 24, kLoadB0 = 26, kLoadBStride = 5;
-    static_assert(kLoadB0 > kBarrier1 && kLoadB0 + 7 * kLoadBStride < 64, "");
     // Where this wave's eight loads of an operand go inside a ring slot's half.
     const uint32_t wave_targets = lds_base + wave * C::kALoads * 1024;
+    // One ring step. Which block and fragments instruction n uses, what is read
+    // and loaded behind it and where the barriers stand is the arithmetic of
+    // paired_schedule.h, which a host-side model of the ring checks for
+    // fragments overwritten too early and ring slots refilled before every
+    // wave has read them.
+    namespace ps = paired_schedule;
+    static_assert(ps::kBlocks == kAB && ps::kBlocks == kBB && ps::kInstructions == 2 * kAB * kBB &&
+                      ps::kLoads == C::kALoads && ps::kLoads == C::kBLoads && ps::kRowsPerLoad == C::kRowsPerLoad &&
+                      ps::kRowsPerBlock == kB && ps::kBlocks * ps::kRowsPerBlock == WM * 32 && WM == WN &&
+                      ps::kWaves * ps::kLoads * ps::kRowsPerLoad == C::kBM && C::kBM == C::kBN,
+                  "");
     auto paired_step = [&](int kt, auto parity_constant, auto full, auto first) {
       constexpr int kParity = decltype(parity_constant)::value;  // of kt, hence the ring slot
       // The depth offset of the loads of step kt + 2 (inside the depth): held
       // in one scalar register for the whole step.
       uint32_t refill_offset = uint32_t(phys(kt + C::kStages)) * kBK;
       if constexpr (decltype(full)::value) asm volatile("" : "+s"(refill_offset));
-      StaticFor<2 * kMmas>([&](auto n_constant) {
+      StaticFor<ps::kInstructions>([&](auto n_constant) {
         constexpr int n = decltype(n_constant)::value;
-        constexpr int pair = n / 2;
-        constexpr int ks = n % 2;
-        constexpr int h = pair / 32;
-        constexpr int cp = (pair % 32) / 4;
-        constexpr int rp = pair % 4;
-        constexpr int j = PairedColumnAt(kParity, h, cp);
-        constexpr int i = 4 * h + (cp % 2 == 0 ? rp : 3 - rp);
-        if constexpr (n == kBarrier1) __syncthreads();
-        if constexpr (n == 64) {
-          WaitVmcnt<8>();
+        constexpr ps::Mma mma = ps::MmaAt(kParity, n);
+        constexpr int ks = mma.half, i = mma.row, j = mma.col;
+        if constexpr (n == ps::kTiming.barrier1) __syncthreads();
+        if constexpr (n == ps::kTiming.barrier2) {
+          WaitVmcnt<ps::kTiming.loads_left_at_barrier2>();
           __syncthreads();
         }
         // uint8 data in place: a fragment is flipped where the step first uses
@@ -881,11 +882,11 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         // flipped ahead of the pair: nothing may write an operand of a pair's
         // second matrix instruction once the first is issued (Int8Traits16).
         if constexpr (kFlip && ks == 0) {
-          if constexpr (cp == 0) {
+          if constexpr (mma.first_use_of_a) {
             fa[0][i] ^= static_cast<int>(args.a_flip);
             fa[1][i] ^= static_cast<int>(args.a_flip);
           }
-          if constexpr (h == 0 && rp == 0) {
+          if constexpr (mma.first_use_of_b) {
             fb[0][j] ^= static_cast<int>(args.b_flip);
             fb[1][j] ^= static_cast<int>(args.b_flip);
           }
@@ -893,7 +894,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           // hazard checks do not see: the distance between the last write of
           // an operand and the pair is kept here, by hand, whatever order the
           // compiler gives the flips above (five wait states).
-          if constexpr (cp == 0 || (h == 0 && rp == 0)) {
+          if constexpr (mma.first_use_of_a || mma.first_use_of_b) {
             __builtin_amdgcn_sched_barrier(0);
             asm volatile("s_nop 4" ::: "memory");
           }
@@ -904,32 +905,29 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         else
           Traits::Mma(fa[ks][i], fb[ks][j], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
-        // The last four columns of this step's first half (needed from instruction 32 on).
-        if constexpr (n < 16 && n % 2 == 0) read_b(kParity, n / 2 % 2, PairedColumnAt(kParity, 0, 4 + n / 4));
-        // A rows 4-7 of this step.
-        if constexpr (n >= kBarrier1 + 1 && n < kBarrier1 + 25 && (n - kBarrier1) % 3 == 1)
-          read_a(kParity, (n - kBarrier1 - 1) / 3 % 2, 4 + (n - kBarrier1 - 1) / 6);
-        // A rows 0-3 of the next step.
-        if constexpr (n >= 65 && n < 81 && n % 2 == 1) read_a(kParity ^ 1, (n - 65) / 2 % 2, (n - 65) / 4);
-        // The first four columns of the second half, as they come free.
-        if constexpr (n >= 72 && n < 104 && (n % 8 == 0 || n % 8 == 2))
-          read_b(kParity ^ 1, n % 8 / 2, PairedColumnAt(kParity, 1, (n - 72) / 8));
+        // The fragment that is read behind this instruction, if any: from this
+        // step's ring slot or from the other one (the step to come).
+        constexpr ps::Read read = ps::ReadBehind(kParity, n);
+        if constexpr (read.valid) {
+          constexpr int slot = read.of_next_step ? kParity ^ 1 : kParity;
+          if constexpr (read.is_a)
+            read_a(slot, read.half, read.index);
+          else
+            read_b(slot, read.half, read.index);
+        }
         // The loads of ring step kt + 2: B behind barrier 1, A behind barrier 2.
         // Inside the depth the LDS address goes to M0 behind the instruction before.
-        constexpr bool kLoadB = n >= kLoadB0 && n < 64 && (n - kLoadB0) % kLoadBStride == 0;
-        constexpr bool kLoadA = n >= 66 && n < 112 && (n - 66) % 6 == 0;
-        constexpr bool kTargetB = n + 1 >= kLoadB0 && n + 1 < 64 && (n + 1 - kLoadB0) % kLoadBStride == 0;
-        constexpr bool kTargetA = n + 1 >= 66 && n + 1 < 112 && (n + 1 - 66) % 6 == 0;
-        if constexpr (decltype(full)::value && (kTargetA || kTargetB)) {
-          constexpr int l = kTargetB ? (n + 1 - kLoadB0) / kLoadBStride : (n + 1 - 66) / 6;
-          SetLdsTargetAt<uint32_t(kParity * C::kStageBytes + (kTargetB ? C::kBM * kBK : 0) + l * 1024)>(wave_targets);
-        }
-        if constexpr (kLoadA || kLoadB) {
-          constexpr int l = kLoadB ? (n - kLoadB0) / kLoadBStride : (n - 66) / 6;
+        constexpr ps::Load target = ps::LoadBehind(n + 1);
+        if constexpr (decltype(full)::value && target.valid)
+          SetLdsTargetAt<uint32_t(kParity * C::kStageBytes + (target.is_b ? C::kBM * kBK : 0) + target.index * 1024)>(
+              wave_targets);
+        constexpr ps::Load load = ps::LoadBehind(n);
+        if constexpr (load.valid) {
           if constexpr (decltype(full)::value)
-            LoadToLdsTarget16(kLoadB ? b_goff[l] : a_goff[l], refill_offset, kLoadB ? b_rsrc : a_rsrc);
+            LoadToLdsTarget16(load.is_b ? b_goff[load.index] : a_goff[load.index], refill_offset,
+                              load.is_b ? b_rsrc : a_rsrc);
           else
-            issue_tail(kt + C::kStages, std::integral_constant<bool, kLoadB>(), l);
+            issue_tail(kt + C::kStages, std::integral_constant<bool, load.is_b>(), load.index);
         }
       });
       __builtin_amdgcn_sched_barrier(0);

@@ -86,6 +86,19 @@ def test_host_launch_arithmetic():
     assert "all passed" in out
 
 
+def test_ring_schedule_of_the_largest_tile_model():
+    """The positions of the matrix instructions, fragment reads, loads and
+    barriers of the 256x256 int8 tile's ring step (kernels/paired_schedule.h,
+    which the kernel is generated from), run through a host model of registers,
+    LDS and barriers; the model must also refuse a list of altered schedules."""
+    exe = os.path.join(ROOT, "tests", "cpp", "paired_schedule_test")
+    subprocess.check_call(["g++", "-std=c++17", "-I" + os.path.join(ROOT, "ruy_amd", "csrc"),
+                           exe + ".cc", "-o", exe])
+    out = subprocess.check_output([exe]).decode()
+    assert "all passed" in out
+    assert out.count("altered (") >= 12
+
+
 @pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "example")),
                     reason="reference tree not present")
 @pytest.mark.parametrize("std", ["c++14", "c++17"])
