@@ -272,10 +272,16 @@ RUYAMD_API void ruyamd_ctx_force_generic_kernel(ruyamd_ctx* ctx, int force);
  * tile_cols destination elements (256x256, 128x128, 128x64, 64x128 or 64x64;
  * plane columns count for int8 x int16) instead of the one their timing model
  * picks, where the kernel has that tile; 0, 0 restores the model's choice.
- * For tests that must reach a particular tile whatever the model was last
- * fitted to, and for measuring every tile on one shape. No counterpart in the
- * reference (its kernel shape is fixed per path, ruy/kernel_x86.h:62-90). */
-RUYAMD_API int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_cols);
+ * depth_parts, looked at with the 256x256 tile forced on int8 data: not 0 =
+ * split the depth over that many workgroups per tile (2, 4 or 8; 1: over none;
+ * rounded down to what leaves no part without a depth step) instead of what
+ * the model says; negative: that many, and the parts of a tile do not wait for
+ * each other to share the adding up, the last one to arrive does it all (the
+ * path a launch takes whose workgroups do not all run at once). For tests that must reach a particular tile whatever the model was
+ * last fitted to, and for measuring every tile on one shape. No counterpart in
+ * the reference (its kernel shape is fixed per path, ruy/kernel_x86.h:62-90;
+ * its split of the work is MakeBlockMap's, ruy/block_map.cc:339-471). */
+RUYAMD_API int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_cols, int depth_parts);
 
 /* Operand sums formed inside the launch of the largest int8 tile (no
  * counterpart in the reference, whose Pack forms them in the pass that already

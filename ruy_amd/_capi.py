@@ -61,7 +61,7 @@ PROTOTYPES = {
     "ruyamd_apply_multiplier": (C.c_int, [_ctx, C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_int64]),
     "ruyamd_ctx_set_kernel_timing": (C.c_int, [_ctx, C.c_int]),
-    "ruyamd_ctx_force_tile": (C.c_int, [_ctx, C.c_int, C.c_int]),
+    "ruyamd_ctx_force_tile": (C.c_int, [_ctx, C.c_int, C.c_int, C.c_int]),
     "ruyamd_ctx_set_sums_in_launch": (C.c_int, [_ctx, C.c_int, C.c_int]),
     "ruyamd_ctx_sums_in_launch_calls": (C.c_int64, [_ctx]),
     "ruyamd_ctx_kernel_timing": (C.c_int, [_ctx, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),

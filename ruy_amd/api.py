@@ -320,8 +320,8 @@ class Context:
     def force_generic_kernel(self, flag):
         lib.ruyamd_ctx_force_generic_kernel(self._h, int(flag))
 
-    def force_tile(self, tile_rows=0, tile_cols=0):
-        self._check(lib.ruyamd_ctx_force_tile(self._h, int(tile_rows), int(tile_cols)))
+    def force_tile(self, tile_rows=0, tile_cols=0, depth_parts=0):
+        self._check(lib.ruyamd_ctx_force_tile(self._h, int(tile_rows), int(tile_cols), int(depth_parts)))
 
     def set_sums_in_launch(self, enable, spin_limit=-1):
         self._check(lib.ruyamd_ctx_set_sums_in_launch(self._h, int(enable), int(spin_limit)))

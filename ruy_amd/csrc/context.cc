@@ -417,10 +417,12 @@ void ruyamd_ctx_set_cache_max_bytes(ruyamd_ctx* ctx, int64_t max_bytes) {
   ctx->cache->SetMaxBuffersBytes(static_cast<std::ptrdiff_t>(max_bytes));
 }
 
-int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_cols) {
+int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_cols, int depth_parts) {
   if (!ctx || tile_rows < 0 || tile_cols < 0) return RUYAMD_E_INVALID;
   ctx->forced_tile_rows = tile_rows;
   ctx->forced_tile_cols = tile_cols;
+  ctx->forced_depth_parts = depth_parts < 0 ? -depth_parts : depth_parts;
+  ctx->forced_split_without_waiting = depth_parts < 0;
   return RUYAMD_OK;
 }
 

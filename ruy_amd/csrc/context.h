@@ -113,6 +113,8 @@ struct ruyamd_ctx {
   int performance_advisories = 0;
   int last_kernel = RUYAMD_KERNEL_NONE;
   bool force_generic = false;
+  int forced_depth_parts = 0;
+  bool forced_split_without_waiting = false;
   int forced_tile_rows = 0, forced_tile_cols = 0;  // diagnostics: 0 = the timing model picks
   std::string last_error;
   ruyamd::Workspace workspace;         // grows on demand (hipMalloc)

@@ -2,7 +2,7 @@
 // planner and a host-only model test: which depth steps a part walks, when a
 // split has no empty part, and who does the write-back.
 //
-// Protocol (tiled kernels, small tiles only). A launch carries `parts`
+// Protocol (the small tiles; the largest int8 tile adds to it, see below). A launch carries `parts`
 // workgroups per destination tile. Each walks its part of the depth steps,
 // stores its raw accumulators to its slice of a scratch buffer, waits until
 // those stores have been performed, and then adds 1 to the tile's arrival
@@ -67,6 +67,54 @@ RUYAMD_HOST_DEVICE inline int PartsWithoutEmpty(int steps, int wanted) {
 // `previous`: what this workgroup's add on the tile's arrival counter returned.
 RUYAMD_HOST_DEVICE inline bool IsLastArrival(unsigned previous, int parts) {
   return previous == static_cast<unsigned>(parts - 1);
+}
+
+// ---- The split of the largest int8 tile (256x256, 8 x 8 blocks of 16x16 a wave) ----
+//
+// Adding up the parts costs in proportion to the tile's area, and here a part
+// is 256 KiB: one workgroup that reads all the others' parts and then writes
+// the whole tile back is busy for longer than the split saves. So the parts
+// share that work as well. Every workgroup stores its accumulators as above
+// and counts itself in; then it waits, a bounded number of looks at the
+// counter, until all parts of its tile have arrived. The tile's destination
+// columns are dealt to the parts (block columns index * 8 / parts ...: every
+// wave of the workgroup owns those of its 8 block columns): a workgroup that
+// has seen everybody arrive claims its columns (one bit per part in a word of
+// claims, set with an atomic OR whose return value says who was first), adds
+// the other parts' accumulators of those columns to its own and writes those
+// columns back. Parts of a tile take the same time, so the wait is short and
+// all parts read and write side by side.
+//
+// Nobody may wait without bound (the other parts' workgroups may not be
+// running: a device shared with somebody else's kernels, a grid larger than
+// the device). A workgroup whose looks are used up leaves without claiming. The
+// last one to arrive never waits; after its own columns it claims whatever
+// nobody has claimed and finishes those columns too: every part's full set of
+// accumulators is in memory, its own are still in its registers. With a limit
+// of zero looks this is the plain protocol above.
+//
+// Every workgroup counts itself out when it leaves; the last one out sets the
+// tile's three words back to zero (nobody reads them any more).
+constexpr int kLargeWordsPerTile = 4;  // arrivals, claims, exits, one unused
+constexpr int kArrivals = 0, kClaims = 1, kExits = 2;
+constexpr int kLargeBlockColumns = 8;
+constexpr int kLargeMaxParts = 8;
+
+// The parts must deal out the block columns evenly.
+RUYAMD_HOST_DEVICE inline bool LargePartsAllowed(int parts) { return parts == 2 || parts == 4 || parts == 8; }
+// The largest allowed number of parts <= wanted that leaves no part without a
+// depth step (1: no split).
+RUYAMD_HOST_DEVICE inline int LargeParts(int steps, int wanted) {
+  for (int parts = kLargeMaxParts; parts >= 2; parts /= 2)
+    if (parts <= wanted && NoEmptyPart(steps, parts)) return parts;
+  return 1;
+}
+RUYAMD_HOST_DEVICE inline int LargeColumnsPerPart(int parts) { return kLargeBlockColumns / parts; }
+// Whether the claim of part `index` succeeded: `claims_before` is what the
+// atomic OR of ClaimBit(index) into the tile's claims returned.
+RUYAMD_HOST_DEVICE inline unsigned ClaimBit(int index) { return 1u << index; }
+RUYAMD_HOST_DEVICE inline bool ClaimSucceeded(unsigned claims_before, int index) {
+  return (claims_before & ClaimBit(index)) == 0;
 }
 
 }  // namespace depth_split

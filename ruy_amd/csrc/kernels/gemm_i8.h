@@ -89,7 +89,16 @@ struct GemmArgs {
   // forced_tile_cols) whatever the timing model says, if the kernel has it.
   int32_t forced_tile_rows = 0;
   int32_t forced_tile_cols = 0;
-  int32_t unused_padding_2 = 0;
+  // With the 256x256 tile forced: not 0 = split the depth into this many parts
+  // (1: do not split) whatever the timing model says.
+  int32_t forced_depth_parts = 0;
+  // Set with split_k > 1: the split is that of the 256x256 int8 tile (which
+  // the launch then runs on), not of the smallest tile.
+  int32_t split_large = 0;
+  // ... and how often a workgroup of such a split looks for the other parts of
+  // its tile to arrive before it leaves the rest to the last one (0: not at
+  // all; what a launch whose parts cannot all run at once should say).
+  int32_t split_spin_limit = 0;
 };
 
 // Buffers of the products of a batched launch (GemmArgs holds what they have
@@ -112,6 +121,7 @@ enum class GemmKind { kInt8, kInt8Int16, kF32 };
 struct DepthSplit {
   int parts = 1;
   size_t partial_bytes = 0;
+  bool large_tile = false;  // goes to GemmArgs::split_large
 };
 DepthSplit GemmDepthSplit(const GemmArgs& args, int num_cus, GemmKind kind);
 // Number of 32-bit counters split_counters must hold.

@@ -382,7 +382,9 @@ void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_row
   const mfma_gemm::Model which = kind == GemmKind::kInt8Int16 ? mfma_gemm::Model::kInt8PlaneSplit
                                  : kind == GemmKind::kF32     ? mfma_gemm::Model::kF32
                                                               : mfma_gemm::Model::kInt8;
-  const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, which);
+  const DepthSplit split = mfma_gemm::PlanDepthSplit(args, num_cus, which);
+  const mfma_gemm::Tile tile =
+      split.large_tile ? mfma_gemm::Tile::k256x256 : mfma_gemm::ChooseTile(args, num_cus, which).tile;
   const mfma_gemm::TimingModel model = mfma_gemm::TimingModelOf(which);
   for (int i = 0; i < model.count; ++i) {
     if (model.tiles[i].tile == tile) {
@@ -390,17 +392,21 @@ void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_row
       *tile_cols = model.tiles[i].bn;
     }
   }
-  *depth_parts = mfma_gemm::PlanDepthSplit(args, num_cus, which).parts;
+  *depth_parts = split.parts;
 }
 
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
-  return mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k64x64;
+  const mfma_gemm::TileChoice choice = mfma_gemm::ChooseTile(args, num_cus, mfma_gemm::Model::kInt8);
+  return choice.large_parts == 1 && choice.tile == mfma_gemm::Tile::k64x64;
 }
 
 bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   const bool flip = args.a_flip != 0 || args.b_flip != 0;
   const int tiles_m = (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
-  return !flip && args.k_bytes / 128 >= fused_sums::kMinDepthSteps &&
+  // (Asked after the depth split has been planned: every part needs its steps.)
+  const int parts = args.split_k > 1 && args.split_large ? args.split_k : 1;
+  const int steps = args.k_bytes / 128;
+  return !flip && depth_split::StepCount(steps, parts, parts - 1) >= fused_sums::kMinDepthSteps &&
          tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows &&
          mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k256x256;
 }

@@ -225,10 +225,11 @@ struct Cfg {
 // the rows of `a`, dealt out over the first workgroups of every tile row, and
 // every workgroup fetches them shortly before its write-back (fused_sums.h).
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
-          bool kDepthWaves = false, bool kRowSums = false>
+          bool kDepthWaves = false, bool kRowSums = false, bool kSplitLarge = false>
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   static_assert(!kRowSums || (Traits::kPaired && !kFlip && !kFusedSums),
                 "row sums in passing exist for the paired schedule on int8 data");
+  static_assert(!kSplitLarge || Traits::kPaired, "kSplitLarge is the depth split of the paired schedule's tile");
   static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
                 "fused sums exist for the tiles with one block (one block per plane) per wave only");
   static_assert(!kFlip || !Traits::kSplitB, "in-place uint8 operands exist for the int8 kernel only");
@@ -288,8 +289,6 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int wave_m = wave >> 1;
   const int wave_n = wave & 1;
 
-  const v4i a_rsrc = MakeRsrc(args.a, args.a_bytes);
-  const v4i b_rsrc = MakeRsrc(args.b, args.b_bytes);
   // The 32-bit LDS address of the dynamic shared array (what M0 wants).
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 
@@ -297,7 +296,30 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // Load i of this wave fills LDS 16-byte slots [chunk*64, chunk*64+64) of the
   // tile; slot p holds tile row p / granules-per-row, granule
   // (p % granules-per-row) ^ Swizzle(row).
-  const int K = args.k_bytes;  // depth in bytes
+  // Depth split (args.split_k > 1; tiles of at most two 32x32 blocks per wave,
+  // and the largest int8 tile in a kernel of its own, kSplitLarge): the
+  // workgroups of grid row blockIdx.y walk the blockIdx.y-th part of the depth
+  // steps only; their accumulators are added up before the write-back (below).
+  constexpr bool kCanSplitDepth = (WM * WN <= 2 && kB == 32) || kSplitLarge;
+  const int split = kCanSplitDepth ? args.split_k : 1;
+  const int split_index = kCanSplitDepth ? blockIdx.y : 0;
+  // Divisions run on the vector unit: their results are read back into scalar
+  // registers here, so that what derives from them (a load's scalar offset
+  // operand among others) is scalar whatever the compiler makes of the
+  // expressions.
+  const int steps_of_whole_depth = (args.k_bytes + kBK - 1) / kBK;
+  const int first_step_of_part =
+      __builtin_amdgcn_readfirstlane(depth_split::FirstStep(steps_of_whole_depth, split, split_index));
+  const int steps_of_part =
+      __builtin_amdgcn_readfirstlane(depth_split::StepCount(steps_of_whole_depth, split, split_index));
+  // The largest tile's schedule knows nothing of parts: a part's workgroup
+  // sees operands that begin at its first depth step and are as deep as its
+  // part (the descriptors below start there as well), and walks them from
+  // step 0.
+  const int part_begin = kSplitLarge ? first_step_of_part * kBK : 0;  // bytes
+  const int K = kSplitLarge ? min(args.k_bytes - part_begin, steps_of_part * kBK) : args.k_bytes;  // depth in bytes
+  const v4i a_rsrc = MakeRsrc(static_cast<const char*>(args.a) + part_begin, args.a_bytes - uint32_t(part_begin));
+  const v4i b_rsrc = MakeRsrc(static_cast<const char*>(args.b) + part_begin, args.b_bytes - uint32_t(part_begin));
   uint32_t a_goff[C::kALoads];
   int a_k[C::kALoads];
 #pragma unroll
@@ -330,32 +352,24 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // time. The order of the steps does not matter for the sums. Steps past the
   // end keep their index, which puts them out of range as before.
   //
-  // Depth split (tiles of at most two blocks per wave, args.split_k > 1): the
-  // workgroups of grid row blockIdx.y walk the blockIdx.y-th part of the depth
-  // steps only; their accumulators are added up before the write-back (below).
   // k_tiles, kt_first: the steps this workgroup walks.
-  const int k_tiles_all = (K + kBK - 1) / kBK;
-  constexpr bool kCanSplitDepth = WM * WN <= 2 && kB == 32;
-  const int split = kCanSplitDepth ? args.split_k : 1;
-  const int split_index = kCanSplitDepth ? blockIdx.y : 0;
-  // Divisions run on the vector unit: their results are read back into scalar
-  // registers here, so that what derives from them (a load's scalar offset
-  // operand among others) is scalar whatever the compiler makes of the
-  // expressions.
-  const int kt_first = __builtin_amdgcn_readfirstlane(depth_split::FirstStep(k_tiles_all, split, split_index));
-  const int k_tiles = __builtin_amdgcn_readfirstlane(depth_split::StepCount(k_tiles_all, split, split_index));
+  const int k_tiles_all = kSplitLarge ? steps_of_part : steps_of_whole_depth;
+  const int kt_first = kSplitLarge ? 0 : first_step_of_part;
+  const int k_tiles = steps_of_part;
   constexpr bool kRotateDepth = WM * WN < 16;
   const int rot = __builtin_amdgcn_readfirstlane(
       kRotateDepth && K % kBK == 0 && k_tiles > 0 ? (tile_m * 5 + split_index * 3) % k_tiles : 0);
   // kRowSums: what this wave does for the sums of its rows.
   fused_sums::WaveShare share = {};
   if constexpr (kRowSums) {
+    // (With the depth split every part's contributors deal out the part's
+    // steps; a row's word collects the contributions of all parts.)
     const fused_sums::WaveShare s =
         fused_sums::ShareOfWave(tiles_m, tiles_n, tile_m, tile_n, wave_n, k_tiles, args.row_sums_uniform_run);
     share.contributes = __builtin_amdgcn_readfirstlane(s.contributes);
     share.first_step = __builtin_amdgcn_readfirstlane(s.first_step);
     share.end_step = __builtin_amdgcn_readfirstlane(s.end_step);
-    share.expected = __builtin_amdgcn_readfirstlane(s.expected);
+    share.expected = __builtin_amdgcn_readfirstlane(s.expected) * split;
   }
   auto phys = [&](int kt) {
     if constexpr (!kRotateDepth) return kt;
@@ -1153,25 +1167,49 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // (depth_split.h says what this ordering rests on). That costs nothing when
   // no split is asked for, where fences at device scope would write back and
   // invalidate whole caches.
+  typedef unsigned long long u64;
+  constexpr int kPartWords = C::kBM * C::kBN;  // 32-bit words of one tile's accumulators
+  bool large_split_last = false, large_split_all = false;  // kSplitLarge: see below
   if constexpr (kCanSplitDepth) {
     if (split > 1) {
-      typedef unsigned long long u64;
-      constexpr int kPartWords = C::kBM * C::kBN;  // 32-bit words of one tile's accumulators
       u64* parts = static_cast<u64*>(args.split_partials) + size_t(t) * split * (kPartWords / 2);
       u64* mine = parts + size_t(split_index) * (kPartWords / 2) + tid;
+      // (kAB x kBB blocks of kAccElems values a thread: two values a word.)
 #pragma unroll
-      for (int i = 0; i < WM; ++i)
+      for (int i = 0; i < kAB; ++i)
 #pragma unroll
-        for (int j = 0; j < WN; ++j)
+        for (int j = 0; j < kBB; ++j)
 #pragma unroll
-          for (int h = 0; h < 8; ++h) {
+          for (int h = 0; h < kAccElems / 2; ++h) {
             const u64 w = u64(uint32_t(Traits::RawBits(acc[i][j][2 * h]))) |
                           (u64(uint32_t(Traits::RawBits(acc[i][j][2 * h + 1]))) << 32);
-            __hip_atomic_store(mine + ((i * WN + j) * 8 + h) * C::kThreads, w, __ATOMIC_RELAXED,
+            __hip_atomic_store(mine + ((i * kBB + j) * (kAccElems / 2) + h) * C::kThreads, w, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
           }
       WaitVmcnt<0>();
       __syncthreads();
+      if constexpr (kSplitLarge) {
+        // The largest tile: the parts share the adding up and the write-back
+        // (depth_split.h). Count in, then look for the others a bounded number
+        // of times; what follows is part of the write-back below.
+        unsigned* words = args.split_counters + depth_split::kLargeWordsPerTile * t;
+        unsigned* shared = reinterpret_cast<unsigned*>(lds);
+        if (tid == 0) {
+          const unsigned before =
+              __hip_atomic_fetch_add(words + depth_split::kArrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          bool all = before + 1 == unsigned(split);
+          for (int looks = 0; !all && looks < args.split_spin_limit; ++looks) {
+            __builtin_amdgcn_s_sleep(4);
+            all = __hip_atomic_load(words + depth_split::kArrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                  unsigned(split);
+          }
+          shared[0] = before;
+          shared[1] = all;
+        }
+        __syncthreads();
+        large_split_last = depth_split::IsLastArrival(shared[0], split);
+        large_split_all = shared[1] != 0;
+      } else {
       unsigned* arrived = reinterpret_cast<unsigned*>(lds);
       if (tid == 0)
         *arrived = __hip_atomic_fetch_add(args.split_counters + t, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1203,6 +1241,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
               acc[i][j][2 * h] += Traits::FromRawBits(static_cast<int>(uint32_t(w)));
               acc[i][j][2 * h + 1] += Traits::FromRawBits(static_cast<int>(uint32_t(w >> 32)));
             }
+      }
       }
     }
   }
@@ -1258,7 +1297,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           const int row = min(first_row + 64 * h + lane, args.M - 1);
           const char* from = static_cast<const char*>(args.a) + size_t(row) * size_t(args.lda);
           int sum = 0;
-          for (int k = 0; k < K; k += kGranule) {
+          for (int k = 0; k < args.k_bytes; k += kGranule) {  // (the whole depth, whatever part this workgroup walked)
             const v4i x = *reinterpret_cast<const v4i*>(from + k);
 #pragma unroll
             for (int d = 0; d < 4; ++d) sum = __builtin_amdgcn_sdot4(x[d], 0x01010101, sum, false);
@@ -1283,15 +1322,79 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // kMode: the form of the write-back arithmetic (Traits::ModeOf); kElt: bytes
     // per destination element. Compile-time, so that the loop below is
     // straight-line code apart from its one branch on the counter.
-    auto half_pass = [&](auto half_constant, auto mode_constant, auto elt_constant) {
+    // The 16 values of `vals` (this lane's four rows in the four row blocks of
+    // half `half` of block column bj), finished and stored.
+    auto finish_block = [&](auto half_constant, auto mode_constant, auto elt_constant, int bj, int32_t (&vals)[16],
+                            const typename Traits::RowParams& row_params,
+                            const typename Traits::ColParams& col_params) {
       constexpr int half = decltype(half_constant)::value;
       constexpr int kMode = decltype(mode_constant)::value;
       constexpr int kElt = decltype(elt_constant)::value;
-      typename Traits::RowParams row_params;
-      Traits::template ReadRowParams<kMode>(area, half * 64 + 4 * (lane >> 4), row_params);
       // After the transposition: the 16 rows this lane stores.
       const int row0 = m0 + wave_m * (WM * 32) + (half * 4 + (lane >> 4)) * 16;
       const bool rows_full = row0 + 16 <= args.M;
+      const int j = col0 + bj * 16;
+      Traits::template Finish16<kMode>(vals, row_params, col_params, ep);
+      // w[p][k]: after the transposition, word p of the kElt words that hold
+      // rows 4k .. 4k+3 of the lane's block. Every lane takes part in the
+      // swaps; columns and rows past the end are left out when storing.
+      int w[kElt][4];
+      // (The values lie inside the destination type's range by now, so the
+      // saturation of v_cvt_pk_i16_i32 does nothing: it is the two-in-one
+      // instruction that puts a pair into one register.)
+      if constexpr (kElt == 1) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const auto low = __builtin_amdgcn_cvt_pk_i16(vals[4 * b], vals[4 * b + 1]);
+          const auto high = __builtin_amdgcn_cvt_pk_i16(vals[4 * b + 2], vals[4 * b + 3]);
+          // The low bytes of the four 16-bit halves.
+          w[0][b] = __builtin_amdgcn_perm(__builtin_bit_cast(int, high), __builtin_bit_cast(int, low), 0x06040200);
+        }
+      } else if constexpr (kElt == 2) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          w[0][b] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(vals[4 * b], vals[4 * b + 1]));
+          w[1][b] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(vals[4 * b + 2], vals[4 * b + 3]));
+        }
+      } else {
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+#pragma unroll
+          for (int b = 0; b < 4; ++b) w[p][b] = vals[4 * b + p];
+      }
+#pragma unroll
+      for (int p = 0; p < kElt; ++p) transpose(w[p]);
+      if (j < args.n_logical && row0 < args.M) {
+        char* out = dst_base + (int64_t(j) * ldd + row0) * kElt;
+        if (rows_full) {
+          // Memory order: rows 4k .. 4k+3 are words w[0][k] .. w[kElt-1][k].
+#pragma unroll
+          for (int x = 0; x < kElt; ++x) {
+            v4i o;
+#pragma unroll
+            for (int y = 0; y < 4; ++y) o[y] = w[(4 * x + y) % kElt][(4 * x + y) / kElt];
+            reinterpret_cast<v4i_unaligned*>(out)[x] = o;
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            if (row0 + r < args.M) {
+              if constexpr (kElt == 1)
+                reinterpret_cast<int8_t*>(out)[r] = static_cast<int8_t>(w[0][r / 4] >> (8 * (r % 4)));
+              else if constexpr (kElt == 2)
+                reinterpret_cast<int16_t*>(out)[r] = static_cast<int16_t>(w[(r % 4) / 2][r / 4] >> (16 * (r % 2)));
+              else
+                reinterpret_cast<int32_t*>(out)[r] = w[r % 4][r / 4];
+            }
+          }
+        }
+      }
+    };
+    auto half_pass = [&](auto half_constant, auto mode_constant, auto elt_constant) {
+      constexpr int half = decltype(half_constant)::value;
+      constexpr int kMode = decltype(mode_constant)::value;
+      typename Traits::RowParams row_params;
+      Traits::template ReadRowParams<kMode>(area, half * 64 + 4 * (lane >> 4), row_params);
       // A compact loop over the block columns: only the gathering of a
       // column's accumulators, whose register numbers must be constants, is
       // written out eight times, behind a branch on the (wave-uniform) counter.
@@ -1300,7 +1403,6 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       Traits::template ReadColParams<kMode>(area, lane & 15, col_ahead);
 #pragma unroll 1
       for (int bj = 0; bj < kBB; ++bj) {
-        const int j = col0 + bj * 16;
         col_params = col_ahead;
         Traits::template ReadColParams<kMode>(area, ((bj + 1) & (kBB - 1)) * 16 + (lane & 15), col_ahead);
         int32_t vals[16];
@@ -1314,83 +1416,140 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
                 vals[4 * b + v] = Traits::Bits(acc[half * 4 + b][kBj][v], acc[half * 4 + b][kBj][v]);
           }
         });
-        Traits::template Finish16<kMode>(vals, row_params, col_params, ep);
-        // w[p][k]: after the transposition, word p of the kElt words that hold
-        // rows 4k .. 4k+3 of the lane's block. Every lane takes part in the
-        // swaps; columns and rows past the end are left out when storing.
-        int w[kElt][4];
-        // (The values lie inside the destination type's range by now, so the
-        // saturation of v_cvt_pk_i16_i32 does nothing: it is the two-in-one
-        // instruction that puts a pair into one register.)
-        if constexpr (kElt == 1) {
-#pragma unroll
-          for (int b = 0; b < 4; ++b) {
-            const auto low = __builtin_amdgcn_cvt_pk_i16(vals[4 * b], vals[4 * b + 1]);
-            const auto high = __builtin_amdgcn_cvt_pk_i16(vals[4 * b + 2], vals[4 * b + 3]);
-            // The low bytes of the four 16-bit halves.
-            w[0][b] = __builtin_amdgcn_perm(__builtin_bit_cast(int, high), __builtin_bit_cast(int, low), 0x06040200);
-          }
-        } else if constexpr (kElt == 2) {
-#pragma unroll
-          for (int b = 0; b < 4; ++b) {
-            w[0][b] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(vals[4 * b], vals[4 * b + 1]));
-            w[1][b] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(vals[4 * b + 2], vals[4 * b + 3]));
-          }
-        } else {
-#pragma unroll
-          for (int p = 0; p < 4; ++p)
-#pragma unroll
-            for (int b = 0; b < 4; ++b) w[p][b] = vals[4 * b + p];
-        }
-#pragma unroll
-        for (int p = 0; p < kElt; ++p) transpose(w[p]);
-        if (j < args.n_logical && row0 < args.M) {
-          char* out = dst_base + (int64_t(j) * ldd + row0) * kElt;
-          if (rows_full) {
-            // Memory order: rows 4k .. 4k+3 are words w[0][k] .. w[kElt-1][k].
-#pragma unroll
-            for (int x = 0; x < kElt; ++x) {
-              v4i o;
-#pragma unroll
-              for (int y = 0; y < 4; ++y) o[y] = w[(4 * x + y) % kElt][(4 * x + y) / kElt];
-              reinterpret_cast<v4i_unaligned*>(out)[x] = o;
-            }
-          } else {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              if (row0 + r < args.M) {
-                if constexpr (kElt == 1)
-                  reinterpret_cast<int8_t*>(out)[r] = static_cast<int8_t>(w[0][r / 4] >> (8 * (r % 4)));
-                else if constexpr (kElt == 2)
-                  reinterpret_cast<int16_t*>(out)[r] = static_cast<int16_t>(w[(r % 4) / 2][r / 4] >> (16 * (r % 2)));
-                else
-                  reinterpret_cast<int32_t*>(out)[r] = w[r % 4][r / 4];
-              }
-            }
-          }
-        }
+        finish_block(half_constant, mode_constant, elt_constant, bj, vals, row_params, col_params);
       }
     };
-    auto write_back = [&](auto mode_constant, auto elt_constant) {
-      half_pass(std::integral_constant<int, 0>(), mode_constant, elt_constant);
-      half_pass(std::integral_constant<int, 1>(), mode_constant, elt_constant);
+    // Depth split of this tile: block columns bj_first .. bj_end - 1 of the
+    // tile, from this workgroup's accumulators and those of the other parts in
+    // memory. A block column of one part is 16 loads of two values a thread;
+    // those of up to four parts are in flight at a time.
+    auto columns_of_parts = [&](auto mode_constant, auto elt_constant, int bj_first, int bj_end) {
+      constexpr int kMode = decltype(mode_constant)::value;
+      typename Traits::RowParams row_params[2];
+      Traits::template ReadRowParams<kMode>(area, 4 * (lane >> 4), row_params[0]);
+      Traits::template ReadRowParams<kMode>(area, 64 + 4 * (lane >> 4), row_params[1]);
+      const u64* parts = static_cast<const u64*>(args.split_partials) + size_t(t) * split * (kPartWords / 2) + tid;
+      constexpr int kInFlight = 4;
+      constexpr int kWordsPerColumn = kAB * (kAccElems / 2);
+#pragma unroll 1
+      for (int bj = bj_first; bj < bj_end; ++bj) {
+        typename Traits::ColParams col_params;
+        Traits::template ReadColParams<kMode>(area, bj * 16 + (lane & 15), col_params);
+        // This workgroup's own part is still in its registers (read, not
+        // written: as the write-back of an unsplit tile reads them).
+        int32_t column[kAB][kAccElems];
+        StaticFor<kBB>([&](auto bj_constant) {
+          constexpr int kBj = decltype(bj_constant)::value;
+          if (bj == kBj) {
+#pragma unroll
+            for (int i = 0; i < kAB; ++i)
+#pragma unroll
+              for (int v = 0; v < kAccElems; ++v) column[i][v] = Traits::Bits(acc[i][kBj][v], acc[i][kBj][v]);
+          }
+        });
+#pragma unroll 1
+        for (int first_part = 0; first_part < split - 1; first_part += kInFlight) {
+          u64 w[kInFlight][kWordsPerColumn];
+          StaticFor<kInFlight>([&](auto slot_constant) {
+            constexpr int slot = decltype(slot_constant)::value;
+            if (first_part + slot < split - 1) {
+              // (Of the other parts: this workgroup's own is skipped.)
+              const int part = first_part + slot + (first_part + slot >= split_index ? 1 : 0);
+              const u64* from = parts + size_t(part) * (kPartWords / 2);
+#pragma unroll
+              for (int i = 0; i < kAB; ++i)
+#pragma unroll
+                for (int h = 0; h < kAccElems / 2; ++h)
+                  w[slot][i * (kAccElems / 2) + h] =
+                      __hip_atomic_load(from + ((i * kBB + bj) * (kAccElems / 2) + h) * C::kThreads, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+            }
+          });
+          StaticFor<kInFlight>([&](auto slot_constant) {
+            constexpr int slot = decltype(slot_constant)::value;
+            if (first_part + slot < split - 1) {
+#pragma unroll
+              for (int i = 0; i < kAB; ++i)
+#pragma unroll
+                for (int h = 0; h < kAccElems / 2; ++h) {
+                  const u64 x = w[slot][i * (kAccElems / 2) + h];
+                  column[i][2 * h] += static_cast<int>(uint32_t(x));
+                  column[i][2 * h + 1] += static_cast<int>(uint32_t(x >> 32));
+                }
+            }
+          });
+        }
+        StaticFor<2>([&](auto half_constant) {
+          constexpr int half = decltype(half_constant)::value;
+          int32_t vals[16];
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) vals[4 * b + v] = column[half * 4 + b][v];
+          finish_block(half_constant, mode_constant, elt_constant, bj, vals, row_params[half], col_params);
+        });
+      }
     };
     // An int32 destination takes the raw form, and only it does; the others
-    // are one or two bytes wide.
+    // are one or two bytes wide. bj_first, bj_end: looked at by the depth
+    // split only.
     const int mode = Traits::ModeOf(ep);
-    if (mode == Traits::kRaw) {
-      write_back(std::integral_constant<int, Traits::kRaw>(), std::integral_constant<int, 4>());
-    } else {
-      StaticFor<Traits::kFinishModes>([&](auto mode_constant) {
-        if constexpr (decltype(mode_constant)::value != Traits::kRaw) {
-          if (mode == decltype(mode_constant)::value) {
-            if (elt == 1)
-              write_back(mode_constant, std::integral_constant<int, 1>());
-            else
-              write_back(mode_constant, std::integral_constant<int, 2>());
-          }
+    auto write_columns = [&](int bj_first, int bj_end) {
+      auto write_back = [&](auto mode_constant, auto elt_constant) {
+        if constexpr (kSplitLarge) {
+          columns_of_parts(mode_constant, elt_constant, bj_first, bj_end);
+        } else {
+          half_pass(std::integral_constant<int, 0>(), mode_constant, elt_constant);
+          half_pass(std::integral_constant<int, 1>(), mode_constant, elt_constant);
         }
-      });
+      };
+      if (mode == Traits::kRaw) {
+        write_back(std::integral_constant<int, Traits::kRaw>(), std::integral_constant<int, 4>());
+      } else {
+        StaticFor<Traits::kFinishModes>([&](auto mode_constant) {
+          if constexpr (decltype(mode_constant)::value != Traits::kRaw) {
+            if (mode == decltype(mode_constant)::value) {
+              if (elt == 1)
+                write_back(mode_constant, std::integral_constant<int, 1>());
+              else
+                write_back(mode_constant, std::integral_constant<int, 2>());
+            }
+          }
+        });
+      }
+    };
+    if constexpr (!kSplitLarge) {
+      write_columns(0, kBB);
+    } else {
+      // Depth split of this tile (depth_split.h): this workgroup's columns, if
+      // every part has arrived and nobody else has taken them; the last one to
+      // arrive goes on to the columns nobody has taken.
+      unsigned* words = args.split_counters + depth_split::kLargeWordsPerTile * t;
+      unsigned* shared = reinterpret_cast<unsigned*>(lds);
+      const int columns = depth_split::LargeColumnsPerPart(split);
+#pragma unroll 1
+      for (int turn = 0; turn < split; ++turn) {
+        if (turn == 0 ? !large_split_all : !large_split_last) break;
+        const int owner = split_index + turn < split ? split_index + turn : split_index + turn - split;
+        __syncthreads();  // (everybody has read the last claim's answer)
+        if (tid == 0)
+          shared[2] = __hip_atomic_fetch_or(words + depth_split::kClaims, depth_split::ClaimBit(owner),
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (!depth_split::ClaimSucceeded(shared[2], owner)) continue;
+        write_columns(owner * columns, owner * columns + columns);
+      }
+      // Count out; the last one out leaves the tile's words at zero for the next launch.
+      __syncthreads();
+      if (tid == 0) {
+        const unsigned before =
+            __hip_atomic_fetch_add(words + depth_split::kExits, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (depth_split::IsLastArrival(before, split)) {
+          __hip_atomic_store(words + depth_split::kArrivals, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(words + depth_split::kClaims, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(words + depth_split::kExits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
     }
     return;
   }
@@ -1571,9 +1730,9 @@ constexpr int WavesPerSimdWanted() {
   return (!kDepthWaves && STAGES == 2 && WM * WN == 2) ? 3 : 1;
 }
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
-          bool kDepthWaves = false, bool kRowSums = false>
+          bool kDepthWaves = false, bool kRowSums = false, bool kSplitLarge = false>
 __global__ __launch_bounds__(256, (WavesPerSimdWanted<WM, WN, STAGES, kDepthWaves>())) void MfmaGemmKernel(GemmArgs args) {
-  MfmaGemmBody<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves, kRowSums>(args);
+  MfmaGemmBody<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves, kRowSums, kSplitLarge>(args);
 }
 
 // Several products of one shape in one launch: grid.z counts the products,
@@ -1612,7 +1771,7 @@ hipError_t LaunchBatch(hipStream_t stream, const GemmArgs& args, const GemmBatch
 }
 
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
-          bool kDepthWaves = false, bool kRowSums = false>
+          bool kDepthWaves = false, bool kRowSums = false, bool kSplitLarge = false>
 hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   using C = Cfg<WM, WN, BK, STAGES, Traits::kSplitB, Traits::kBlock>;
   const int tiles_m = (args.M + C::kBM - 1) / C::kBM;
@@ -1621,7 +1780,7 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int grid = ((total + 7) / 8) * 8;
   // The depth-per-wave schedule: two ring slots of 16 KiB for each of four waves.
   const size_t lds_bytes = kDepthWaves ? size_t(4 * 2 * 128 * BK) : size_t(C::kLdsBytes);
-  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves, kRowSums>;
+  auto kernel = MfmaGemmKernel<Traits, WM, WN, BK, STAGES, kFusedSums, kFlip, kDepthWaves, kRowSums, kSplitLarge>;
   if (kRowSums != (args.row_sums != nullptr)) return hipErrorInvalidValue;
   if (kRowSums && (!args.row_sums_to_zero || tiles_m * C::kBM > fused_sums::kMaxRows ||
                    args.row_sums_zero_rows > fused_sums::kMaxRows))
@@ -1637,10 +1796,17 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   const int split = args.split_k;
   if (split != 1) {
     const int k_tiles = (args.k_bytes + BK - 1) / BK;
-    if (WM * WN > 2 || Traits::kBlock != 32 || split < 1 || !args.split_partials || !args.split_counters || total > kSplitCounters ||
+    const bool can_split = kSplitLarge || (WM * WN <= 2 && Traits::kBlock == 32);
+    if (!can_split || split < 1 || !args.split_partials || !args.split_counters || total > kSplitCounters ||
         !depth_split::NoEmptyPart(k_tiles, split))
       return hipErrorInvalidValue;
+    if (kSplitLarge && (!depth_split::LargePartsAllowed(split) ||
+                        total * depth_split::kLargeWordsPerTile > kSplitCounters || args.split_spin_limit < 0))
+      return hipErrorInvalidValue;
   }
+  // (The split form of the largest tile is a kernel of its own: the plain one
+  // does not carry the exchange of the parts.)
+  if (kSplitLarge && split < 2) return hipErrorInvalidValue;
   hipLaunchKernelGGL(kernel, dim3(grid, split), dim3(C::kThreads), lds_bytes, stream, args);
   return hipGetLastError();
 }
@@ -1798,11 +1964,40 @@ inline bool ShallowRing(const GemmArgs& args, int num_cus, int bm, int bn) {
   return TileCount(args, bm, bn) > num_cus;
 }
 
-inline Tile PickTile(const GemmArgs& args, int num_cus, Model which) {
+// The depth split of the 256x256 int8 tile (a kernel of its own, kSplitLarge):
+// for destinations of so few tiles that the 256x256 grid leaves most CUs idle,
+// with depths so long that a part still has kLargeSplitMinSteps ring steps.
+// Adding up the parts costs in proportion to the tile's area - every part
+// writes 256 KiB of accumulators, the last to arrive reads those of the
+// others - which one 128x128 tile per CU, at 55 % of the large tile's rate,
+// only loses to beyond depths of about 10000.
+constexpr int kLargeSplitMinSteps = 16;
+// Microseconds to store a part and to add one other part to one's own.
+constexpr double kLargeSplitStore = 2.5, kLargeSplitAddPart = 2.6;
+inline int LargeSplitPartsWanted(int tiles, int k_steps, int num_cus) {
+  if (tiles <= 0 || tiles * depth_split::kLargeWordsPerTile > kSplitCounters) return 1;
+  return depth_split::LargeParts(k_steps, std::min(num_cus / tiles, k_steps / kLargeSplitMinSteps));
+}
+
+// The tile a launch should run on, and large_parts > 1 if it should rather run
+// on the 256x256 tile with its depth split that many ways (if the buffers for
+// that can be had: `tile` is the answer without).
+struct TileChoice {
+  Tile tile;
+  int large_parts;
+};
+inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
   const TimingModel model = TimingModelOf(which);
-  for (int i = 0; i < model.count; ++i)
-    if (model.tiles[i].bm == args.forced_tile_rows && model.tiles[i].bn == args.forced_tile_cols)
-      return model.tiles[i].tile;
+  const int k_steps = std::max(1, (args.k_bytes + 127) / 128);
+  for (int i = 0; i < model.count; ++i) {
+    if (model.tiles[i].bm == args.forced_tile_rows && model.tiles[i].bn == args.forced_tile_cols) {
+      int parts = 1;
+      if (which == Model::kInt8 && model.tiles[i].tile == Tile::k256x256 && args.forced_depth_parts > 1 &&
+          TileCount(args, 256, 256) * depth_split::kLargeWordsPerTile <= kSplitCounters)
+        parts = depth_split::LargeParts(k_steps, args.forced_depth_parts);
+      return {model.tiles[i].tile, parts};
+    }
+  }
   Tile best = model.tiles[0].tile;
   double best_time = ModelledMicroseconds(args, num_cus, model, model.tiles[0]);
   for (int i = 1; i < model.count; ++i) {
@@ -1812,13 +2007,42 @@ inline Tile PickTile(const GemmArgs& args, int num_cus, Model which) {
       best = model.tiles[i].tile;
     }
   }
-  return best;
+  int large_parts = 1;
+  if (which == Model::kInt8 && model.tiles[0].tile == Tile::k256x256) {
+    const TileTiming& t = model.tiles[0];
+    const int tiles = TileCount(args, t.bm, t.bn);
+    const int parts = LargeSplitPartsWanted(tiles, k_steps, num_cus);
+    if (parts > 1) {
+      const double fraction = double(tiles * parts) / num_cus;  // (at most one round)
+      const double time = t.fixed +
+                          (t.last_round + (1 - t.last_round) * fraction) * t.step *
+                              (t.overhead + depth_split::StepsPerPart(k_steps, parts)) +
+                          kLargeSplitStore + kLargeSplitAddPart * (parts - 1);
+      if (time < best_time) large_parts = parts;
+    }
+  }
+  return {best, large_parts};
+}
+
+// The tile a launch of these arguments runs on (whose split_k and split_large
+// say what buffers the caller could get).
+inline Tile PickTile(const GemmArgs& args, int num_cus, Model which) {
+  if (which == Model::kInt8 && args.split_k > 1 && args.split_large) return Tile::k256x256;
+  return ChooseTile(args, num_cus, which).tile;
 }
 
 // Depth split for a launch of `args` (see GemmArgs::split_k and DepthSplitParts).
 inline DepthSplit PlanDepthSplit(const GemmArgs& args, int num_cus, Model which) {
   const TimingModel model = TimingModelOf(which);
-  if (PickTile(args, num_cus, which) != model.smallest) return DepthSplit();
+  const TileChoice choice = ChooseTile(args, num_cus, which);
+  if (choice.large_parts > 1) {
+    DepthSplit split;
+    split.parts = choice.large_parts;
+    split.partial_bytes = size_t(choice.large_parts) * TileCount(args, 256, 256) * 256 * 256 * 4;
+    split.large_tile = true;
+    return split;
+  }
+  if (choice.tile != model.smallest) return DepthSplit();
   const bool split_b = which == Model::kInt8PlaneSplit;
   const int bm = 64, bn = split_b ? 128 : 64;
   const int tiles = TileCount(args, bm, bn);
@@ -1861,8 +2085,14 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
   switch (tile) {
     case Tile::k256x256:
       if constexpr (Traits::LargeTile::kPaired && !kFlip) {
+        if (args.row_sums && args.split_k > 1)
+          return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, false, false, true, true>(stream, args);
         if (args.row_sums)
           return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, false, false, true>(stream, args);
+      }
+      if constexpr (Traits::LargeTile::kPaired) {
+        if (args.split_k > 1)
+          return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip, false, false, true>(stream, args);
       }
       return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip>(stream, args);
     case Tile::k128x128:

@@ -242,6 +242,11 @@ int PrepareOperand8(ruyamd_ctx* ctx, MulCall* call, int side, int32_t zero_point
   return RUYAMD_OK;
 }
 
+// How often a workgroup of the 256x256 tile's depth split looks for the other
+// parts of its tile (a look takes a microsecond or two; the parts of a tile
+// finish within a few of each other).
+constexpr int kLargeSplitLooks = 2048;
+
 // Few destination tiles and a long depth: lets the kernel split the depth over
 // several workgroups per tile if the workspace has (or may get) room for their
 // partial accumulators. Without room the launch simply stays unsplit.
@@ -259,6 +264,14 @@ void PlanDepthSplit(ruyamd_ctx* ctx, GemmKind kind, GemmArgs* args) {
     if (LaunchFillZero(ctx->stream, counters, static_cast<uint32_t>(GemmDepthSplitCounters())) != hipSuccess) return;
   }
   args->split_k = split.parts;
+  args->split_large = split.large_tile ? 1 : 0;
+  if (split.large_tile) {
+    // The parts of a tile wait for each other (briefly, and not without bound)
+    // only where all of them run at once.
+    const int tiles = ((args->M + 255) / 256) * ((args->N + 255) / 256);
+    const bool all_at_once = tiles * split.parts <= ctx->multiprocessor_count;
+    args->split_spin_limit = all_at_once && !ctx->forced_split_without_waiting ? kLargeSplitLooks : 0;
+  }
   args->split_partials = partials;
   args->split_counters = counters;
 }
@@ -274,6 +287,7 @@ bool SetupInt8Gemm(ruyamd_ctx* ctx, const MulCall& call, const Operand8& a, cons
                    int32_t rzp, GemmArgs* out) {
   GemmArgs& args = *out;
   args.forced_tile_rows = ctx->forced_tile_rows;
+  args.forced_depth_parts = ctx->forced_depth_parts;
   args.forced_tile_cols = ctx->forced_tile_cols;
   const int M = call.lhs.rows, K = call.lhs.cols, N = call.rhs.cols;
   args.k_bytes = RoundUp(K, 16);  // packed/in-place depth; the padding is zero
@@ -391,6 +405,7 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   // shares the GPU's static scratch area with other contexts.
   Operand8& kernel_a = swap ? b : a;
   bool row_sums_in_launch = false;
+  PlanDepthSplit(ctx, GemmKind::kInt8, &args);  // (first: what the sums can do depends on it)
   if (!args.fuse_sums && kernel_a.sums_pending && ctx->row_sums_in_launch && !ctx->capturing && !ctx->no_alloc &&
       GemmI8CanFormRowSums(args, ctx->multiprocessor_count)) {
     const int set = ctx->row_sums_next;
@@ -401,7 +416,7 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     args.row_sums_fetch_late = ctx->row_sums_fetch_late;
     const int tiles_m = (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
     const int tiles_n = (args.N + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
-    if (fused_sums::FirstContributorIsZero(tiles_m, tiles_n))
+    if (args.split_k == 1 && fused_sums::FirstContributorIsZero(tiles_m, tiles_n))
       args.row_sums_uniform_run = fused_sums::StepsPerWave(
           (args.k_bytes + 127) / 128, std::min(tiles_n, fused_sums::kMaxContributorTiles));
     kernel_a.sums_pending = false;
@@ -414,7 +429,6 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   args.ep.lhs_sums = (swap ? b : a).sums;
   args.ep.rhs_sums = (swap ? a : b).sums;
   if (row_sums_in_launch) args.ep.lhs_sums = nullptr;  // the kernel does not look there
-  PlanDepthSplit(ctx, GemmKind::kInt8, &args);
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
@@ -610,6 +624,7 @@ int RunF32(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   }
   GemmArgs args;
   args.forced_tile_rows = ctx->forced_tile_rows;
+  args.forced_depth_parts = ctx->forced_depth_parts;
   args.forced_tile_cols = ctx->forced_tile_cols;
   args.k_bytes = RoundUp(K, 4) * 4;
   const bool swap = SetupDestination(*call, &args);
@@ -642,6 +657,7 @@ int RunI8I16(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   const int M = call->lhs.rows, K = call->lhs.cols, N = call->rhs.cols;
   GemmArgs args;
   args.forced_tile_rows = ctx->forced_tile_rows;
+  args.forced_depth_parts = ctx->forced_depth_parts;
   args.forced_tile_cols = ctx->forced_tile_cols;
   const bool swap = SetupDestination(*call, &args);  // true: A side = rhs
   const int side8 = swap ? 1 : 0;
@@ -802,6 +818,7 @@ int RunMulBatch(ruyamd_ctx* ctx, const MulCall& first, const BatchBuffers* items
   if (ShouldCache(first.lhs_cache_policy, N) || ShouldCache(first.rhs_cache_policy, M)) return RUYAMD_OK;
   GemmArgs shape;
   shape.forced_tile_rows = ctx->forced_tile_rows;
+  shape.forced_depth_parts = ctx->forced_depth_parts;
   shape.forced_tile_cols = ctx->forced_tile_cols;
   shape.M = M;
   shape.N = N;

@@ -13,6 +13,9 @@
 // it sees every part, the sum is taken in part order, and the counters are
 // back at zero for the next launch.
 //
+// The same for the split of the 256x256 int8 tile, whose parts also share the
+// adding up and the write-back by waiting for each other a bounded time.
+//
 // Row sums formed inside the launch of the largest int8 tile: which
 // workgroups of a tile row add up which depth steps (kernels/fused_sums.h).
 // Checked for every grid up to 48 x 48 tiles and several depths: the shares of
@@ -169,6 +172,110 @@ static void TestDepthSplitArrivalProtocol() {
   }
 }
 
+// The split of the largest int8 tile (depth_split.h, second half): the parts
+// of a tile also share the adding up and the write-back. One host thread per
+// workgroup runs the kernel's protocol on the tile's three words - count in,
+// look for the others a bounded number of times, claim one's own columns, the
+// last one to arrive claims what is left, count out, last one out clears the
+// words - with every kind of patience (no look at all, a few, many) and small
+// random delays. Checked: every block column of every tile is finished exactly
+// once, from all parts' values; the words are zero again after every launch;
+// with no patience at all the last arriver does everything.
+struct LargeSplitModel {
+  int tiles, steps;
+  std::vector<std::atomic<unsigned>> words;  // kLargeWordsPerTile per tile
+  std::vector<long long> slices;             // [tile][part][block column]
+  std::vector<std::atomic<int>> finished;    // [tile][block column]: how often
+  std::vector<long long> result;             // [tile][block column]
+  std::vector<std::atomic<int>> columns_by_last;  // [tile]: columns the last arriver finished
+  LargeSplitModel(int tiles, int steps)
+      : tiles(tiles), steps(steps), words(size_t(tiles) * ds::kLargeWordsPerTile),
+        slices(size_t(tiles) * ds::kLargeMaxParts * ds::kLargeBlockColumns),
+        finished(size_t(tiles) * ds::kLargeBlockColumns), result(size_t(tiles) * ds::kLargeBlockColumns),
+        columns_by_last(tiles) {
+    for (auto& w : words) w.store(0);
+  }
+  static long long Value(int t, int k, int column) { return (t + 1) * 1000003ll + k * 7919ll - column * 31ll; }
+  void Launch(int parts, int looks, unsigned seed) {
+    for (auto& f : finished) f.store(0);
+    for (auto& c : columns_by_last) c.store(0);
+    std::vector<std::thread> threads;
+    for (int t = 0; t < tiles; ++t)
+      for (int z = 0; z < parts; ++z)
+        threads.emplace_back([this, t, z, parts, looks, seed] {
+          unsigned rng = seed * 2654435761u + unsigned(t * 131 + z * 17 + 1);
+          auto pause = [&rng] {
+            rng = rng * 1664525u + 1013904223u;
+            if ((rng >> 28) < 6) std::this_thread::yield();
+          };
+          std::atomic<unsigned>* w = &words[size_t(t) * ds::kLargeWordsPerTile];
+          // The part's accumulators: all block columns go to memory.
+          const int first = ds::FirstStep(steps, parts, z);
+          for (int c = 0; c < ds::kLargeBlockColumns; ++c) {
+            long long sum = 0;
+            for (int k = first; k < first + ds::StepCount(steps, parts, z); ++k) sum += Value(t, k, c);
+            slices[(size_t(t) * ds::kLargeMaxParts + z) * ds::kLargeBlockColumns + c] = sum;
+          }
+          pause();
+          const unsigned before = w[ds::kArrivals].fetch_add(1, std::memory_order_acq_rel);
+          const bool last = ds::IsLastArrival(before, parts);
+          bool all = last;
+          for (int look = 0; !all && look < looks; ++look) {
+            pause();
+            all = w[ds::kArrivals].load(std::memory_order_acquire) == unsigned(parts);
+          }
+          const int columns = ds::LargeColumnsPerPart(parts);
+          for (int turn = 0; turn < parts; ++turn) {
+            if (turn == 0 ? !all : !last) break;
+            const int owner = z + turn < parts ? z + turn : z + turn - parts;
+            const unsigned claims = w[ds::kClaims].fetch_or(ds::ClaimBit(owner), std::memory_order_acq_rel);
+            if (!ds::ClaimSucceeded(claims, owner)) continue;
+            for (int c = owner * columns; c < (owner + 1) * columns; ++c) {
+              long long sum = 0;
+              for (int p = 0; p < parts; ++p)
+                sum += slices[(size_t(t) * ds::kLargeMaxParts + p) * ds::kLargeBlockColumns + c];
+              result[size_t(t) * ds::kLargeBlockColumns + c] = sum;
+              finished[size_t(t) * ds::kLargeBlockColumns + c].fetch_add(1);
+              if (last) columns_by_last[t].fetch_add(1);
+              pause();
+            }
+          }
+          if (ds::IsLastArrival(w[ds::kExits].fetch_add(1, std::memory_order_acq_rel), parts)) {
+            w[ds::kArrivals].store(0);
+            w[ds::kClaims].store(0);
+            w[ds::kExits].store(0);
+          }
+        });
+    for (auto& th : threads) th.join();
+  }
+};
+
+static void TestLargeTileSplitProtocol() {
+  const int tiles = 5, steps = 40;
+  LargeSplitModel model(tiles, steps);
+  EXPECT(ds::LargeParts(steps, 8) == 8 && ds::LargeParts(steps, 7) == 4 && ds::LargeParts(steps, 3) == 2 &&
+         ds::LargeParts(steps, 1) == 1 && ds::LargeParts(3, 8) == 2 && ds::LargeParts(1, 8) == 1 &&
+         ds::LargeParts(7, 8) == 4 &&
+         ds::LargeParts(41, 8) == 4);  // (41 steps in 8 parts of 6 would leave the last one empty)
+  for (int launch = 0; launch < 60; ++launch) {
+    const int parts = 2 << (launch % 3);
+    const int looks = launch % 4 == 0 ? 0 : (launch % 4 == 1 ? 3 : 100000);
+    EXPECT(ds::LargePartsAllowed(parts) && ds::NoEmptyPart(steps, parts));
+    model.Launch(parts, looks, unsigned(launch));
+    for (int t = 0; t < tiles; ++t) {
+      for (int c = 0; c < ds::kLargeBlockColumns; ++c) {
+        EXPECT(model.finished[size_t(t) * ds::kLargeBlockColumns + c].load() == 1);
+        long long want = 0;
+        for (int k = 0; k < steps; ++k) want += LargeSplitModel::Value(t, k, c);
+        EXPECT(model.result[size_t(t) * ds::kLargeBlockColumns + c] == want);
+      }
+      for (int i = 0; i < ds::kLargeWordsPerTile; ++i)
+        EXPECT(model.words[size_t(t) * ds::kLargeWordsPerTile + i].load() == 0);
+      if (looks == 0) EXPECT(model.columns_by_last[t].load() == ds::kLargeBlockColumns);
+    }
+  }
+}
+
 namespace fs = ruyamd::fused_sums;
 
 static void CheckRowSumShares(int tiles_m, int tiles_n, int depth_steps) {
@@ -258,6 +365,7 @@ int main() {
   TestElementwiseBlocks();
   TestDepthPartsCoverEveryStepOnce();
   TestDepthSplitArrivalProtocol();
+  TestLargeTileSplitProtocol();
   if (g_failures) {
     std::fprintf(stderr, "host_logic_test: %d failure(s)\n", g_failures);
     return 1;

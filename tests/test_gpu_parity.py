@@ -807,6 +807,96 @@ def test_deep_shapes_that_split_the_depth(device_ctx, tup):
                 compare(p, D.device_mul(device_ctx, p), want)
 
 
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.U8), (S.I8, S.U8, S.I32, S.I32),
+                                 (S.I8, S.I8, S.I32, S.I16)], ids=cases.tuple_name)
+def test_largest_int8_tile_with_its_depth_split(device_ctx, tup):
+    """The 256x256 tile with the depth dealt to several workgroups per tile
+    (what a destination of few such tiles with a very long depth gets): two to
+    eight parts, parts of one step and of many, depths that divide unevenly and
+    end in a partial step, ragged destination edges, operands in place (uint8
+    bytes flipped on the way in) and packed, both destination orders. Every
+    element against the oracle; every problem three times on one context (the
+    arrival counters must be back at zero after each launch). The last shapes
+    are not forced: the timing model itself must send them there."""
+    from ruy_amd import device_problem as D
+    rng = np.random.default_rng(5150 + tup[3])
+    # (Negative: the parts do not wait for each other, the last to arrive adds
+    # up and writes the whole tile; 3, 5, 7 are rounded down to 2 and 4.)
+    forced = [((256, 4096, 256), 4), ((512, 2048, 300), 3), ((700, 5016, 256), 5), ((256, 1024, 512), 8),
+              ((300, 384, 200), 2), ((256, 640, 256), -8), ((513, 3000, 257), 7), ((512, 2048, 512), -4),
+              ((256, 1100, 200), -2)]
+    try:
+        for shape, parts in forced:
+            for orders in (cases.RCC, (1, 0, 1)):
+                p = W.random_problem(rng, *tup, *shape, *orders, strided=False,
+                                     name="%s %s %s in %d parts" % (cases.tuple_name(tup), shape, orders, parts))
+                p.lhs.zero_point = 119 if tup[0] == S.U8 else -7  # (zero points that bring the sums in)
+                p.rhs.zero_point = 133 if tup[1] == S.U8 else 11
+                announce(p.name)
+                want = expected(p)
+                device_ctx.force_tile(256, 256, parts)
+                for _ in range(3):
+                    compare(p, D.device_mul(device_ctx, p), want)
+                    assert device_ctx.last_kernel_name() == "i8_mfma"
+                # ... and the same parts added up must equal the unsplit tile's result
+                device_ctx.force_tile(256, 256, 1)
+                compare(p, D.device_mul(device_ctx, p), want)
+    finally:
+        device_ctx.force_tile(0, 0)
+    if tup == (S.I8, S.I8, S.I32, S.I8):
+        _split_tile_with_sums_in_the_launch(rng)
+    for shape in [(2048, 16384, 2048), (1024, 16400, 2304)]:
+        assert api_tile(*shape)[:2] == (256, 256) and api_tile(*shape)[2] > 1, api_tile(*shape)
+        M, K, N = shape
+        p = W.random_problem(rng, *tup, *shape, *cases.RCC, strided=False,
+                             name="%s %s as the model splits it" % (cases.tuple_name(tup), shape))
+        p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+        announce(p.name)
+        want = O.full_size_expected(p)
+        for _ in range(2):
+            got = D.device_mul(device_ctx, p, dst_fill=0)
+            rows, cols = _boundary_sample(rng, M), _boundary_sample(rng, N)
+            g, w = _sample_block(p, got, rows, cols)
+            assert (g == w).all(), "%s: %d mismatches in the sampled block" % (p.name, (g != w).sum())
+            if want is not None:
+                bad = np.nonzero(got != want)[0]
+                assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+
+
+def _split_tile_with_sums_in_the_launch(rng):
+    """The split tile forms the sums of its `a` operand's rows in passing as
+    the unsplit one does (every part's first workgroups deal out the part's
+    depth steps; a row's word collects the contributions of all parts): with
+    the sums fetched ahead, formed by every wave itself, and by the separate
+    kernel; parts that wait for each other and parts that do not."""
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    tup = (S.I8, S.I8, S.I32, S.I8)
+    problems = []
+    for shape, parts in [((256, 4096, 256), 4), ((700, 5008, 256), 4), ((256, 8192, 768), -4),
+                         ((300, 2048, 200), 2), ((512, 8192, 512), 8)]:
+        for orders in (cases.RCC, (1, 0, 1)):
+            p = W.random_problem(rng, *tup, *shape, *orders, strided=False,
+                                 name="%s %s in %d parts" % (shape, orders, parts))
+            p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+            p.lhs.zero_point, p.rhs.zero_point = 9, -5
+            problems.append((p, parts, expected(p)))
+    for mode, (enable, spin) in {"ahead": (1, -1), "own": (2, 0), "separate": (0, -1)}.items():
+        ctx = api.Context()
+        try:
+            ctx.set_sums_in_launch(enable, spin)
+            calls = 0
+            for p, parts, want in problems:
+                announce("%s, sums %s" % (p.name, mode))
+                ctx.force_tile(256, 256, parts)
+                for _ in range(2):
+                    compare(p, D.device_mul(ctx, p), want)
+                    calls += mode != "separate"
+                    assert ctx.sums_in_launch_calls() == calls
+        finally:
+            ctx.close()
+
+
 def _boundary_sample(rng, n, step=256, random_count=40):
     """Indices in [0, n): a random handful, both ends, and two either side of
     every multiple of `step` (where tiles, and launches cut between tiles, meet)."""

@@ -185,8 +185,8 @@ def test_tile_choice_of_the_timing_model():
     configurations that rely on the smallest tile (its fused sums, its batched
     launch, the int16 operand read in place) get it, the 8192^3 product gets
     the 256 x 256 tile, few tiles with a long depth split it over workgroups,
-    and the choice never splits the depth on a larger tile. Arguments that
-    make no sense are refused."""
+    and the choice splits the depth on no other tile but the 256 x 256 one of
+    the int8 kernel. Arguments that make no sense are refused."""
     from ruy_amd import api
     assert api.tile_for(0, 256, 256, 256) == (64, 64, 1)        # C1
     assert api.tile_for(2, 1024, 1024, 1024) == (64, 64, 1)     # C2
@@ -196,6 +196,10 @@ def test_tile_choice_of_the_timing_model():
     assert api.tile_for(0, 4096, 4096, 4096) == (256, 256, 1)   # exactly one round of large tiles
     rows, cols, parts = api.tile_for(0, 128, 65536, 128)
     assert (rows, cols) == (64, 64) and parts == 32
+    # Few 256x256 tiles with a very long depth: that tile, its depth dealt to 2, 4 or 8 workgroups.
+    assert api.tile_for(0, 2048, 16384, 2048) == (256, 256, 4)
+    assert api.tile_for(0, 2048, 32768, 1024) == (256, 256, 8)
+    assert api.tile_for(0, 2048, 8192, 2048) == (128, 128, 1)   # not worth it at this depth
     rows, cols, parts = api.tile_for(2, 64, 32768, 64)
     assert (rows, cols) == (64, 64) and parts > 1
     for kind in (0, 1, 2):
@@ -205,7 +209,9 @@ def test_tile_choice_of_the_timing_model():
             tiles = ((256, 128), (128, 64), (64, 64)) if kind == 1 else \
                 ((256, 256), (128, 128), (128, 64), (64, 128), (64, 64))
             assert (rows, cols) in tiles, (kind, m, k, n)
-            assert parts == 1 or (rows, cols) == (64, 64)
+            # Only the smallest tile splits the depth, and the 256x256 tile of the int8 kernel.
+            assert parts == 1 or (rows, cols) == (64, 64) or (kind == 0 and (rows, cols) == (256, 256)), \
+                (kind, m, k, n)
     # Fewer compute units: a grid that fills 256 CUs once is four rounds on 64 and stays on the large tile.
     assert api.tile_for(0, 4096, 4096, 4096, compute_units=64) == (256, 256, 1)
     for bad in [(3, 64, 64, 64), (0, 0, 64, 64), (0, 64, -1, 64), (0, 64, 64, 0)]:
