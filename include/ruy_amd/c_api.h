@@ -277,8 +277,9 @@ RUYAMD_API void ruyamd_ctx_force_generic_kernel(ruyamd_ctx* ctx, int force);
  * rounded down to what leaves no part without a depth step) instead of what
  * the model says; negative: that many, and the parts of a tile do not wait for
  * each other to share the adding up, the last one to arrive does it all (the
- * path a launch takes whose workgroups do not all run at once). For tests that must reach a particular tile whatever the model was
- * last fitted to, and for measuring every tile on one shape. No counterpart in
+ * path a launch takes whose workgroups do not all run at once). For tests
+ * that must reach a particular tile whatever the model was last fitted to, and
+ * for measuring every tile on one shape. No counterpart in
  * the reference (its kernel shape is fixed per path, ruy/kernel_x86.h:62-90;
  * its split of the work is MakeBlockMap's, ruy/block_map.cc:339-471). */
 RUYAMD_API int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_cols, int depth_parts);
