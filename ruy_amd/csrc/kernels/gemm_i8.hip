@@ -406,6 +406,11 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   // (Asked after the depth split has been planned: every part needs its steps.)
   const int parts = args.split_k > 1 && args.split_large ? args.split_k : 1;
   const int steps = args.k_bytes / 128;
+  // A row's sums take contributions from every part: the parts' workgroups
+  // must all run at once, or the first ones wait (a bounded but long time) for
+  // contributors that start when they are gone.
+  const int tiles = tiles_m * ((args.N + fused_sums::kTileRows - 1) / fused_sums::kTileRows);
+  if (parts > 1 && tiles * parts > num_cus) return false;
   return !flip && depth_split::StepCount(steps, parts, parts - 1) >= fused_sums::kMinDepthSteps &&
          tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows &&
          mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k256x256;

@@ -1917,9 +1917,10 @@ inline TimingModel TimingModelOf(Model model) {
 // workgroup streams operands that are not in L2 at 80-100 GB/s at best (what
 // its ring keeps in flight over a round trip to memory), so a problem with few
 // tiles and a long depth only gets faster by putting more workgroups on it.
-// Only the smallest tile has the split: adding up the parts costs time in
-// proportion to the tile's area, and with larger tiles that outweighed the
-// gain at every shape measured.
+// Of the tiles on 32x32 blocks only the smallest has the split: adding up the
+// parts costs time in proportion to the tile's area, and with the tiles of 128
+// rows that outweighed the gain at every shape measured. (The 256x256 tile of
+// the int8 kernel has a split of its own, whose parts share that work: below.)
 inline int DepthSplitParts(int tiles, int k_steps, int num_cus, int min_steps_per_part) {
   constexpr int kMaxParts = 32;
   if (tiles <= 0 || tiles > kSplitCounters) return 1;
@@ -1968,15 +1969,44 @@ inline bool ShallowRing(const GemmArgs& args, int num_cus, int bm, int bn) {
 // for destinations of so few tiles that the 256x256 grid leaves most CUs idle,
 // with depths so long that a part still has kLargeSplitMinSteps ring steps.
 // Adding up the parts costs in proportion to the tile's area - every part
-// writes 256 KiB of accumulators, the last to arrive reads those of the
-// others - which one 128x128 tile per CU, at 55 % of the large tile's rate,
-// only loses to beyond depths of about 10000.
+// writes 256 KiB of accumulators and reads those of the others for its share
+// of the tile's columns - which one 128x128 tile per CU, at 55 % of the large
+// tile's rate, only loses to beyond depths of about 10000.
 constexpr int kLargeSplitMinSteps = 16;
-// Microseconds to store a part and to add one other part to one's own.
-constexpr double kLargeSplitStore = 2.5, kLargeSplitAddPart = 2.6;
-inline int LargeSplitPartsWanted(int tiles, int k_steps, int num_cus) {
+// What the exchange of the parts costs: a fixed 1.5 us and 0.18 us per MiB that
+// goes through the memory side of the device (every part stores its 256 KiB,
+// and reads those of the others for its share of the columns: 2 - 1/parts
+// times 256 KiB per workgroup). Fitted to 2048x16384x2048 (64 tiles in 4
+// parts: 112 MiB, 21.7 us), 1024x32768x1024 (16 in 8: 60 MiB, 13.5 us),
+// 1536x16384x1536 (36 in 4) and 2560x16384x2560 (100 in 2).
+constexpr double kLargeSplitFixed = 1.5, kLargeSplitPerMiB = 0.18;
+// The modelled time of the split into `parts` (a whole number of rounds is not
+// needed: the parts all run at once).
+inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps, int parts, int num_cus) {
+  const double fraction = double(tiles * parts) / num_cus;
+  // (A workgroup moves its own (2 - 1/parts) * 256 KiB at 60 GB/s or so: what
+  // the exchange costs at least, however few workgroups there are.)
+  const double mib_per_workgroup = 0.25 * (2.0 - 1.0 / parts);
+  const double exchange = std::max(kLargeSplitPerMiB * tiles * parts * mib_per_workgroup, mib_per_workgroup / 0.06);
+  return t.fixed + (t.last_round + (1 - t.last_round) * fraction) * t.step *
+                       (t.overhead + depth_split::StepsPerPart(k_steps, parts)) +
+         kLargeSplitFixed + exchange;
+}
+// The best number of parts (2, 4, 8) by that model among those that fit the
+// CUs at once and leave every part kLargeSplitMinSteps steps; 1 if none does.
+inline int LargeSplitPartsWanted(const TileTiming& t, int tiles, int k_steps, int num_cus, double* time) {
   if (tiles <= 0 || tiles * depth_split::kLargeWordsPerTile > kSplitCounters) return 1;
-  return depth_split::LargeParts(k_steps, std::min(num_cus / tiles, k_steps / kLargeSplitMinSteps));
+  const int most = std::min(num_cus / tiles, k_steps / kLargeSplitMinSteps);
+  int best = 1;
+  for (int parts = 2; parts <= depth_split::kLargeMaxParts; parts *= 2) {
+    if (parts > most || !depth_split::NoEmptyPart(k_steps, parts)) continue;
+    const double modelled = LargeSplitMicroseconds(t, tiles, k_steps, parts, num_cus);
+    if (best == 1 || modelled < *time) {
+      best = parts;
+      *time = modelled;
+    }
+  }
+  return best;
 }
 
 // The tile a launch should run on, and large_parts > 1 if it should rather run
@@ -2011,15 +2041,22 @@ inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
   if (which == Model::kInt8 && model.tiles[0].tile == Tile::k256x256) {
     const TileTiming& t = model.tiles[0];
     const int tiles = TileCount(args, t.bm, t.bn);
-    const int parts = LargeSplitPartsWanted(tiles, k_steps, num_cus);
-    if (parts > 1) {
-      const double fraction = double(tiles * parts) / num_cus;  // (at most one round)
-      const double time = t.fixed +
-                          (t.last_round + (1 - t.last_round) * fraction) * t.step *
-                              (t.overhead + depth_split::StepsPerPart(k_steps, parts)) +
-                          kLargeSplitStore + kLargeSplitAddPart * (parts - 1);
-      if (time < best_time) large_parts = parts;
+    double time = 0;
+    const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus, &time);
+    // What the split is held against. The smallest tile's step was fitted to
+    // depths of up to 128 steps, mostly short ones; with a workgroup on (nearly)
+    // every CU its step is bound by what L2 delivers (16 KiB per workgroup and
+    // step) and takes 0.25 us, not 0.19: 1024x32768x1024 takes 68.5 us where
+    // the model says 53.
+    double against = best_time;
+    if (best == model.smallest) {
+      const TileTiming& small = model.tiles[model.count - 1];
+      const int small_tiles = TileCount(args, small.bm, small.bn);
+      const int small_parts = DepthSplitParts(small_tiles, k_steps, num_cus, model.min_steps_per_part);
+      const double busy = std::min(1.0, double(small_tiles) * small_parts / num_cus);
+      if (busy >= 0.75) against += 0.06 * depth_split::StepsPerPart(k_steps, small_parts) * busy;
     }
+    if (parts > 1 && time < against) large_parts = parts;
   }
   return {best, large_parts};
 }

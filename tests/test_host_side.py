@@ -200,6 +200,9 @@ def test_tile_choice_of_the_timing_model():
     assert api.tile_for(0, 2048, 16384, 2048) == (256, 256, 4)
     assert api.tile_for(0, 2048, 32768, 1024) == (256, 256, 8)
     assert api.tile_for(0, 2048, 8192, 2048) == (128, 128, 1)   # not worth it at this depth
+    assert api.tile_for(0, 1024, 32768, 1024) == (256, 256, 8)  # ... rather than 256 of the 64x64 tiles
+    assert api.tile_for(0, 1024, 16384, 1024) == (64, 64, 1)
+    assert api.tile_for(0, 2560, 8192, 2560) == (256, 256, 2)
     rows, cols, parts = api.tile_for(2, 64, 32768, 64)
     assert (rows, cols) == (64, 64) and parts > 1
     for kind in (0, 1, 2):
