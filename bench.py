@@ -34,7 +34,9 @@ One JSON line is printed:
 Every entry of `other_configs` (and `gemv`) carries its own roofline and
 cpu_baseline objects. The calls of `other_configs` take microseconds: each is
 measured after its own settling period and over at least 400 calls
-(`calls_timed`), whatever --steps says.
+(`calls_timed`), whatever --steps says. `other_shapes`: the int8 GEMM
+configuration at a few more shapes (OTHER_SHAPES), whole calls, with the tile
+and the number of depth parts the planner picked.
 """
 import argparse
 import ctypes as C
@@ -306,6 +308,38 @@ def bench_gemm(ctx, args):
             problem, ops, "TOP/s", "the full shape M=N=K=%d, every call on all of it" % n, min_secs=0.7,
             repeats=2, min_secs_1_thread=1e-3)
     return problem, out
+
+
+# Other shapes of the int8 GEMM configuration that the default run times
+# (bench_other_shapes): the sizes between the small configurations and the
+# headline, and few large tiles with a very long depth, which the planner puts
+# on the 256x256 tile with its depth dealt to several workgroups.
+OTHER_SHAPES = [(2048, 2048, 2048), (4096, 4096, 4096), (2048, 16384, 2048)]
+
+
+def bench_other_shapes(ctx, args):
+    """Each of OTHER_SHAPES timed like the other configurations: back-to-back
+    asynchronous calls without a per-launch event pair (which would add several
+    microseconds to steps this short), at least 400 of them; with the tile and
+    the number of depth parts the planner picked."""
+    from ruy_amd import api
+    from ruy_amd import workloads as W
+    out = []
+    ctx.set_kernel_timing(False)
+    for M, K, N in OTHER_SHAPES:
+        problem = W.config_int8_gemm_shape(M, K, N)
+        dp = device_problem(problem)
+        dp.run(ctx)
+        calls = max(args.steps, 400)
+        t = time_steps(lambda: dp.run(ctx), calls, args.warmup, ctx, settle=not args.no_settle, events_every=10)
+        rows, cols, parts = api.tile_for(0, M, K, N)
+        out.append({"shape": [M, K, N], "kernel": ctx.last_kernel_name(), "tile": [rows, cols], "depth_parts": parts,
+                    "calls_timed": calls, "us_per_step": t["step_s"] * 1e6, "us_per_step_min": t["step_min_s"] * 1e6,
+                    "stream_us_per_call": t["region_ms"] * 1e3, "TOP/s": problem.ops() / t["step_s"] / 1e12,
+                    "frac_of_int8_peak": problem.ops() / (t["region_ms"] * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS})
+        del dp
+    ctx.set_kernel_timing(True)
+    return out
 
 
 def bench_shape(ctx, args):
@@ -644,6 +678,7 @@ def main():
             line["gemv"] = gv
     if args.workload == "all":
         line["other_configs"] = bench_other_configs(ctx, args)
+        line["other_shapes"] = bench_other_shapes(ctx, args)
     if args.copy_calibration:
         a = torch.full((256 << 20,), 3, dtype=torch.uint8, device="cuda")
         b = torch.empty_like(a)
