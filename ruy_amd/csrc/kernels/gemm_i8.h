@@ -99,6 +99,13 @@ struct GemmArgs {
   // its tile to arrive before it leaves the rest to the last one (0: not at
   // all; what a launch whose parts cannot all run at once should say).
   int32_t split_spin_limit = 0;
+  // What the planner's timing model is told about operand sums that nobody has
+  // formed yet (the int8 kernel; set once, before the first question about the
+  // tile, so that every question gets the same answer): bit 0 = those of a's
+  // rows are wanted, bit 1 = those of b's rows, bit 2 = the 256x256 tile may
+  // form a's inside its launch. A tile that needs a sums kernel in front is
+  // charged for it.
+  int32_t sums_wanted = 0;
 };
 
 // Buffers of the products of a batched launch (GemmArgs holds what they have

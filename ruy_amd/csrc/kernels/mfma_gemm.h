@@ -1823,10 +1823,12 @@ enum class Tile { k256x256, k128x128, k128x64, k64x128, k64x64 };
 // elements, square, oblong and ragged, depths of 2 to 128 steps; each tile
 // timed over 200 calls after the clock had settled, twice, in mirrored order).
 // The fit is within 3-14 % root mean square of the measurements. Picking by
-// it costs 1.0 % of time over always picking the fastest tile on the shapes
-// it was fitted to and 2.2 % (int8), 2 % (fp32) on shapes held out of the fit:
-// among the 128x128, 128x64 and 64x128 tiles the times are often closer than
-// the model is good, and their order changes from card to card.
+// it costs 0.7 % of time over always picking the fastest tile on the shapes
+// it was fitted to (int8, last refitted with the kernels as they are now: 7
+// of 179 shapes lose more than 5 %, the worst 20 %) and about 2 % on shapes
+// held out of the fit: among the 128x128, 128x64 and 64x128 tiles the times
+// are often closer than the model is good, and their order changes from card
+// to card.
 //
 // Workgroups are dealt to the CUs in rounds, and a workgroup costs its ring
 // fill and write-back (`overhead`, in depth steps) plus its depth steps:
@@ -1850,8 +1852,8 @@ enum class Tile { k256x256, k128x128, k128x64, k64x128, k64x64 };
 // discounted as above with `shared_last_round`.
 //
 // What the fit says about the kernels: on int8 the 256x256 tile's depth step
-// (1.12 us) is a third of what the 64x64 tile needs for the same area (16 x
-// 0.191 us) and 58 % of the 128x128 tile's (4 x 0.96 us / 2 side by side), so it
+// (1.16 us) is well under half of what the 64x64 tile needs for the same area
+// (16 x 0.195 us) and 54 % of the 128x128 tile's (4 x 1.07 us / 2 side by side), so it
 // wins whenever its tiles fill most of a round; fp32 is bound by its matrix
 // instructions at every tile size (7.85 us against 16 x 0.562 us) and the small
 // tiles, which fill the CUs more evenly, win up to destinations of 4096^2.
@@ -1876,11 +1878,11 @@ struct TimingModel {
   double reduce;           // microseconds to add up the parts of a split
 };
 constexpr TileTiming kInt8Timings[] = {
-    {Tile::k256x256, 256, 256, 3.17, 8.81, 1.120, 0.81, 1, {}, 0},
-    {Tile::k128x128, 128, 128, 3.99, 3.91, 0.514, 0.89, 2, {0.732, 0.962}, 0.67},
-    {Tile::k128x64, 128, 64, 3.66, 3.02, 0.328, 0.96, 3, {0.470, 0.582, 0.919}, 0.61},
-    {Tile::k64x128, 64, 128, 4.65, 0.06, 0.328, 0.93, 3, {0.503, 0.726, 1.558}, 0.12},
-    {Tile::k64x64, 64, 64, 1.51, 13.95, 0.191, 0.94, 1, {}, 0},
+    {Tile::k256x256, 256, 256, 3.26, 8.27, 1.163, 0.77, 1, {}, 0},
+    {Tile::k128x128, 128, 128, 4.20, 3.70, 0.530, 0.84, 2, {0.610, 1.068}, 0.37},
+    {Tile::k128x64, 128, 64, 3.59, 2.98, 0.333, 0.93, 3, {0.453, 0.607, 0.973}, 0.52},
+    {Tile::k64x128, 64, 128, 4.55, 0.17, 0.334, 0.90, 3, {0.501, 0.742, 1.567}, 0.12},
+    {Tile::k64x64, 64, 64, 1.47, 13.42, 0.195, 0.94, 1, {}, 0},
 };
 constexpr TileTiming kF32Timings[] = {
     {Tile::k256x256, 256, 256, 0.0, 2.21, 7.854, 0.88, 1, {}, 0},
@@ -1905,7 +1907,7 @@ inline TimingModel TimingModelOf(Model model) {
     case Model::kInt8PlaneSplit:
       return {kInt8PlaneSplitTimings, 3, Tile::k64x128, 8, 3.6};
     default:
-      return {kInt8Timings, 5, Tile::k64x64, 16, 2.4};
+      return {kInt8Timings, 5, Tile::k64x64, 16, 2.44};
   }
 }
 
@@ -1927,6 +1929,35 @@ inline int DepthSplitParts(int tiles, int k_steps, int num_cus, int min_steps_pe
   const int parts = std::min({num_cus / tiles, k_steps / min_steps_per_part, kMaxParts});
   if (parts < 2) return 1;
   return depth_split::PartsWithoutEmpty(k_steps, parts);
+}
+
+// Operand sums that nobody has formed yet (GemmArgs::sums_wanted; the int8
+// kernel on operands used in place): what they add to a launch on tile `t`.
+// The 128- and 64-row tiles need a kernel of their own in front, which streams
+// the operand once more (1.5 us + 0.134 us per MiB: 16384 x 16384 in 36 us); the
+// smallest tile forms them with a matrix instruction more per side and
+// sub-step (its step gets 15 % longer, returned in *factor); the 256x256 tile
+// deals those of `a` out over its first workgroups where it may (a microsecond
+// and a half) and needs the kernel for those of `b`.
+inline double SumsKernelMicroseconds(double bytes) { return 1.5 + bytes / (1024.0 * 1024.0) * 0.134; }
+inline double PendingSumsMicroseconds(const GemmArgs& args, const TimingModel& model, const TileTiming& t,
+                                      double* factor) {
+  *factor = 1.0;
+  const bool a = (args.sums_wanted & 1) != 0, b = (args.sums_wanted & 2) != 0;
+  if (!a && !b) return 0.0;
+  if (t.tile == model.smallest) {
+    *factor = 1.15;
+    return 0.0;
+  }
+  const double a_kernel = SumsKernelMicroseconds(double(args.M) * args.k_bytes);
+  const double b_kernel = SumsKernelMicroseconds(double(args.N) * args.k_bytes);
+  double extra = b ? b_kernel : 0.0;
+  if (a) {
+    const bool in_launch = t.tile == Tile::k256x256 && (args.sums_wanted & 4) && !args.a_flip && !args.b_flip &&
+                           args.k_bytes / 128 >= fused_sums::kMinDepthSteps && args.M <= fused_sums::kMaxRows;
+    extra += in_launch ? 1.5 : a_kernel;
+  }
+  return extra;
 }
 
 inline double ModelledMicroseconds(const GemmArgs& args, int num_cus, const TimingModel& model, const TileTiming& t) {
@@ -1951,7 +1982,9 @@ inline double ModelledMicroseconds(const GemmArgs& args, int num_cus, const Timi
     rounds = cu_with(q);
     if (r) rounds += (cu_with(q + 1) - cu_with(q)) * (t.shared_last_round + (1 - t.shared_last_round) * fraction);
   }
-  return t.fixed + rounds * (t.overhead + k_steps) + (parts > 1 ? model.reduce : 0.0);
+  double sums_factor = 1.0;
+  const double sums = PendingSumsMicroseconds(args, model, t, &sums_factor);
+  return t.fixed + sums_factor * rounds * (t.overhead + k_steps) + (parts > 1 ? model.reduce : 0.0) + sums;
 }
 
 // The 128x128, 128x64 and 64x128 tiles come with two ring depths. Four stages
@@ -1982,25 +2015,31 @@ constexpr int kLargeSplitMinSteps = 16;
 constexpr double kLargeSplitFixed = 1.5, kLargeSplitPerMiB = 0.18;
 // The modelled time of the split into `parts` (a whole number of rounds is not
 // needed: the parts all run at once).
-inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps, int parts, int num_cus) {
+inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps, int parts, int num_cus,
+                                     double operand_bytes) {
   const double fraction = double(tiles * parts) / num_cus;
   // (A workgroup moves its own (2 - 1/parts) * 256 KiB at 60 GB/s or so: what
   // the exchange costs at least, however few workgroups there are.)
   const double mib_per_workgroup = 0.25 * (2.0 - 1.0 / parts);
   const double exchange = std::max(kLargeSplitPerMiB * tiles * parts * mib_per_workgroup, mib_per_workgroup / 0.06);
-  return t.fixed + (t.last_round + (1 - t.last_round) * fraction) * t.step *
-                       (t.overhead + depth_split::StepsPerPart(k_steps, parts)) +
-         kLargeSplitFixed + exchange;
+  // The workgroups of this tile keep a step and a half of loads in flight each:
+  // operands that are read once (few tile columns or rows) stream at 3.5 TB/s
+  // at best (16384 x 16384 x 256: 101 us for 260 MiB and the exchange).
+  const double main_loop = (t.last_round + (1 - t.last_round) * fraction) * t.step *
+                           (t.overhead + depth_split::StepsPerPart(k_steps, parts));
+  const double streaming = operand_bytes / 3.5e6;
+  return t.fixed + std::max(main_loop, streaming) + kLargeSplitFixed + exchange;
 }
 // The best number of parts (2, 4, 8) by that model among those that fit the
 // CUs at once and leave every part kLargeSplitMinSteps steps; 1 if none does.
-inline int LargeSplitPartsWanted(const TileTiming& t, int tiles, int k_steps, int num_cus, double* time) {
+inline int LargeSplitPartsWanted(const TileTiming& t, int tiles, int k_steps, int num_cus, double operand_bytes,
+                                 double* time) {
   if (tiles <= 0 || tiles * depth_split::kLargeWordsPerTile > kSplitCounters) return 1;
   const int most = std::min(num_cus / tiles, k_steps / kLargeSplitMinSteps);
   int best = 1;
   for (int parts = 2; parts <= depth_split::kLargeMaxParts; parts *= 2) {
     if (parts > most || !depth_split::NoEmptyPart(k_steps, parts)) continue;
-    const double modelled = LargeSplitMicroseconds(t, tiles, k_steps, parts, num_cus);
+    const double modelled = LargeSplitMicroseconds(t, tiles, k_steps, parts, num_cus, operand_bytes);
     if (best == 1 || modelled < *time) {
       best = parts;
       *time = modelled;
@@ -2042,7 +2081,10 @@ inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
     const TileTiming& t = model.tiles[0];
     const int tiles = TileCount(args, t.bm, t.bn);
     double time = 0;
-    const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus, &time);
+    const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus,
+                                            (double(args.M) + args.N) * args.k_bytes, &time);
+    double unused_factor;
+    time += PendingSumsMicroseconds(args, model, t, &unused_factor);
     // What the split is held against. The smallest tile's step was fitted to
     // depths of up to 128 steps, mostly short ones; with a workgroup on (nearly)
     // every CU its step is bound by what L2 delivers (16 KiB per workgroup and

@@ -309,6 +309,8 @@ bool SetupInt8Gemm(ruyamd_ctx* ctx, const MulCall& call, const Operand8& a, cons
   args.n_logical = args.N;
   args.ep.lhs_zero_point = swap ? rzp : lzp;
   args.ep.rhs_zero_point = swap ? lzp : rzp;
+  args.sums_wanted = (x.sums_pending ? 1 : 0) | (y.sums_pending ? 2 : 0) |
+                     (ctx->row_sums_in_launch && !ctx->capturing && !ctx->no_alloc ? 4 : 0);
   if ((a.sums_pending || b.sums_pending) && GemmI8CanFuseSums(args, ctx->multiprocessor_count)) {
     args.fuse_sums = 1;
     if (x.sums_pending) {
