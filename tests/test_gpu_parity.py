@@ -845,6 +845,7 @@ def test_largest_int8_tile_with_its_depth_split(device_ctx, tup):
         device_ctx.force_tile(0, 0)
     if tup == (S.I8, S.I8, S.I32, S.I8):
         _split_tile_with_sums_in_the_launch(rng)
+        _split_tile_recorded_into_a_graph(rng)
     for shape in [(2048, 16384, 2048), (1024, 16400, 2304)]:
         assert api_tile(*shape)[:2] == (256, 256) and api_tile(*shape)[2] > 1, api_tile(*shape)
         M, K, N = shape
@@ -861,6 +862,48 @@ def test_largest_int8_tile_with_its_depth_split(device_ctx, tup):
             if want is not None:
                 bad = np.nonzero(got != want)[0]
                 assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+
+
+def _split_tile_recorded_into_a_graph(rng):
+    """The split tile's launch recorded into a HIP graph and replayed with
+    fresh right-hand values: the tile's arrival, claim and exit words must be
+    back at zero after every replay, and the parts' buffer (taken from the
+    workspace by the eager call before the capture) stays where it is."""
+    import torch
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    ctx = api.Context()
+    try:
+        stream = torch.cuda.Stream()
+        ctx.set_stream(stream.cuda_stream)
+        ctx.set_synchronous(False)
+        ctx.force_tile(256, 256, 4)
+        p = W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, 300, 4096, 520, *cases.RCC, strided=False,
+                             name="(300, 4096, 520) in 4 parts, recorded")
+        p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+        p.lhs.zero_point, p.rhs.zero_point = 9, -5
+        announce(p.name)
+        dp = D.DeviceProblem(p, dst_fill=0)
+        with torch.cuda.stream(stream):
+            dp.run(ctx)  # (eager: the workspace grows to what the recorded call needs)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            dp.run(ctx)
+        for replay in range(3):
+            lo, hi = S.INT_RANGES[p.rhs.dtype]
+            p.rhs.storage[:] = rng.integers(lo, hi + 1, p.rhs.storage.size).astype(p.rhs.storage.dtype)
+            dp.rhs_t.copy_(torch.from_numpy(p.rhs.storage))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            compare(p, dp.result(), expected(p, fill=0))
+            with torch.cuda.stream(stream):
+                dp.run(ctx)  # an eager call between the replays
+            stream.synchronize()
+            compare(p, dp.result(), expected(p, fill=0))
+    finally:
+        ctx.close()
 
 
 def _split_tile_with_sums_in_the_launch(rng):
