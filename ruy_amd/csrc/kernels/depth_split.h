@@ -117,6 +117,27 @@ RUYAMD_HOST_DEVICE inline bool ClaimSucceeded(unsigned claims_before, int index)
   return (claims_before & ClaimBit(index)) == 0;
 }
 
+// Which tile and part a workgroup of such a launch takes. The hardware deals
+// workgroups to the device's 8 XCDs round-robin by their linear number, and
+// every XCD has an L2 of its own: an XCD gets workgroups of one depth part
+// only, and a contiguous run of the tile order, so that the operand panels in
+// its L2 serve all of them. (Parts of one tile share no operand bytes.)
+// `tile` == total_tiles: a workgroup without work (the grid is rounded up).
+struct LargeSplitWork {
+  int tile;
+  int part;
+};
+RUYAMD_HOST_DEVICE inline LargeSplitWork LargeSplitWorkOf(int linear_workgroup, int total_tiles, int parts) {
+  const int xcd = linear_workgroup & 7, place = linear_workgroup >> 3;
+  const int xcds_per_part = 8 / parts;
+  const int tiles_per_xcd = (total_tiles + xcds_per_part - 1) / xcds_per_part;
+  LargeSplitWork w;
+  w.part = xcd % parts;
+  w.tile = place < tiles_per_xcd ? (xcd / parts) * tiles_per_xcd + place : total_tiles;
+  if (w.tile > total_tiles) w.tile = total_tiles;
+  return w;
+}
+
 }  // namespace depth_split
 }  // namespace ruyamd
 

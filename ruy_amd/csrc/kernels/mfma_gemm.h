@@ -48,6 +48,7 @@
 #include <utility>
 
 #include <algorithm>
+#include <cmath>
 
 #include "../epilogue.h"
 #include "../internal.h"
@@ -262,7 +263,28 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int tiles_n = (args.N + C::kBN - 1) / C::kBN;
   const int total = tiles_m * tiles_n;
   const int per_xcd = (total + 7) / 8;
-  const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  // kSplitLarge (the depth of every tile dealt to args.split_k = 2, 4 or 8
+  // workgroups, all of which run at once): an XCD gets workgroups of ONE
+  // depth part only, and a contiguous run of the tile order of that part, so
+  // that what its L2 holds of the operand panels serves all its workgroups.
+  // (With the tile taken from blockIdx.x and the part from blockIdx.y as for
+  // the small tiles, an XCD holds every part of a few tiles, which share
+  // nothing: 2048 x 16384 x 2048 then fetched 254 MB per launch where the
+  // operands are 67 MB and the parts read back 50 MB.) Workgroups go to the
+  // XCDs round-robin by their linear number.
+  int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  int part_of_workgroup = blockIdx.y;
+  // (Not for a single row or column of tiles, which share one operand's panel
+  // whatever the part: 16384 x 16384 x 256 measured 116 us this way and 107 us
+  // with every part of a tile on one XCD.)
+  if constexpr (kSplitLarge) {
+    if (tiles_m > 1 && tiles_n > 1) {
+      const depth_split::LargeSplitWork work = depth_split::LargeSplitWorkOf(
+          int(blockIdx.y) * int(gridDim.x) + int(blockIdx.x), total, args.split_k);
+      part_of_workgroup = work.part;
+      t = work.tile;
+    }
+  }
   if constexpr (kRowSums) {
     // The sums of the launch after this one: every workgroup clears its share
     // (nothing in this launch looks at them).
@@ -302,7 +324,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // steps only; their accumulators are added up before the write-back (below).
   constexpr bool kCanSplitDepth = (WM * WN <= 2 && kB == 32) || kSplitLarge;
   const int split = kCanSplitDepth ? args.split_k : 1;
-  const int split_index = kCanSplitDepth ? blockIdx.y : 0;
+  const int split_index = kCanSplitDepth ? part_of_workgroup : 0;
   // Divisions run on the vector unit: their results are read back into scalar
   // registers here, so that what derives from them (a load's scalar offset
   // operand among others) is scalar whatever the compiler makes of the
@@ -2027,7 +2049,8 @@ inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps
   // at best (16384 x 16384 x 256: 101 us for 260 MiB and the exchange).
   const double main_loop = (t.last_round + (1 - t.last_round) * fraction) * t.step *
                            (t.overhead + depth_split::StepsPerPart(k_steps, parts));
-  const double streaming = operand_bytes / 3.5e6;
+  // (... with a workgroup on every CU; fewer of them stream less: 2.8 TB/s with 128.)
+  const double streaming = operand_bytes / (3.5e6 * std::sqrt(std::min(1.0, fraction)));
   return t.fixed + std::max(main_loop, streaming) + kLargeSplitFixed + exchange;
 }
 // The best number of parts (2, 4, 8) by that model among those that fit the

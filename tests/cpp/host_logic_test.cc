@@ -250,6 +250,36 @@ struct LargeSplitModel {
   }
 };
 
+// Every (tile, part) of a split launch of the large tile is some workgroup's
+// work exactly once, an XCD sees one part only, and its tiles are a run of the
+// tile order.
+static void TestLargeTileSplitWork() {
+  for (int total = 1; total <= 256; ++total) {
+    const int grid = (total + 7) / 8 * 8;
+    for (int parts = 2; parts <= 8; parts *= 2) {
+      std::vector<int> taken(size_t(total) * parts, 0);
+      int part_of_xcd[8], first_of_xcd[8], count_of_xcd[8] = {};
+      bool ok = true;
+      for (int linear = 0; linear < grid * parts; ++linear) {
+        const ds::LargeSplitWork w = ds::LargeSplitWorkOf(linear, total, parts);
+        ok = ok && w.part >= 0 && w.part < parts && w.tile >= 0 && w.tile <= total;
+        if (!ok || w.tile == total) continue;
+        ++taken[size_t(w.tile) * parts + w.part];
+        const int xcd = linear & 7;
+        if (count_of_xcd[xcd] == 0) {
+          part_of_xcd[xcd] = w.part;
+          first_of_xcd[xcd] = w.tile;
+        }
+        ok = ok && part_of_xcd[xcd] == w.part && w.tile == first_of_xcd[xcd] + count_of_xcd[xcd];
+        ++count_of_xcd[xcd];
+      }
+      for (int x : taken) ok = ok && x == 1;
+      EXPECT(ok);
+      if (!ok) return;
+    }
+  }
+}
+
 static void TestLargeTileSplitProtocol() {
   const int tiles = 5, steps = 40;
   LargeSplitModel model(tiles, steps);
@@ -366,6 +396,7 @@ int main() {
   TestDepthPartsCoverEveryStepOnce();
   TestDepthSplitArrivalProtocol();
   TestLargeTileSplitProtocol();
+  TestLargeTileSplitWork();
   if (g_failures) {
     std::fprintf(stderr, "host_logic_test: %d failure(s)\n", g_failures);
     return 1;
