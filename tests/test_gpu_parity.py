@@ -864,6 +864,41 @@ def test_largest_int8_tile_with_its_depth_split(device_ctx, tup):
                 assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
 
 
+def test_random_deep_and_weight_streaming_products_every_element(device_ctx):
+    """Random shapes of the two families the planner treats specially - few
+    256x256 tiles with a very long depth (the split tile, 2 to 8 parts) and a
+    large left-hand operand with a few dozen to a few hundred destination
+    columns (smallest tile with fused sums, 128-row tiles, the split tile) - in
+    random type tuples, destination orders and zero points, operands in place:
+    every element against the stock reference library (skipped without it)."""
+    from ruy_amd import device_problem as D
+    rng = np.random.default_rng(777)
+    tups = [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.U8, S.I32, S.U8), (S.I8, S.U8, S.I32, S.I32), (S.U8, S.I8, S.I32, S.I16)]
+    done = 0
+    for it in range(14):
+        if it % 2 == 0:
+            M, K, N = (int(rng.integers(2, 11)) * 256 - int(rng.integers(0, 40)), int(rng.integers(96, 250)) * 128,
+                       int(rng.integers(2, 11)) * 256 - int(rng.integers(0, 40)))
+        else:
+            M, K, N = int(rng.integers(16, 60)) * 256, int(rng.integers(16, 60)) * 256, int(rng.integers(17, 300))
+        tup = tups[rng.integers(0, len(tups))]
+        orders = [cases.RCC, (1, 0, 1)][rng.integers(0, 2)]
+        p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
+                             name="%s %s %s" % (cases.tuple_name(tup), (M, K, N), orders))
+        p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+        p.lhs.zero_point = (128 if tup[0] == S.U8 else 0) + int(rng.integers(-9, 10)) * int(rng.integers(0, 2))
+        p.rhs.zero_point = (128 if tup[1] == S.U8 else 0) + int(rng.integers(-9, 10)) * int(rng.integers(0, 2))
+        announce(p.name)
+        want = O.full_size_expected(p)
+        if want is None:
+            pytest.skip("the stock reference library is not built")
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+        done += 1
+    assert done == 14
+
+
 def _split_tile_recorded_into_a_graph(rng):
     """The split tile's launch recorded into a HIP graph and replayed with
     fresh right-hand values: the tile's arrival, claim and exit words must be
