@@ -14,6 +14,13 @@
 // row's sums in global memory with atomic adds. Every workgroup of the row
 // fetches the finished sums shortly before its write-back.
 //
+// uint8 data used in place is flipped to int8 in the fragment registers at
+// its first use in a ring step, so at the point between two ring steps where
+// the registers are added up, the fragments of the step just done are flipped
+// and those of the step to come are not yet: the latter get the flip applied
+// to the dot product's operand (one more v_xor per register), and the sums
+// are those of the int8 values either way.
+//
 // Every workgroup walks the depth forwards, so the share of the last depth
 // steps is only added when the main loops of the contributors end, which is
 // when they themselves need the sums: the workgroups of the first round wait a

@@ -411,7 +411,9 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   // contributors that start when they are gone.
   const int tiles = tiles_m * ((args.N + fused_sums::kTileRows - 1) / fused_sums::kTileRows);
   if (parts > 1 && tiles * parts > num_cus) return false;
-  return !flip && depth_split::StepCount(steps, parts, parts - 1) >= fused_sums::kMinDepthSteps &&
+  // (uint8 data in place needs whole depth steps, which LaunchGemmI8 insists on.)
+  if (flip && args.k_bytes % 128 != 0) return false;
+  return depth_split::StepCount(steps, parts, parts - 1) >= fused_sums::kMinDepthSteps &&
          tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows &&
          mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k256x256;
 }

@@ -228,8 +228,7 @@ struct Cfg {
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false, bool kRowSums = false, bool kSplitLarge = false>
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
-  static_assert(!kRowSums || (Traits::kPaired && !kFlip && !kFusedSums),
-                "row sums in passing exist for the paired schedule on int8 data");
+  static_assert(!kRowSums || (Traits::kPaired && !kFusedSums), "row sums in passing exist for the paired schedule");
   static_assert(!kSplitLarge || Traits::kPaired, "kSplitLarge is the depth split of the paired schedule's tile");
   static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
                 "fused sums exist for the tiles with one block (one block per plane) per wave only");
@@ -990,7 +989,13 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-          for (int d = 0; d < 4; ++d) row_sum[i] = __builtin_amdgcn_sdot4(fa[ks][i][d], 0x01010101, row_sum[i], false);
+          for (int d = 0; d < 4; ++d) {
+            // uint8 data in place: between two ring steps rows 0-3 hold the
+            // step to come as it was read from LDS, rows 4-7 the step just
+            // done, flipped to int8 where that step first used them.
+            const int bytes = kFlip && kFirst == 0 ? fa[ks][i][d] ^ static_cast<int>(args.a_flip) : fa[ks][i][d];
+            row_sum[i] = __builtin_amdgcn_sdot4(bytes, 0x01010101, row_sum[i], false);
+          }
     };
     auto publish = [&]() {
       long long* out = args.row_sums + m0 + wave_m * (WM * 32) + (lane & 15);
@@ -1322,7 +1327,8 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           for (int k = 0; k < args.k_bytes; k += kGranule) {  // (the whole depth, whatever part this workgroup walked)
             const v4i x = *reinterpret_cast<const v4i*>(from + k);
 #pragma unroll
-            for (int d = 0; d < 4; ++d) sum = __builtin_amdgcn_sdot4(x[d], 0x01010101, sum, false);
+            for (int d = 0; d < 4; ++d)
+              sum = __builtin_amdgcn_sdot4(kFlip ? x[d] ^ static_cast<int>(args.a_flip) : x[d], 0x01010101, sum, false);
           }
           edge.sums[h] = sum;
         }
@@ -1975,7 +1981,7 @@ inline double PendingSumsMicroseconds(const GemmArgs& args, const TimingModel& m
   const double b_kernel = SumsKernelMicroseconds(double(args.N) * args.k_bytes);
   double extra = b ? b_kernel : 0.0;
   if (a) {
-    const bool in_launch = t.tile == Tile::k256x256 && (args.sums_wanted & 4) && !args.a_flip && !args.b_flip &&
+    const bool in_launch = t.tile == Tile::k256x256 && (args.sums_wanted & 4) &&
                            args.k_bytes / 128 >= fused_sums::kMinDepthSteps && args.M <= fused_sums::kMaxRows;
     extra += in_launch ? 1.5 : a_kernel;
   }
@@ -2186,11 +2192,11 @@ template <typename Traits, bool kFlip = false>
 hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int num_cus) {
   switch (tile) {
     case Tile::k256x256:
-      if constexpr (Traits::LargeTile::kPaired && !kFlip) {
+      if constexpr (Traits::LargeTile::kPaired) {
         if (args.row_sums && args.split_k > 1)
-          return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, false, false, true, true>(stream, args);
+          return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip, false, true, true>(stream, args);
         if (args.row_sums)
-          return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, false, false, true>(stream, args);
+          return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip, false, true>(stream, args);
       }
       if constexpr (Traits::LargeTile::kPaired) {
         if (args.split_k > 1)

@@ -1131,16 +1131,28 @@ def test_operand_sums_formed_inside_the_launch(mode):
             if want is not None:
                 bad = np.nonzero(got != want)[0]
                 assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
-        # Not while a graph is being recorded and not for uint8 data used in place: the separate kernel.
-        u8 = W.random_problem(rng, S.U8, S.I8, S.I32, S.I8, 4096, 2048, 4096, *cases.RCC, strided=False, name="u8 lhs")
-        u8.lhs.cache_policy = u8.rhs.cache_policy = S.CACHE_NEVER
-        u8.lhs.zero_point, u8.rhs.zero_point = 121, -5
-        announce(u8.name)
-        got = D.device_mul(ctx, u8, dst_fill=0)
-        assert ctx.sums_in_launch_calls() == expected_calls
-        rows, cols = _boundary_sample(rng, 4096, step=128), _boundary_sample(rng, 4096, step=128)
-        g, w = _sample_block(u8, got, rows, cols)
-        assert (g == w).all()
+        # uint8 data used in place (flipped to int8 in the fragment registers: the rows that
+        # are added up between two ring steps are partly flipped already, partly not yet),
+        # either side or both, both destination orders.
+        for tup8, (M, K, N), orders in [((S.U8, S.I8, S.I32, S.I8), (4096, 2048, 4096), cases.RCC),
+                                        ((S.U8, S.U8, S.I32, S.U8), (3900, 2176, 4000), (1, 0, 1)),
+                                        ((S.I8, S.U8, S.I32, S.I16), (4096, 1152, 3072), cases.RCC)]:
+            u8 = W.random_problem(rng, *tup8, M, K, N, *orders, strided=False,
+                                  name="%s %s %s %s" % (cases.tuple_name(tup8), (M, K, N), orders, mode))
+            u8.lhs.cache_policy = u8.rhs.cache_policy = S.CACHE_NEVER
+            u8.lhs.zero_point = 121 if tup8[0] == S.U8 else 9
+            u8.rhs.zero_point = 133 if tup8[1] == S.U8 else -5
+            announce(u8.name)
+            got = D.device_mul(ctx, u8, dst_fill=0)
+            expected_calls += mode != "separate"
+            assert ctx.sums_in_launch_calls() == expected_calls
+            rows, cols = _boundary_sample(rng, M, step=128), _boundary_sample(rng, N, step=128)
+            g, w = _sample_block(u8, got, rows, cols)
+            assert (g == w).all(), "%s: %d mismatches in the sampled block" % (u8.name, (g != w).sum())
+            want = O.full_size_expected(u8)
+            if want is not None:
+                bad = np.nonzero(got != want)[0]
+                assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (u8.name, bad.size, got.size, bad[0])
     finally:
         ctx.close()
 
