@@ -367,11 +367,16 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // the end of the depth are issued too (they fetch zeros) so that the number
   // of loads in flight, which the vmcnt waits count, never depends on K.
   // Load number n (0 .. kLoadsPerStage-1) of depth step kt: A loads first.
-  // All tiles but the largest (grids of few rounds of workgroups): every tile row walks
-  // the depth from its own starting step and wraps around, so that workgroups
-  // running side by side do not ask the same memory channels at the same
-  // time. The order of the steps does not matter for the sums. Steps past the
-  // end keep their index, which puts them out of range as before.
+  // All tiles but the largest, on a single row or column of tiles (a long
+  // operand streamed once against a small one): every tile walks the depth
+  // from its own starting step and wraps around, so that workgroups running
+  // side by side do not ask the same memory channels at the same time. The
+  // order of the steps does not matter for the sums. Steps past the end keep
+  // their index, which puts them out of range as before. (Not on a grid of
+  // rows and columns: tile rows that are at different depths at the same time
+  // find nothing of their column's panel in L2 that another row has brought
+  // in; 2048^3 on 128x128 tiles 17.7 -> 15.7 us without it, 2560^3 29.0 ->
+  // 26.4 us.)
   //
   // k_tiles, kt_first: the steps this workgroup walks.
   const int k_tiles_all = kSplitLarge ? steps_of_part : steps_of_whole_depth;
@@ -379,7 +384,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   const int k_tiles = steps_of_part;
   constexpr bool kRotateDepth = WM * WN < 16;
   const int rot = __builtin_amdgcn_readfirstlane(
-      kRotateDepth && K % kBK == 0 && k_tiles > 0 ? (tile_m * 5 + split_index * 3) % k_tiles : 0);
+      kRotateDepth && K % kBK == 0 && k_tiles > 0 && (tiles_m == 1 || tiles_n == 1)
+          ? ((tile_m + tile_n) * 5 + split_index * 3) % k_tiles
+          : 0);
   // kRowSums: what this wave does for the sums of its rows.
   fused_sums::WaveShare share = {};
   if constexpr (kRowSums) {
@@ -397,8 +404,11 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     const int p = kt + rot;
     return kt >= k_tiles ? k_tiles_all + kt : kt_first + (p >= k_tiles ? p - k_tiles : p);
   };
-  auto issue_one = [&](int kt, int n) {
-    const int kbase = phys(kt) * kBK;
+  // (`kbase`: the byte offset of step kt in the depth, phys(kt) * kBK, which
+  // the callers that deal a step's loads out between matrix instructions work
+  // out once per step: left to every load, the compiler turns the choice
+  // inside phys() into a branch around each of them.)
+  auto issue_one_at = [&](int kt, int n, int kbase) {
     const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
     if (n < C::kALoads) {
       const uint32_t off = (kbase + a_k[n] < K) ? a_goff[n] + kbase : kOutOfRange;
@@ -409,11 +419,11 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, off, b_rsrc);
     }
   };
+  auto issue_one = [&](int kt, int n) { issue_one_at(kt, n, phys(kt) * kBK); };
   // The same for a ring step that lies entirely inside the depth: no
   // per-granule test, and the step's depth offset travels as the instruction's
   // scalar offset, so nothing but the load itself is issued.
-  auto issue_one_full = [&](int kt, int n) {
-    const uint32_t kbase = phys(kt) * kBK;
+  auto issue_one_full_at = [&](int kt, int n, uint32_t kbase) {
     const uint32_t stage = lds_base + (kt % C::kStages) * C::kStageBytes;
     if (n < C::kALoads) {
       LoadToLds16(stage + (wave * C::kALoads + n) * 1024, a_goff[n], kbase, a_rsrc);
@@ -422,6 +432,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, b_goff[i], kbase, b_rsrc);
     }
   };
+  auto issue_one_full = [&](int kt, int n) { issue_one_full_at(kt, n, phys(kt) * kBK); };
   auto issue = [&](int kt) {
 #pragma unroll
     for (int n = 0; n < C::kLoadsPerStage; ++n) issue_one(kt, n);
@@ -502,7 +513,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // second instruction, so that the barrier at the end of a ring step, which
   // waits for every LDS read, finds them done.)
   constexpr int kReadSlots = kB == 16 ? kMmas / 2 : (kMmas < kFrags ? kMmas : kFrags);
-  auto sub_step = [&](const Frags& cur_raw, Frags& next, int kt_next, int ks_next, int kt_dma,
+  auto sub_step = [&](const Frags& cur_raw, Frags& next, int kt_next, int ks_next, int kt_dma, int kbase_dma,
                       auto dma_is_full_step) {
     Frags flipped;
     if constexpr (kFlip) {
@@ -545,9 +556,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         constexpr int kFirst = n * C::kLoadsPerStage / kMmas;
         StaticFor<(n + 1) * C::kLoadsPerStage / kMmas - kFirst>([&](auto l) {
           if (decltype(dma_is_full_step)::value)
-            issue_one_full(kt_dma, kFirst + decltype(l)::value);
+            issue_one_full_at(kt_dma, kFirst + decltype(l)::value, kbase_dma);
           else
-            issue_one(kt_dma, kFirst + decltype(l)::value);
+            issue_one_at(kt_dma, kFirst + decltype(l)::value, kbase_dma);
         });
       }
     });
@@ -650,14 +661,21 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // Depth offset and limit of the b operand in bytes: twice those of `a`
     // when it is int16 data.
     constexpr int kBScale = kRawB ? 2 : 1;
-    auto issue_step = [&](int step, int slot) {
-      const int kbase = phys(step) * kBK;
+    // A step that lies inside the depth: its depth offset travels as the
+    // loads' scalar offset.
+    auto issue_full_step = [&](int step, int slot) {
+      const int kbase = __builtin_amdgcn_readfirstlane(phys(step) * kBK);
       const uint32_t dst = ring_base + slot * kSlotBytes;
-      if (kbase + kBK <= K) {
 #pragma unroll
-        for (int n = 0; n < kLoads; ++n)
-          LoadToLds16(dst + n * 1024, goff[n], uint32_t(n < 8 ? kbase : kBScale * kbase), n < 8 ? a_rsrc : b_rsrc);
+      for (int n = 0; n < kLoads; ++n)
+        LoadToLds16(dst + n * 1024, goff[n], uint32_t(n < 8 ? kbase : kBScale * kbase), n < 8 ? a_rsrc : b_rsrc);
+    };
+    auto issue_step = [&](int step, int slot) {
+      const int kbase = __builtin_amdgcn_readfirstlane(phys(step) * kBK);
+      if (kbase + kBK <= K) {
+        issue_full_step(step, slot);
       } else {
+        const uint32_t dst = ring_base + slot * kSlotBytes;
 #pragma unroll
         for (int n = 0; n < kLoads; ++n) {
           const int scale = n < 8 ? 1 : kBScale;
@@ -738,21 +756,34 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     if (my_steps > 1) issue_step(depth_way + kDepthWays, 1);
     load_edge_params();
     Frags4 fr[2];
-    for (int i = 0; i < my_steps; ++i) {
-      if (i + 1 < my_steps)
-        WaitVmcnt<kLoads>();  // in-order completion: only the next step's loads may be outstanding
-      else
-        WaitVmcnt<0>();
-      const int slot = i & 1;
+    auto walk_slot = [&](int slot) {
       read4(slot, 0, fr[0]);
 #pragma unroll
       for (int ks = 0; ks < C::kKSteps; ++ks) {
         if (ks + 1 < C::kKSteps) read4(slot, ks + 1, fr[(ks + 1) & 1]);
         mma4(fr[ks & 1]);
       }
-      // Every LDS read of the slot has been consumed; refill it.
+      // Every LDS read of the slot has been consumed: it can be refilled.
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      if (i + 2 < my_steps) issue_step(depth_way + kDepthWays * (i + 2), slot);
+    };
+    // The steps whose slot is refilled with a step that lies inside the depth
+    // (only the last step of the whole depth can be a partial one, and the
+    // depth is not rotated then): nothing in their loop is conditional.
+    const int last_is_partial = my_steps > 0 && phys(depth_way + kDepthWays * (my_steps - 1)) * kBK + kBK > K ? 1 : 0;
+    const int refills_of_full_steps = my_steps - 2 - last_is_partial;
+    int i = 0;
+    for (; i < refills_of_full_steps; ++i) {
+      WaitVmcnt<kLoads>();  // in-order completion: only the next step's loads may be outstanding
+      walk_slot(i & 1);
+      issue_full_step(depth_way + kDepthWays * (i + 2), i & 1);
+    }
+    for (; i < my_steps; ++i) {
+      if (i + 1 < my_steps)
+        WaitVmcnt<kLoads>();
+      else
+        WaitVmcnt<0>();
+      walk_slot(i & 1);
+      if (i + 2 < my_steps) issue_step(depth_way + kDepthWays * (i + 2), i & 1);
     }
     if constexpr (kFusedSums) {
       const uint32_t fa = static_cast<uint32_t>(args.fused_a_factor);
@@ -1101,18 +1132,20 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // the whole depth was in the ring from the start, see below).
     auto ring_step = [&](int kt, auto dma_is_full_step, auto parity, auto refill) {
       constexpr int kParity = decltype(parity)::value;
+      const int kbase_dma =
+          decltype(refill)::value ? __builtin_amdgcn_readfirstlane(phys(kt + C::kStages) * kBK) : 0;
 #pragma unroll
       for (int ks = 0; ks < C::kKSteps; ++ks) {
         Frags& cur = f[(kParity + ks) & 1];
         Frags& next = f[(kParity + ks + 1) & 1];
         if (ks + 1 < C::kKSteps) {
-          sub_step(cur, next, kt, ks + 1, -1, dma_is_full_step);
+          sub_step(cur, next, kt, ks + 1, -1, 0, dma_is_full_step);
         } else if constexpr (decltype(refill)::value) {
           WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
           __syncthreads();
-          sub_step(cur, next, kt + 1, 0, kt + C::kStages, dma_is_full_step);
+          sub_step(cur, next, kt + 1, 0, kt + C::kStages, kbase_dma, dma_is_full_step);
         } else {
-          sub_step(cur, next, kt + 1, 0, -1, dma_is_full_step);
+          sub_step(cur, next, kt + 1, 0, -1, 0, dma_is_full_step);
         }
       }
     };
