@@ -399,10 +399,18 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     share.end_step = __builtin_amdgcn_readfirstlane(s.end_step);
     share.expected = __builtin_amdgcn_readfirstlane(s.expected) * split;
   }
+  // Where in the depth the kt-th step that this workgroup walks lies. For a
+  // step that exists (kt < k_tiles) the wrap-around is one unsigned minimum:
+  // p - k_tiles is the smaller of the two exactly when p has passed the end.
+  // (Written as a choice, the compiler branches on it inside the loops.)
+  auto phys_inside = [&](int kt) {
+    if constexpr (!kRotateDepth) return kt;
+    const uint32_t p = uint32_t(kt + rot);
+    return kt_first + int(min(p, p - uint32_t(k_tiles)));
+  };
   auto phys = [&](int kt) {
     if constexpr (!kRotateDepth) return kt;
-    const int p = kt + rot;
-    return kt >= k_tiles ? k_tiles_all + kt : kt_first + (p >= k_tiles ? p - k_tiles : p);
+    return kt >= k_tiles ? k_tiles_all + kt : phys_inside(kt);
   };
   // (`kbase`: the byte offset of step kt in the depth, phys(kt) * kBK, which
   // the callers that deal a step's loads out between matrix instructions work
@@ -664,7 +672,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // A step that lies inside the depth: its depth offset travels as the
     // loads' scalar offset.
     auto issue_full_step = [&](int step, int slot) {
-      const int kbase = __builtin_amdgcn_readfirstlane(phys(step) * kBK);
+      const int kbase = __builtin_amdgcn_readfirstlane(phys_inside(step) * kBK);
       const uint32_t dst = ring_base + slot * kSlotBytes;
 #pragma unroll
       for (int n = 0; n < kLoads; ++n)
@@ -1132,8 +1140,11 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // the whole depth was in the ring from the start, see below).
     auto ring_step = [&](int kt, auto dma_is_full_step, auto parity, auto refill) {
       constexpr int kParity = decltype(parity)::value;
-      const int kbase_dma =
-          decltype(refill)::value ? __builtin_amdgcn_readfirstlane(phys(kt + C::kStages) * kBK) : 0;
+      // (A step that lies inside the depth is one that exists.)
+      const int kbase_dma = !decltype(refill)::value ? 0
+                            : decltype(dma_is_full_step)::value
+                                ? __builtin_amdgcn_readfirstlane(phys_inside(kt + C::kStages) * kBK)
+                                : __builtin_amdgcn_readfirstlane(phys(kt + C::kStages) * kBK);
 #pragma unroll
       for (int ks = 0; ks < C::kKSteps; ++ks) {
         Frags& cur = f[(kParity + ks) & 1];
