@@ -1160,6 +1160,26 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         }
       }
     };
+    // One of the last kStages steps: its slot is not refilled, and of the
+    // loads still in flight those of the `remaining` - 1 steps behind the
+    // next one may stay outstanding.
+    auto last_ring_step = [&](int kt, auto remaining_constant) {
+      constexpr int kRemaining = decltype(remaining_constant)::value;
+#pragma unroll
+      for (int ks = 0; ks < C::kKSteps; ++ks) {
+        Frags& cur = f[ks & 1];
+        Frags& next = f[(ks + 1) & 1];
+        if (ks + 1 < C::kKSteps) {
+          sub_step(cur, next, kt, ks + 1, -1, 0, std::false_type());
+        } else {
+          if constexpr (kRemaining > 0) {
+            WaitVmcnt<(kRemaining - 1) * C::kLoadsPerStage>();
+            __syncthreads();
+          }
+          sub_step(cur, next, kt + 1, 0, -1, 0, std::false_type());
+        }
+      }
+    };
     using Even = std::integral_constant<int, 0>;
     using Odd = std::integral_constant<int, 1>;
     if (C::kKSteps % 2 == 0 && k_tiles <= C::kStages) {
@@ -1185,14 +1205,18 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     __syncthreads();
     read_frags(0, 0, f[0]);
     // While the step whose loads are being issued (kt + kStages) lies entirely
-    // inside the depth, the cheap form of the loads is used; the last few steps
-    // (a partial step and the ones past the end, which fetch zeros) take the
-    // bounds-tested form.
+    // inside the depth, the cheap form of the loads is used; a partial last
+    // step takes the bounds-tested form; the last kStages steps (there are
+    // more than kStages steps here) issue nothing and wait for less and less.
     int kt = 0;
     const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
     if constexpr (C::kKSteps % 2 == 0) {
       for (; kt < full_end; ++kt) ring_step(kt, std::true_type(), Even(), std::true_type());
-      for (; kt < k_tiles; ++kt) ring_step(kt, std::false_type(), Even(), std::true_type());
+      for (; kt < k_tiles - C::kStages; ++kt) ring_step(kt, std::false_type(), Even(), std::true_type());
+      StaticFor<C::kStages>([&](auto j_constant) {
+        constexpr int j = decltype(j_constant)::value;
+        last_ring_step(kt + j, std::integral_constant<int, C::kStages - 1 - j>());
+      });
     } else {
       // One sub-step per ring step: the steps are taken in pairs, so that each
       // finds its fragments in a buffer known at compile time.
