@@ -440,7 +440,6 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       LoadToLds16(stage + C::kBM * kBK + (wave * C::kBLoads + i) * 1024, b_goff[i], kbase, b_rsrc);
     }
   };
-  auto issue_one_full = [&](int kt, int n) { issue_one_full_at(kt, n, phys(kt) * kBK); };
   auto issue = [&](int kt) {
 #pragma unroll
     for (int n = 0; n < C::kLoadsPerStage; ++n) issue_one(kt, n);
