@@ -1197,12 +1197,38 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       read_frags(0, 0, f[0]);
       for (int kt = 0; kt < k_tiles; ++kt) ring_step(kt, std::false_type(), Even(), std::false_type());
     } else {
+    // A ring of four stages starts on two: a wave cannot begin its first
+    // step before it has issued every load in front of it, and with all
+    // workgroups starting at once the address units take as long to accept
+    // four stages as the first takes to arrive. Stages 2 and 3 (which exist
+    // and lie inside the depth: there are more than kStages steps, and only
+    // the last can be a partial one) go out between the matrix instructions
+    // of step 0's first two sub-steps, in the order the waits expect.
+    constexpr bool kStartOnTwoStages = C::kStages == 4 && C::kKSteps == 4;
+    if constexpr (kStartOnTwoStages) {
+      issue(0);
+      load_edge_params();
+      issue(1);
+      WaitVmcnt<C::kLoadsPerStage>();
+    } else {
 #pragma unroll
-    for (int s = 0; s < C::kStages; ++s) issue(s);
-    load_edge_params();
-    WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
+      for (int s = 0; s < C::kStages; ++s) issue(s);
+      load_edge_params();
+      WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
+    }
     __syncthreads();
     read_frags(0, 0, f[0]);
+    auto first_step = [&](auto dma_is_full_step) {
+      sub_step(f[0], f[1], 0, 1, 2, __builtin_amdgcn_readfirstlane(phys_inside(2) * kBK), std::true_type());
+      sub_step(f[1], f[0], 0, 2, 3, __builtin_amdgcn_readfirstlane(phys_inside(3) * kBK), std::true_type());
+      sub_step(f[0], f[1], 0, 3, -1, 0, std::true_type());
+      const int kbase_dma = decltype(dma_is_full_step)::value
+                                ? __builtin_amdgcn_readfirstlane(phys_inside(C::kStages) * kBK)
+                                : __builtin_amdgcn_readfirstlane(phys(C::kStages) * kBK);
+      WaitVmcnt<(C::kStages - 2) * C::kLoadsPerStage>();
+      __syncthreads();
+      sub_step(f[1], f[0], 1, 0, C::kStages, kbase_dma, dma_is_full_step);
+    };
     // While the step whose loads are being issued (kt + kStages) lies entirely
     // inside the depth, the cheap form of the loads is used; a partial last
     // step takes the bounds-tested form; the last kStages steps (there are
@@ -1210,6 +1236,13 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     int kt = 0;
     const int full_end = min(k_tiles, K / kBK - kt_first) - C::kStages;
     if constexpr (C::kKSteps % 2 == 0) {
+      if constexpr (kStartOnTwoStages) {
+        if (full_end > 0)
+          first_step(std::true_type());
+        else
+          first_step(std::false_type());
+        kt = 1;
+      }
       for (; kt < full_end; ++kt) ring_step(kt, std::true_type(), Even(), std::true_type());
       for (; kt < k_tiles - C::kStages; ++kt) ring_step(kt, std::false_type(), Even(), std::true_type());
       StaticFor<C::kStages>([&](auto j_constant) {
