@@ -397,7 +397,11 @@ void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_row
 
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
   const mfma_gemm::TileChoice choice = mfma_gemm::ChooseTile(args, num_cus, mfma_gemm::Model::kInt8);
-  return choice.large_parts == 1 && choice.tile == mfma_gemm::Tile::k64x64;
+  if (choice.large_parts != 1) return false;
+  if (choice.tile == mfma_gemm::Tile::k64x64) return true;
+  // The 128x128 tile forms the row sums of `a`, and only those, in grids of
+  // at most one workgroup per CU.
+  return choice.tile == mfma_gemm::Tile::k128x128 && mfma_gemm::RowSumming128Applies(args, num_cus);
 }
 
 bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
@@ -425,6 +429,9 @@ hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
   if (args.fuse_sums) {
     // Exists for the smallest tile only.
     if (!GemmI8CanFuseSums(args, num_cus)) return hipErrorInvalidValue;
+    if (mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k128x128)
+      return flip ? mfma_gemm::LaunchRowSumming128<Int8Traits, true>(stream, args, num_cus)
+                  : mfma_gemm::LaunchRowSumming128<Int8Traits>(stream, args, num_cus);
     return flip ? mfma_gemm::LaunchSmallestTile<Int8Traits, true, true>(stream, args)
                 : mfma_gemm::LaunchSmallestTile<Int8Traits, true>(stream, args);
   }
@@ -435,7 +442,10 @@ hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {
 hipError_t LaunchGemmI8Batch(hipStream_t stream, const GemmArgs& args, const GemmBatch& batch, int count,
                              int num_cus) {
   const bool flip = args.a_flip != 0 || args.b_flip != 0;
-  if (!GemmI8CanFuseSums(args, num_cus) || (flip && args.k_bytes % 128 != 0)) return hipErrorInvalidValue;
+  // (Batches exist for the smallest tile.)
+  if (mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) != mfma_gemm::Tile::k64x64 ||
+      (flip && args.k_bytes % 128 != 0))
+    return hipErrorInvalidValue;
   if (args.ep.lhs_sums || args.ep.rhs_sums || (!args.fuse_sums && (args.ep.lhs_zero_point || args.ep.rhs_zero_point)))
     return hipErrorInvalidValue;  // sums arrays are per product: only the fused form is batched
   if (flip) {

@@ -230,8 +230,15 @@ template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums =
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   static_assert(!kRowSums || (Traits::kPaired && !kFusedSums), "row sums in passing exist for the paired schedule");
   static_assert(!kSplitLarge || Traits::kPaired, "kSplitLarge is the depth split of the paired schedule's tile");
-  static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))),
-                "fused sums exist for the tiles with one block (one block per plane) per wave only");
+  // kFusedSums on the 128x128 tile (two by two blocks per wave, waves sharing
+  // every step): the row sums of `a` only, one more matrix instruction per
+  // block row and sub-step. That tile's steps wait for LDS, not for the matrix
+  // pipe, as long as a CU holds one workgroup, which is when it is used.
+  constexpr bool kRowSumsOfFourBlocks = kFusedSums && WM == 2 && WN == 2;
+  static_assert(!kFusedSums || (WM == 1 && (WN == 1 || (Traits::kSplitB && WN == 2))) ||
+                    (kRowSumsOfFourBlocks && Traits::kBlock == 32 && !kDepthWaves && !Traits::kSplitB),
+                "fused sums exist for the tiles with one block (one block per plane) per wave, and for the rows of "
+                "the 128x128 tile");
   static_assert(!kFlip || !Traits::kSplitB, "in-place uint8 operands exist for the int8 kernel only");
   static_assert(!kDepthWaves || (WM == 1 && WN == (Traits::kSplitB ? 2 : 1) && BK == 128),
                 "the depth-per-wave schedule exists for the smallest tile of each kernel");
@@ -498,10 +505,12 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   if constexpr (!Traits::kPaired) clear_accumulators();
 
   typename Traits::Acc sum_a, sum_b;  // kFusedSums: row sums of a / column sums of b, in every column / row
+  typename Traits::Acc sum_a_second;  // kRowSumsOfFourBlocks: those of the wave's second block row
 #pragma unroll
   for (int v = 0; v < kAccElems; ++v) {
     sum_a[v] = 0;
     sum_b[v] = 0;
+    sum_a_second[v] = 0;
   }
   const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
 
@@ -550,8 +559,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         // Once per sub-step. The plane-split operand has zero point 0 by
         // definition, so its column sums are never needed.
         Traits::Mma(cur.a[0], ones, sum_a);
-        if constexpr (!Traits::kSplitB) Traits::Mma(ones, cur.b[0], sum_b);
+        if constexpr (!Traits::kSplitB && !kRowSumsOfFourBlocks) Traits::Mma(ones, cur.b[0], sum_b);
       }
+      if constexpr (kRowSumsOfFourBlocks && n == kBB) Traits::Mma(cur.a[1], ones, sum_a_second);
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (!kReadsFirst && n < kReadSlots) {
         constexpr int kFirst = n * kFrags / kReadSlots;
@@ -1273,10 +1283,24 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     // Plane-split operand: the correction belongs to the low plane's block
     // (the write-back combines 256 * high + low).
     constexpr int kBlock = Traits::kSplitB ? 1 : 0;
+    if constexpr (kRowSumsOfFourBlocks) {
+      // (A block of sums has the sum of its row in every column: it lines up
+      // with every accumulator block of that block row.)
 #pragma unroll
-    for (int v = 0; v < 16; ++v)
-      acc[0][kBlock][v] = static_cast<int>(static_cast<uint32_t>(acc[0][kBlock][v]) -
-                                           fa * static_cast<uint32_t>(sum_a[v]) - fb * static_cast<uint32_t>(sum_b[v]));
+      for (int j = 0; j < kBB; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          acc[0][j][v] = static_cast<int>(static_cast<uint32_t>(acc[0][j][v]) - fa * static_cast<uint32_t>(sum_a[v]));
+          acc[1][j][v] =
+              static_cast<int>(static_cast<uint32_t>(acc[1][j][v]) - fa * static_cast<uint32_t>(sum_a_second[v]));
+        }
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        acc[0][kBlock][v] =
+            static_cast<int>(static_cast<uint32_t>(acc[0][kBlock][v]) - fa * static_cast<uint32_t>(sum_a[v]) -
+                             fb * static_cast<uint32_t>(sum_b[v]));
+    }
   }
 
   // ---- depth split: add up the partial accumulators ----
@@ -2068,8 +2092,20 @@ inline int DepthSplitParts(int tiles, int k_steps, int num_cus, int min_steps_pe
 // deals those of `a` out over its first workgroups where it may (a microsecond
 // and a half) and needs the kernel for those of `b`.
 inline double SumsKernelMicroseconds(double bytes) { return 1.5 + bytes / (1024.0 * 1024.0) * 0.134; }
-inline double PendingSumsMicroseconds(const GemmArgs& args, const TimingModel& model, const TileTiming& t,
-                                      double* factor) {
+// The 128x128 tile can form the row sums of `a` itself (one matrix instruction
+// more per block row and sub-step) when only those are pending and the grid
+// leaves every CU at most one workgroup (with two, the matrix pipe is the
+// bound). Measured on 2048 x K x 2048 against the same launch without sums:
+// + 1.0 us at K = 512, + 2.3 us at 2048, + 7.2 us at 8192, where the sums
+// kernel in front costs 2.1, 2.3 and 3.8 us: it pays for short depths.
+inline double RowSumming128Microseconds(int k_steps) { return 0.6 + 0.103 * k_steps; }
+inline bool RowSumming128Applies(const GemmArgs& args, int num_cus) {
+  const int tiles = ((args.M + 127) / 128) * ((args.N + 127) / 128);
+  return (args.sums_wanted & 3) == 1 && tiles <= num_cus &&
+         RowSumming128Microseconds((args.k_bytes + 127) / 128) < SumsKernelMicroseconds(double(args.M) * args.k_bytes);
+}
+inline double PendingSumsMicroseconds(const GemmArgs& args, int num_cus, const TimingModel& model,
+                                      const TileTiming& t, double* factor) {
   *factor = 1.0;
   const bool a = (args.sums_wanted & 1) != 0, b = (args.sums_wanted & 2) != 0;
   if (!a && !b) return 0.0;
@@ -2077,6 +2113,8 @@ inline double PendingSumsMicroseconds(const GemmArgs& args, const TimingModel& m
     *factor = 1.15;
     return 0.0;
   }
+  if (t.tile == Tile::k128x128 && model.smallest == Tile::k64x64 && RowSumming128Applies(args, num_cus))
+    return RowSumming128Microseconds((args.k_bytes + 127) / 128);
   const double a_kernel = SumsKernelMicroseconds(double(args.M) * args.k_bytes);
   const double b_kernel = SumsKernelMicroseconds(double(args.N) * args.k_bytes);
   double extra = b ? b_kernel : 0.0;
@@ -2111,7 +2149,7 @@ inline double ModelledMicroseconds(const GemmArgs& args, int num_cus, const Timi
     if (r) rounds += (cu_with(q + 1) - cu_with(q)) * (t.shared_last_round + (1 - t.shared_last_round) * fraction);
   }
   double sums_factor = 1.0;
-  const double sums = PendingSumsMicroseconds(args, model, t, &sums_factor);
+  const double sums = PendingSumsMicroseconds(args, num_cus, model, t, &sums_factor);
   return t.fixed + sums_factor * rounds * (t.overhead + k_steps) + (parts > 1 ? model.reduce : 0.0) + sums;
 }
 
@@ -2213,7 +2251,7 @@ inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
     const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus,
                                             (double(args.M) + args.N) * args.k_bytes, &time);
     double unused_factor;
-    time += PendingSumsMicroseconds(args, model, t, &unused_factor);
+    time += PendingSumsMicroseconds(args, num_cus, model, t, &unused_factor);
     // What the split is held against. The smallest tile's step was fitted to
     // depths of up to 128 steps, mostly short ones; with a workgroup on (nearly)
     // every CU its step is bound by what L2 delivers (16 KiB per workgroup and
@@ -2286,6 +2324,14 @@ hipError_t LaunchSmallestTileBatch(hipStream_t stream, const GemmArgs& args, con
   if (k_tiles < kDepthWays)
     return LaunchBatch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, false>(stream, args, batch, count);
   return LaunchBatch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, true>(stream, args, batch, count);
+}
+
+// The 128x128 tile with the row sums of `a` formed in the kernel: for grids of
+// at most one workgroup per CU (see kRowSumsOfFourBlocks in the kernel).
+template <typename Traits, bool kFlip = false>
+hipError_t LaunchRowSumming128(hipStream_t stream, const GemmArgs& args, int num_cus) {
+  if (ShallowRing(args, num_cus, 128, 128) || args.split_k > 1) return hipErrorInvalidValue;
+  return Launch<Traits, 2, 2, 128, 4, true, kFlip>(stream, args);
 }
 
 template <typename Traits, bool kFlip = false>

@@ -899,6 +899,38 @@ def test_random_deep_and_weight_streaming_products_every_element(device_ctx):
     assert done == 14
 
 
+def test_row_sums_formed_by_the_128_tile_every_element(device_ctx):
+    """A grid of at most one 128x128 tile per CU with a short depth, one
+    operand's zero point set and that operand's partner used in place: the
+    tile adds up the rows of its `a` side with one more matrix instruction per
+    block row (no sums kernel in front). int8 and uint8 data (flipped in the
+    registers), either destination order (a row-major destination swaps the
+    operands, so the sums are those of the right-hand side's columns), ragged
+    edges: every element against the stock reference library."""
+    from ruy_amd import device_problem as D
+    rng = np.random.default_rng(4242)
+    done = 0
+    for tup, (M, K, N), orders, lzp, rzp in [
+            ((S.I8, S.I8, S.I32, S.I8), (2048, 1024, 2048), cases.RCC, 0, -3),
+            ((S.U8, S.I8, S.I32, S.I16), (1900, 640, 1800), cases.RCC, 128, 7),
+            ((S.I8, S.U8, S.I32, S.U8), (1536, 768, 2000), cases.RCC, 0, 121),
+            ((S.I8, S.I8, S.I32, S.I8), (1800, 512, 2040), (1, 0, 1), -5, 0),
+            ((S.U8, S.U8, S.I32, S.I32), (1280, 896, 1664), (1, 0, 1), 131, 128)]:
+        p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
+                             name="%s %s %s" % (cases.tuple_name(tup), (M, K, N), orders))
+        p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+        p.lhs.zero_point, p.rhs.zero_point = lzp, rzp
+        announce(p.name)
+        want = O.full_size_expected(p)
+        if want is None:
+            pytest.skip("the stock reference library is not built")
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+        done += 1
+    assert done == 5
+
+
 def _split_tile_recorded_into_a_graph(rng):
     """The split tile's launch recorded into a HIP graph and replayed with
     fresh right-hand values: the tile's arrival, claim and exit words must be
