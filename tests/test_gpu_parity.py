@@ -590,6 +590,50 @@ def test_shapes_that_take_the_rectangular_and_large_tiles(device_ctx, tup):
             compare(p, got, want)
 
 
+@pytest.mark.parametrize("tup", [(S.I8, S.I8, S.I32, S.I8), (S.U8, S.I8, S.I32, S.I16), (S.F32, S.F32, S.F32, S.F32)],
+                         ids=cases.tuple_name)
+def test_first_and_last_ring_steps_of_every_tile(tup):
+    """Depths of one to eleven ring steps, with and without a partial last
+    step, on every tile of the shared-step and depth-per-wave schedules (tile
+    forced): the whole depth in the ring, a ring that starts on two of its four
+    stages, the last steps that issue no loads and wait for fewer and fewer,
+    a refill with a partial step. Small grids (the four-stage kernels) and, for
+    the 8-bit tuples, grids of more tiles than CUs (the two-stage kernels)."""
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    rng = np.random.default_rng(31)
+    elt = 4 if tup[0] == S.F32 else 1
+    ctx = api.Context()
+    try:
+        for tile in [(64, 64), (64, 128), (128, 64), (128, 128)]:
+            ctx.force_tile(tile[0], tile[1], 0)
+            for step_bytes in [128, 256 + 16, 3 * 128, 4 * 128, 4 * 128 + 48, 5 * 128, 5 * 128 + 16, 6 * 128, 7 * 128 + 64,
+                               8 * 128, 9 * 128, 11 * 128 + 32]:
+                K = step_bytes // elt
+                p = W.random_problem(rng, *tup, 300, K, 200, *cases.RCC, strided=False,
+                                     name="%s tile %s depth %d bytes" % (cases.tuple_name(tup), tile, step_bytes))
+                p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+                announce(p.name)
+                compare(p, D.device_mul(ctx, p, dst_fill=0), expected(p, fill=0))
+            if tup[0] == S.F32:
+                continue
+            # more tiles than CUs: two workgroups (three) to a CU, rings of two stages
+            for step_bytes in [3 * 128, 5 * 128 + 16]:
+                p = W.random_problem(rng, *tup, 2500, step_bytes, 2300, *cases.RCC, strided=False,
+                                     name="%s tile %s depth %d bytes, large grid" % (cases.tuple_name(tup), tile, step_bytes))
+                p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+                announce(p.name)
+                want = O.full_size_expected(p)
+                if want is None:
+                    continue
+                got = D.device_mul(ctx, p, dst_fill=0)
+                bad = np.nonzero(got != want)[0]
+                assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+    finally:
+        ctx.force_tile(0, 0, 0)
+        ctx.close()
+
+
 def test_two_contexts_on_two_threads():
     """The reference's rule (ruy/ruy.h:82-95): a Context serves one thread, and
     concurrent Mul calls need distinct Contexts. Two threads, each with its own
