@@ -4,6 +4,8 @@
 // MultiplyByQuantizedMultiplier, destination zero point, clamp).
 #include <hip/hip_runtime.h>
 
+#include <tuple>
+
 #include "mfma_gemm.h"
 
 namespace ruyamd {
@@ -417,9 +419,18 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   if (parts > 1 && tiles * parts > num_cus) return false;
   // (uint8 data in place needs whole depth steps, which LaunchGemmI8 insists on.)
   if (flip && args.k_bytes % 128 != 0) return false;
+  const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
+  // The tiles in between: by the workgroups of the grid, each for a share of the rows.
+  for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k128x128, 128, 128},
+                                    std::tuple{mfma_gemm::Tile::k128x64, 128, 64},
+                                    std::tuple{mfma_gemm::Tile::k64x128, 64, 128}}) {
+    if (tile == mid)
+      return parts == 1 && mfma_gemm::LeadSumsApply(args, num_cus, bm, bn) &&
+             mfma_gemm::LeadSumsMicroseconds(args, bm, bn) <
+                 mfma_gemm::SumsKernelMicroseconds(double(args.M) * args.k_bytes);
+  }
   return depth_split::StepCount(steps, parts, parts - 1) >= fused_sums::kMinDepthSteps &&
-         tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows &&
-         mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8) == mfma_gemm::Tile::k256x256;
+         tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows && tile == mfma_gemm::Tile::k256x256;
 }
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {

@@ -228,7 +228,18 @@ struct Cfg {
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false, bool kRowSums = false, bool kSplitLarge = false>
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
-  static_assert(!kRowSums || (Traits::kPaired && !kFusedSums), "row sums in passing exist for the paired schedule");
+  static_assert(!kRowSums || !kFusedSums, "one way of forming the sums at a time");
+  // kRowSums on the tiles of 32x32 blocks whose waves share every step (grids
+  // of at most one workgroup per CU): the rows of `a` are dealt out over the
+  // workgroups of the grid, each of which adds up its few rows from global
+  // memory while its first ring stages are on their way (a 1/256 share of the
+  // operand: some tens of bytes a thread) and puts the sums into the rows'
+  // words (fused_sums.h: one contribution completes a word). Every wave looks
+  // at the words of its rows in front of its write-back, microseconds later;
+  // words that are not complete are read again a bounded number of times,
+  // after which the wave forms the sums of its rows itself.
+  constexpr bool kLeadSums = kRowSums && !Traits::kPaired;
+  static_assert(!kLeadSums || (Traits::kBlock == 32 && !kDepthWaves && !Traits::kSplitB && !kSplitLarge), "");
   static_assert(!kSplitLarge || Traits::kPaired, "kSplitLarge is the depth split of the paired schedule's tile");
   // kFusedSums on the 128x128 tile (two by two blocks per wave, waves sharing
   // every step): the row sums of `a` only, one more matrix instruction per
@@ -301,7 +312,51 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
         __hip_atomic_store(args.row_sums_to_zero + at, 0ll, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  if (t >= total) return;
+  // kLeadSums: this workgroup's share of the rows, by its number in the grid
+  // (workgroups beyond the last tile have a share too).
+  auto add_up_rows_of_share = [&]() {
+    constexpr int kLanesPerRow = 32;
+    constexpr int kRowsPerPass = C::kThreads / kLanesPerRow;
+    const int rows_per_group = (args.M + int(gridDim.x) - 1) / int(gridDim.x);
+    const int first = int(blockIdx.x) * rows_per_group;
+    const int end = min(args.M, first + rows_per_group);
+    const int lane_in_row = threadIdx.x % kLanesPerRow;
+    for (int row = first + int(threadIdx.x) / kLanesPerRow; row < end; row += kRowsPerPass) {
+      const char* from = static_cast<const char*>(args.a) + size_t(row) * size_t(args.lda);
+      int sum = 0;
+      // (The depth is a whole number of 16-byte granules; bytes past it in the
+      // last one are zero.) Eight loads in flight per lane: one after the other
+      // they would take a round trip to memory each.
+      constexpr int kInFlight = 8;
+      for (int k0 = lane_in_row * kGranule; k0 < args.k_bytes; k0 += kInFlight * kLanesPerRow * kGranule) {
+        v4i x[kInFlight];
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j) {
+          const int k = k0 + j * kLanesPerRow * kGranule;
+          x[j] = v4i{0, 0, 0, 0};
+          if (k < args.k_bytes) x[j] = *reinterpret_cast<const v4i*>(from + k);
+        }
+#pragma unroll
+        for (int j = 0; j < kInFlight; ++j) {
+          const bool inside = k0 + j * kLanesPerRow * kGranule < args.k_bytes;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const int bytes = kFlip && inside ? x[j][d] ^ static_cast<int>(args.a_flip) : x[j][d];
+            sum = __builtin_amdgcn_sdot4(bytes, 0x01010101, sum, false);
+          }
+        }
+      }
+#pragma unroll
+      for (int offset = kLanesPerRow / 2; offset > 0; offset /= 2) sum += __shfl_xor(sum, offset, kLanesPerRow);
+      if (lane_in_row == 0)
+        __hip_atomic_fetch_add(args.row_sums + row, fused_sums::Contribution(sum), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+  if (t >= total) {
+    if constexpr (kLeadSums) add_up_rows_of_share();
+    return;
+  }
   constexpr int kGroupM = 4;
   const int band = t / (kGroupM * tiles_n);
   const int band_rows = min(kGroupM, tiles_m - band * kGroupM);
@@ -396,7 +451,8 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           : 0);
   // kRowSums: what this wave does for the sums of its rows.
   fused_sums::WaveShare share = {};
-  if constexpr (kRowSums) {
+  if constexpr (kLeadSums) share.expected = 1;
+  if constexpr (kRowSums && !kLeadSums) {
     // (With the depth split every part's contributors deal out the part's
     // steps; a row's word collects the contributions of all parts.)
     const fused_sums::WaveShare s =
@@ -1201,6 +1257,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
       for (int s = 0; s < C::kStages; ++s)
         if (s < k_tiles) issue(s);
+      if constexpr (kLeadSums) add_up_rows_of_share();
       WaitVmcnt<0>();
       __syncthreads();
       load_edge_params();
@@ -1219,11 +1276,15 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       issue(0);
       load_edge_params();
       issue(1);
+      // (Its loads stand behind those of the ring: waiting for them is waiting
+      // for stage 0, which the first step needs anyway, and for stage 1.)
+      if constexpr (kLeadSums) add_up_rows_of_share();
       WaitVmcnt<C::kLoadsPerStage>();
     } else {
 #pragma unroll
       for (int s = 0; s < C::kStages; ++s) issue(s);
       load_edge_params();
+      if constexpr (kLeadSums) add_up_rows_of_share();
       WaitVmcnt<(C::kStages - 1) * C::kLoadsPerStage>();
     }
     __syncthreads();
@@ -1730,6 +1791,41 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // every column it writes: their parameters are read once, here.
   static_assert(kDepthWaves ? 4 * 2 * 128 * BK >= C::kEpilogueBytes + C::kParamBytes : true, "");
   int* const area = reinterpret_cast<int*>(lds + C::kEpilogueBytes) + wave * Traits::kParamInts;
+  if constexpr (kLeadSums) {
+    // The sums of the two rows whose parameters this lane stages (rows l and
+    // l + 64 from the wave's first), complete or not.
+    const int first_row = m0 + wave_m * (WM * 32);
+    const int row_of[2] = {min(first_row + lane, args.M - 1), min(first_row + 64 + lane, args.M - 1)};
+    long long word[2] = {0, 0};
+    bool ready = false;
+    for (int looks = 0; !ready && looks < args.row_sums_spin_limit; ++looks) {
+      if (looks) __builtin_amdgcn_s_sleep(8);
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        word[h] = __hip_atomic_load(args.row_sums + row_of[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ready = __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
+                    fused_sums::ContributionsIn(word[1]) == share.expected);
+    }
+    if (ready) {
+      edge.sums[0] = fused_sums::SumIn(word[0]);
+      edge.sums[1] = fused_sums::SumIn(word[1]);
+    } else {
+      // (Workgroups that never got to run, on a device shared with somebody
+      // else's work, must not be waited for without end.)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const char* from = static_cast<const char*>(args.a) + size_t(row_of[h]) * size_t(args.lda);
+        int sum = 0;
+        for (int k = 0; k < args.k_bytes; k += kGranule) {
+          const v4i x = *reinterpret_cast<const v4i*>(from + k);
+#pragma unroll
+          for (int d = 0; d < 4; ++d)
+            sum = __builtin_amdgcn_sdot4(kFlip ? x[d] ^ static_cast<int>(args.a_flip) : x[d], 0x01010101, sum, false);
+        }
+        edge.sums[h] = sum;
+      }
+    }
+  }
   Traits::Stage(ep, edge, area, lane);
   typename Traits::RowState rows;
   rows.Read(area, chunk * 16);
@@ -2099,9 +2195,24 @@ inline double SumsKernelMicroseconds(double bytes) { return 1.5 + bytes / (1024.
 // + 1.0 us at K = 512, + 2.3 us at 2048, + 7.2 us at 8192, where the sums
 // kernel in front costs 2.1, 2.3 and 3.8 us: it pays for short depths.
 inline double RowSumming128Microseconds(int k_steps) { return 0.6 + 0.103 * k_steps; }
+// The tiles of 32x32 blocks whose waves share every step can have the rows of
+// `a` added up by the workgroups of their own grid, each taking a share of
+// the rows while its first loads are on their way (kLeadSums in the kernel),
+// where the caller allows sums formed inside a launch (bit 4 of sums_wanted)
+// and the grid leaves every CU at most one workgroup, so that all of them run
+// at once. A workgroup reads its share at some 100 GB/s.
+inline bool LeadSumsApply(const GemmArgs& args, int num_cus, int bm, int bn) {
+  const int tiles = ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
+  return (args.sums_wanted & 1) && (args.sums_wanted & 4) && tiles <= num_cus && args.M <= fused_sums::kMaxRows;
+}
+inline double LeadSumsMicroseconds(const GemmArgs& args, int bm, int bn) {
+  const int tiles = ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
+  const int groups = (tiles + 7) / 8 * 8;
+  return 0.5 + double(args.M) * args.k_bytes / groups / 100e3;
+}
 inline bool RowSumming128Applies(const GemmArgs& args, int num_cus) {
   const int tiles = ((args.M + 127) / 128) * ((args.N + 127) / 128);
-  return (args.sums_wanted & 3) == 1 && tiles <= num_cus &&
+  return (args.sums_wanted & 3) == 1 && tiles <= num_cus && !LeadSumsApply(args, num_cus, 128, 128) &&
          RowSumming128Microseconds((args.k_bytes + 127) / 128) < SumsKernelMicroseconds(double(args.M) * args.k_bytes);
 }
 inline double PendingSumsMicroseconds(const GemmArgs& args, int num_cus, const TimingModel& model,
@@ -2118,6 +2229,8 @@ inline double PendingSumsMicroseconds(const GemmArgs& args, int num_cus, const T
   const double a_kernel = SumsKernelMicroseconds(double(args.M) * args.k_bytes);
   const double b_kernel = SumsKernelMicroseconds(double(args.N) * args.k_bytes);
   double extra = b ? b_kernel : 0.0;
+  if (a && model.smallest == Tile::k64x64 && t.tile != Tile::k256x256 && LeadSumsApply(args, num_cus, t.bm, t.bn))
+    return extra + std::min(a_kernel, LeadSumsMicroseconds(args, t.bm, t.bn));
   if (a) {
     const bool in_launch = t.tile == Tile::k256x256 && (args.sums_wanted & 4) &&
                            args.k_bytes / 128 >= fused_sums::kMinDepthSteps && args.M <= fused_sums::kMaxRows;
@@ -2352,10 +2465,16 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
     case Tile::k128x128:
       if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128))
         return Launch<Traits, 2, 2, 128, 2, false, kFlip>(stream, args);
+      if constexpr (Traits::kModel == Model::kInt8) {
+        if (args.row_sums) return Launch<Traits, 2, 2, 128, 4, false, kFlip, false, true>(stream, args);
+      }
       return Launch<Traits, 2, 2, 128, 4, false, kFlip>(stream, args);
     case Tile::k64x128:
       if constexpr (Traits::kSplitB) return LaunchSmallestTile<Traits>(stream, args);
       if (ShallowRing(args, num_cus, 64, 128)) return Launch<Traits, 1, 2, 128, 2, false, kFlip>(stream, args);
+      if constexpr (Traits::kModel == Model::kInt8) {
+        if (args.row_sums) return Launch<Traits, 1, 2, 128, 4, false, kFlip, false, true>(stream, args);
+      }
       return Launch<Traits, 1, 2, 128, 4, false, kFlip>(stream, args);
     default:
       break;
@@ -2364,6 +2483,9 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
     switch (tile) {
       case Tile::k128x64:
         if (ShallowRing(args, num_cus, 128, 64)) return Launch<Traits, 2, 1, 128, 2, false, kFlip>(stream, args);
+        if constexpr (Traits::kModel == Model::kInt8) {
+          if (args.row_sums) return Launch<Traits, 2, 1, 128, 4, false, kFlip, false, true>(stream, args);
+        }
         return Launch<Traits, 2, 1, 128, 4, false, kFlip>(stream, args);
       default:
         return LaunchSmallestTile<Traits, false, kFlip>(stream, args);

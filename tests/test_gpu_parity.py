@@ -943,6 +943,54 @@ def test_random_deep_and_weight_streaming_products_every_element(device_ctx):
     assert done == 14
 
 
+@pytest.mark.parametrize("mode", ["in launch", "own", "separate"])
+def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
+    """Grids of at most one 128x128, 128x64 or 64x128 tile per CU: the rows of
+    the `a` operand are dealt out over the grid's workgroups, which add them up
+    from global memory while their first loads are on their way; every wave
+    picks up the sums of its rows in front of its write-back. Modes: that; the
+    sums never looked for, so that every wave forms those of its rows itself
+    (what it does when the others' do not arrive); the separate kernel (and,
+    for a short depth on the 128x128 tile, the extra matrix instruction).
+    int8 and uint8 data, both destination orders, ragged edges, calls of
+    different heights in a row on one context (each launch meets the words the
+    launch before cleared for it): every element against the stock library."""
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    ctx = api.Context()
+    try:
+        ctx.set_sums_in_launch({"in launch": 1, "own": 1, "separate": 0}[mode], 0 if mode == "own" else -1)
+        rng = np.random.default_rng(515)
+        calls = 0
+        for tup, (M, K, N), orders, lzp, rzp in [
+                ((S.I8, S.I8, S.I32, S.I8), (2048, 2048, 2048), cases.RCC, 0, -3),       # 128x128, 256 tiles
+                ((S.U8, S.I8, S.I32, S.I16), (1900, 3072, 1800), cases.RCC, 128, 7),     # uint8 rows, ragged
+                ((S.I8, S.I8, S.I32, S.I8), (1280, 4096, 1280), (1, 0, 1), -5, 0),       # operands swapped
+                ((S.I8, S.U8, S.I32, S.U8), (1024, 1024, 1024), cases.RCC, 3, 121),      # both sides' sums
+                ((S.I8, S.I8, S.I32, S.I32), (3000, 2560, 600), cases.RCC, 0, 11),       # a tall grid
+                ((S.U8, S.U8, S.I32, S.U8), (640, 1152, 3100), (1, 0, 1), 131, 128),     # a wide one
+                ((S.I8, S.I8, S.I32, S.I8), (2048, 1024, 2048), cases.RCC, 0, -3)]:      # short depth
+            p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
+                                 name="%s %s %s %s" % (cases.tuple_name(tup), (M, K, N), orders, mode))
+            p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+            p.lhs.zero_point, p.rhs.zero_point = lzp, rzp
+            announce(p.name)
+            want = O.full_size_expected(p)
+            if want is None:
+                pytest.skip("the stock reference library is not built")
+            before = ctx.sums_in_launch_calls()
+            got = D.device_mul(ctx, p, dst_fill=0)
+            calls += ctx.sums_in_launch_calls() - before
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+        if mode == "separate":
+            assert calls == 0
+        else:
+            assert calls >= 4, calls   # (the planner may give some of the shapes to other tiles)
+    finally:
+        ctx.close()
+
+
 def test_row_sums_formed_by_the_128_tile_every_element(device_ctx):
     """A grid of at most one 128x128 tile per CU with a short depth, one
     operand's zero point set and that operand's partner used in place: the
