@@ -65,7 +65,7 @@ struct GemmArgs {
   int32_t split_k = 1;
   void* split_partials = nullptr;
   uint32_t* split_counters = nullptr;
-  // int8 kernel, largest tile only (GemmI8CanFormRowSums): with row_sums set
+  // int8 kernel (GemmI8CanFormRowSums): with row_sums set
   // the kernel forms the depth sums of a's rows itself (fused_sums.h), in
   // row_sums (one 64-bit word per row, rounded up to whole tiles: sum and
   // number of contributions), zero when the launch starts, and reads them
@@ -85,6 +85,10 @@ struct GemmArgs {
   // many depth steps (fused_sums::StepsPerWave): the kernel need not work
   // either out.
   int32_t row_sums_uniform_run = 0;
+  // The tiles of 32x32 blocks (the rows dealt out over the grid's workgroups):
+  // the first row_sums_producers workgroups of the grid, which all run at
+  // once, take a share of the rows each.
+  int32_t row_sums_producers = 0;
   // Diagnostics/tests: not 0 = run on the tile of (forced_tile_rows x
   // forced_tile_cols) whatever the timing model says, if the kernel has it.
   int32_t forced_tile_rows = 0;
@@ -145,6 +149,9 @@ bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus);
 // b_flip are looked at) on its largest tile in the form that can also produce
 // the depth sums of a's rows (GemmArgs::row_sums).
 bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus);
+// For GemmArgs::row_sums_producers: how many workgroups of the launch share the
+// rows out among themselves (0: the largest tile, which has its own scheme).
+int GemmI8RowSumsProducers(const GemmArgs& args, int num_cus);
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
 // `count` <= kGemmBatchMax products of the shape and parameters of `args`, each
 // on its own buffers, in one launch. Only for arguments that run on the

@@ -426,11 +426,19 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
                                     std::tuple{mfma_gemm::Tile::k64x128, 64, 128}}) {
     if (tile == mid)
       return parts == 1 && mfma_gemm::LeadSumsApply(args, num_cus, bm, bn) &&
-             mfma_gemm::LeadSumsMicroseconds(args, bm, bn) <
+             mfma_gemm::LeadSumsMicroseconds(args, num_cus, bm, bn) <
                  mfma_gemm::SumsKernelMicroseconds(double(args.M) * args.k_bytes);
   }
   return depth_split::StepCount(steps, parts, parts - 1) >= fused_sums::kMinDepthSteps &&
          tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows && tile == mfma_gemm::Tile::k256x256;
+}
+
+int GemmI8RowSumsProducers(const GemmArgs& args, int num_cus) {
+  const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
+  if (tile == mfma_gemm::Tile::k128x128) return mfma_gemm::LeadSumsProducers(args, num_cus, 128, 128);
+  if (tile == mfma_gemm::Tile::k128x64) return mfma_gemm::LeadSumsProducers(args, num_cus, 128, 64);
+  if (tile == mfma_gemm::Tile::k64x128) return mfma_gemm::LeadSumsProducers(args, num_cus, 64, 128);
+  return 0;
 }
 
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus) {

@@ -313,11 +313,15 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     }
   }
   // kLeadSums: this workgroup's share of the rows, by its number in the grid
-  // (workgroups beyond the last tile have a share too).
+  // (workgroups beyond the last tile have a share too): the first
+  // args.row_sums_producers workgroups, which the hardware starts first and
+  // which all fit the device at once, deal the rows out among themselves.
   auto add_up_rows_of_share = [&]() {
     constexpr int kLanesPerRow = 32;
     constexpr int kRowsPerPass = C::kThreads / kLanesPerRow;
-    const int rows_per_group = (args.M + int(gridDim.x) - 1) / int(gridDim.x);
+    const int producers = args.row_sums_producers;
+    if (int(blockIdx.x) >= producers) return;
+    const int rows_per_group = (args.M + producers - 1) / producers;
     const int first = int(blockIdx.x) * rows_per_group;
     const int end = min(args.M, first + rows_per_group);
     const int lane_in_row = threadIdx.x % kLanesPerRow;
@@ -2033,6 +2037,8 @@ hipError_t Launch(hipStream_t stream, const GemmArgs& args) {
   if (kRowSums && (!args.row_sums_to_zero || tiles_m * C::kBM > fused_sums::kMaxRows ||
                    args.row_sums_zero_rows > fused_sums::kMaxRows))
     return hipErrorInvalidValue;
+  if (kRowSums && !Traits::kPaired && (args.row_sums_producers <= 0 || args.row_sums_producers > grid))
+    return hipErrorInvalidValue;
   if (lds_bytes > 48 * 1024) {
     // Once per process; static initialisation is safe against concurrent callers.
     static const hipError_t attr = hipFuncSetAttribute(
@@ -2198,17 +2204,22 @@ inline double RowSumming128Microseconds(int k_steps) { return 0.6 + 0.103 * k_st
 // The tiles of 32x32 blocks whose waves share every step can have the rows of
 // `a` added up by the workgroups of their own grid, each taking a share of
 // the rows while its first loads are on their way (kLeadSums in the kernel),
-// where the caller allows sums formed inside a launch (bit 4 of sums_wanted)
-// and the grid leaves every CU at most one workgroup, so that all of them run
-// at once. A workgroup reads its share at some 100 GB/s.
-inline bool LeadSumsApply(const GemmArgs& args, int num_cus, int bm, int bn) {
-  const int tiles = ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
-  return (args.sums_wanted & 1) && (args.sums_wanted & 4) && tiles <= num_cus && args.M <= fused_sums::kMaxRows;
+// where the caller allows sums formed inside a launch (bit 4 of sums_wanted).
+// A workgroup reads its share at some 100 GB/s.
+inline bool LeadSumsApply(const GemmArgs& args, int, int, int) {
+  return (args.sums_wanted & 1) && (args.sums_wanted & 4) && args.M <= fused_sums::kMaxRows;
 }
-inline double LeadSumsMicroseconds(const GemmArgs& args, int bm, int bn) {
+// The workgroups that share the rows out: those of the grid's first round (a
+// grid of more tiles than CUs runs on the rings of two stages, two workgroups
+// of the 128x128 tile or three of the 128x64 and 64x128 tiles to a CU).
+inline int LeadSumsProducers(const GemmArgs& args, int num_cus, int bm, int bn) {
   const int tiles = ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
-  const int groups = (tiles + 7) / 8 * 8;
-  return 0.5 + double(args.M) * args.k_bytes / groups / 100e3;
+  const int grid = (tiles + 7) / 8 * 8;
+  const int per_cu = tiles <= num_cus ? 1 : (bm == 128 && bn == 128 ? 2 : 3);
+  return std::min(grid, num_cus * per_cu);
+}
+inline double LeadSumsMicroseconds(const GemmArgs& args, int num_cus, int bm, int bn) {
+  return 0.5 + double(args.M) * args.k_bytes / LeadSumsProducers(args, num_cus, bm, bn) / 100e3;
 }
 inline bool RowSumming128Applies(const GemmArgs& args, int num_cus) {
   const int tiles = ((args.M + 127) / 128) * ((args.N + 127) / 128);
@@ -2230,7 +2241,7 @@ inline double PendingSumsMicroseconds(const GemmArgs& args, int num_cus, const T
   const double b_kernel = SumsKernelMicroseconds(double(args.N) * args.k_bytes);
   double extra = b ? b_kernel : 0.0;
   if (a && model.smallest == Tile::k64x64 && t.tile != Tile::k256x256 && LeadSumsApply(args, num_cus, t.bm, t.bn))
-    return extra + std::min(a_kernel, LeadSumsMicroseconds(args, t.bm, t.bn));
+    return extra + std::min(a_kernel, LeadSumsMicroseconds(args, num_cus, t.bm, t.bn));
   if (a) {
     const bool in_launch = t.tile == Tile::k256x256 && (args.sums_wanted & 4) &&
                            args.k_bytes / 128 >= fused_sums::kMinDepthSteps && args.M <= fused_sums::kMaxRows;
@@ -2463,18 +2474,22 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
       }
       return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip>(stream, args);
     case Tile::k128x128:
-      if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128))
-        return Launch<Traits, 2, 2, 128, 2, false, kFlip>(stream, args);
       if constexpr (Traits::kModel == Model::kInt8) {
+        if (args.row_sums && ShallowRing(args, num_cus, 128, 128))
+          return Launch<Traits, 2, 2, 128, 2, false, kFlip, false, true>(stream, args);
         if (args.row_sums) return Launch<Traits, 2, 2, 128, 4, false, kFlip, false, true>(stream, args);
       }
+      if (!Traits::kSplitB && ShallowRing(args, num_cus, 128, 128))
+        return Launch<Traits, 2, 2, 128, 2, false, kFlip>(stream, args);
       return Launch<Traits, 2, 2, 128, 4, false, kFlip>(stream, args);
     case Tile::k64x128:
       if constexpr (Traits::kSplitB) return LaunchSmallestTile<Traits>(stream, args);
-      if (ShallowRing(args, num_cus, 64, 128)) return Launch<Traits, 1, 2, 128, 2, false, kFlip>(stream, args);
       if constexpr (Traits::kModel == Model::kInt8) {
+        if (args.row_sums && ShallowRing(args, num_cus, 64, 128))
+          return Launch<Traits, 1, 2, 128, 2, false, kFlip, false, true>(stream, args);
         if (args.row_sums) return Launch<Traits, 1, 2, 128, 4, false, kFlip, false, true>(stream, args);
       }
+      if (ShallowRing(args, num_cus, 64, 128)) return Launch<Traits, 1, 2, 128, 2, false, kFlip>(stream, args);
       return Launch<Traits, 1, 2, 128, 4, false, kFlip>(stream, args);
     default:
       break;
@@ -2482,10 +2497,12 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
   if constexpr (!Traits::kSplitB) {
     switch (tile) {
       case Tile::k128x64:
-        if (ShallowRing(args, num_cus, 128, 64)) return Launch<Traits, 2, 1, 128, 2, false, kFlip>(stream, args);
         if constexpr (Traits::kModel == Model::kInt8) {
+          if (args.row_sums && ShallowRing(args, num_cus, 128, 64))
+            return Launch<Traits, 2, 1, 128, 2, false, kFlip, false, true>(stream, args);
           if (args.row_sums) return Launch<Traits, 2, 1, 128, 4, false, kFlip, false, true>(stream, args);
         }
+        if (ShallowRing(args, num_cus, 128, 64)) return Launch<Traits, 2, 1, 128, 2, false, kFlip>(stream, args);
         return Launch<Traits, 2, 1, 128, 4, false, kFlip>(stream, args);
       default:
         return LaunchSmallestTile<Traits, false, kFlip>(stream, args);

@@ -416,6 +416,7 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     args.row_sums_zero_rows = ctx->row_sums_dirty_rows[set ^ 1];
     args.row_sums_spin_limit = ctx->row_sums_spin_limit;
     args.row_sums_fetch_late = ctx->row_sums_fetch_late;
+    args.row_sums_producers = GemmI8RowSumsProducers(args, ctx->multiprocessor_count);
     const int tiles_m = (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
     const int tiles_n = (args.N + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
     if (args.split_k == 1 && fused_sums::FirstContributorIsZero(tiles_m, tiles_n))

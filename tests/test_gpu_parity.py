@@ -945,9 +945,9 @@ def test_random_deep_and_weight_streaming_products_every_element(device_ctx):
 
 @pytest.mark.parametrize("mode", ["in launch", "own", "separate"])
 def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
-    """Grids of at most one 128x128, 128x64 or 64x128 tile per CU: the rows of
-    the `a` operand are dealt out over the grid's workgroups, which add them up
-    from global memory while their first loads are on their way; every wave
+    """Grids of 128x128, 128x64 or 64x128 tiles: the rows of the `a` operand
+    are dealt out over the workgroups of the grid's first round, which add them
+    up from global memory while their first loads are on their way; every wave
     picks up the sums of its rows in front of its write-back. Modes: that; the
     sums never looked for, so that every wave forms those of its rows itself
     (what it does when the others' do not arrive); the separate kernel (and,
@@ -969,7 +969,11 @@ def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
                 ((S.I8, S.U8, S.I32, S.U8), (1024, 1024, 1024), cases.RCC, 3, 121),      # both sides' sums
                 ((S.I8, S.I8, S.I32, S.I32), (3000, 2560, 600), cases.RCC, 0, 11),       # a tall grid
                 ((S.U8, S.U8, S.I32, S.U8), (640, 1152, 3100), (1, 0, 1), 131, 128),     # a wide one
-                ((S.I8, S.I8, S.I32, S.I8), (2048, 1024, 2048), cases.RCC, 0, -3)]:      # short depth
+                ((S.I8, S.I8, S.I32, S.I8), (2048, 1024, 2048), cases.RCC, 0, -3),       # short depth
+                # more tiles than CUs (rings of two stages): the first round's workgroups share the rows out
+                ((S.I8, S.I8, S.I32, S.I8), (2560, 2560, 2560), cases.RCC, 0, -3),       # 400 tiles, one round
+                ((S.U8, S.I8, S.I32, S.I8), (3000, 1024, 3072), cases.RCC, 128, 9),      # 576 tiles, two rounds
+                ((S.I8, S.I8, S.I32, S.I16), (4096, 1024, 1000), (1, 0, 1), 4, 0)]:      # swapped, a wide grid
             p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
                                  name="%s %s %s %s" % (cases.tuple_name(tup), (M, K, N), orders, mode))
             p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
@@ -986,7 +990,7 @@ def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
         if mode == "separate":
             assert calls == 0
         else:
-            assert calls >= 4, calls   # (the planner may give some of the shapes to other tiles)
+            assert calls >= 6, calls   # (the planner may give some of the shapes to other tiles)
     finally:
         ctx.close()
 
