@@ -287,10 +287,10 @@ RUYAMD_API int ruyamd_ctx_force_tile(ruyamd_ctx* ctx, int tile_rows, int tile_co
 /* Operand sums formed inside the launch of the product (no counterpart in
  * the reference, whose Pack forms them in the pass that already touches the
  * data, ruy/pack.h:105-132): by the largest int8 tile in passing, and by the
- * workgroups of the first round of a grid of 128- or 64-row tiles. On by
- * default: an 8-bit product whose left-hand rows (as the kernel
- * sees them) need their depth sums is then one launch instead of a sums
- * kernel followed by the product. `enable` 0
+ * workgroups of the first round of a grid of 128- or 64-row tiles (either
+ * operand's). On by default: an 8-bit product whose operands need their depth
+ * sums is then one launch instead of one or two sums kernels followed by the
+ * product. `enable` 0
  * restores the separate kernel; 2 is 1 with no wave fetching the sums ahead of
  * the end of its main loop. `spin_limit`: how often a wave that finds the sums
  * unfinished after its main loop looks again before it forms the sums of its

@@ -89,6 +89,11 @@ struct GemmArgs {
   // the first row_sums_producers workgroups of the grid, which all run at
   // once, take a share of the rows each.
   int32_t row_sums_producers = 0;
+  // The same tiles: which operands' depth sums the workgroups form (1: the
+  // rows of a, 2: those of b, 3: both). The words of b's N rows stand
+  // col_sums_offset words behind those of a's rows in row_sums.
+  int32_t row_sums_sides = 1;
+  int32_t col_sums_offset = 0;
   // Diagnostics/tests: not 0 = run on the tile of (forced_tile_rows x
   // forced_tile_cols) whatever the timing model says, if the kernel has it.
   int32_t forced_tile_rows = 0;
@@ -152,6 +157,10 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus);
 // For GemmArgs::row_sums_producers: how many workgroups of the launch share the
 // rows out among themselves (0: the largest tile, which has its own scheme).
 int GemmI8RowSumsProducers(const GemmArgs& args, int num_cus);
+// Whether the launch should also form the depth sums of b's rows (the tiles of
+// 128 and 64 rows only), and where their words then stand in row_sums.
+bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus);
+int GemmI8ColumnSumsOffset(const GemmArgs& args);
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
 // `count` <= kGemmBatchMax products of the shape and parameters of `args`, each
 // on its own buffers, in one launch. Only for arguments that run on the

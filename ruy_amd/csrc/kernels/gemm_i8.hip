@@ -88,11 +88,12 @@ struct Int8Traits {
       p.bias[2] = bias[col[0]];
       p.bias[3] = bias[col[1]];
     }
-    if (ep.rhs_zero_point && !kSkipRowSums) {
+    // (No array: the kernel forms that side's sums itself and fills them in later.)
+    if (ep.rhs_zero_point && !kSkipRowSums && ep.lhs_sums) {
       p.sums[0] = ep.lhs_sums[row[0]];
       p.sums[1] = ep.lhs_sums[row[1]];
     }
-    if (ep.lhs_zero_point) {
+    if (ep.lhs_zero_point && ep.rhs_sums) {
       p.sums[2] = ep.rhs_sums[col[0]];
       p.sums[3] = ep.rhs_sums[col[1]];
     }
@@ -432,6 +433,23 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   return depth_split::StepCount(steps, parts, parts - 1) >= fused_sums::kMinDepthSteps &&
          tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows && tile == mfma_gemm::Tile::k256x256;
 }
+
+bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus) {
+  if (args.split_k > 1 || !mfma_gemm::LeadColumnSumsApply(args)) return false;
+  const bool flip = args.a_flip != 0 || args.b_flip != 0;
+  if (flip && args.k_bytes % 128 != 0) return false;
+  const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
+  for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k128x128, 128, 128},
+                                    std::tuple{mfma_gemm::Tile::k128x64, 128, 64},
+                                    std::tuple{mfma_gemm::Tile::k64x128, 64, 128}}) {
+    if (tile == mid)
+      return mfma_gemm::LeadColumnSumsMicroseconds(args, num_cus, bm, bn) <
+             mfma_gemm::SumsKernelMicroseconds(double(args.N) * args.k_bytes);
+  }
+  return false;
+}
+
+int GemmI8ColumnSumsOffset(const GemmArgs& args) { return mfma_gemm::ColumnSumsOffset(args); }
 
 int GemmI8RowSumsProducers(const GemmArgs& args, int num_cus) {
   const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);

@@ -316,17 +316,17 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // (workgroups beyond the last tile have a share too): the first
   // args.row_sums_producers workgroups, which the hardware starts first and
   // which all fit the device at once, deal the rows out among themselves.
-  auto add_up_rows_of_share = [&]() {
+  auto add_up_share_of = [&](const void* operand, int ld, int rows, uint32_t flip, long long* words) {
     constexpr int kLanesPerRow = 32;
     constexpr int kRowsPerPass = C::kThreads / kLanesPerRow;
     const int producers = args.row_sums_producers;
     if (int(blockIdx.x) >= producers) return;
-    const int rows_per_group = (args.M + producers - 1) / producers;
+    const int rows_per_group = (rows + producers - 1) / producers;
     const int first = int(blockIdx.x) * rows_per_group;
-    const int end = min(args.M, first + rows_per_group);
+    const int end = min(rows, first + rows_per_group);
     const int lane_in_row = threadIdx.x % kLanesPerRow;
     for (int row = first + int(threadIdx.x) / kLanesPerRow; row < end; row += kRowsPerPass) {
-      const char* from = static_cast<const char*>(args.a) + size_t(row) * size_t(args.lda);
+      const char* from = static_cast<const char*>(operand) + size_t(row) * size_t(ld);
       int sum = 0;
       // (The depth is a whole number of 16-byte granules; bytes past it in the
       // last one are zero.) Eight loads in flight per lane: one after the other
@@ -345,7 +345,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
           const bool inside = k0 + j * kLanesPerRow * kGranule < args.k_bytes;
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            const int bytes = kFlip && inside ? x[j][d] ^ static_cast<int>(args.a_flip) : x[j][d];
+            const int bytes = kFlip && inside ? x[j][d] ^ static_cast<int>(flip) : x[j][d];
             sum = __builtin_amdgcn_sdot4(bytes, 0x01010101, sum, false);
           }
         }
@@ -353,9 +353,13 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
 #pragma unroll
       for (int offset = kLanesPerRow / 2; offset > 0; offset /= 2) sum += __shfl_xor(sum, offset, kLanesPerRow);
       if (lane_in_row == 0)
-        __hip_atomic_fetch_add(args.row_sums + row, fused_sums::Contribution(sum), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(words + row, fused_sums::Contribution(sum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+  };
+  auto add_up_rows_of_share = [&]() {
+    if (args.row_sums_sides & 1) add_up_share_of(args.a, args.lda, args.M, args.a_flip, args.row_sums);
+    if (args.row_sums_sides & 2)
+      add_up_share_of(args.b, args.ldb, args.n_logical, args.b_flip, args.row_sums + args.col_sums_offset);
   };
   if (t >= total) {
     if constexpr (kLeadSums) add_up_rows_of_share();
@@ -663,7 +667,8 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     const int col = (Traits::kSplitB ? n0 / 2 : n0) + wave_n * (C::kLogicalWN * 32) + lane;
     const int row_idx[2] = {min(row, args.M - 1), min(row + 64, args.M - 1)};
     const int col_idx[2] = {min(col, args.n_logical - 1), min(col + 64, args.n_logical - 1)};
-    if constexpr (kRowSums)
+    // (kLeadSums: the sides whose sums come later have no array to load from.)
+    if constexpr (kRowSums && !kLeadSums)
       Traits::template LoadEdgeParams<true>(ep, row_idx, col_idx, edge);  // the sums of the rows come later
     else
       Traits::LoadEdgeParams(ep, row_idx, col_idx, edge);
@@ -1796,38 +1801,54 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   static_assert(kDepthWaves ? 4 * 2 * 128 * BK >= C::kEpilogueBytes + C::kParamBytes : true, "");
   int* const area = reinterpret_cast<int*>(lds + C::kEpilogueBytes) + wave * Traits::kParamInts;
   if constexpr (kLeadSums) {
-    // The sums of the two rows whose parameters this lane stages (rows l and
-    // l + 64 from the wave's first), complete or not.
-    const int first_row = m0 + wave_m * (WM * 32);
-    const int row_of[2] = {min(first_row + lane, args.M - 1), min(first_row + 64 + lane, args.M - 1)};
-    long long word[2] = {0, 0};
-    bool ready = false;
-    for (int looks = 0; !ready && looks < args.row_sums_spin_limit; ++looks) {
-      if (looks) __builtin_amdgcn_s_sleep(8);
+    // The sums of the two rows (columns) whose parameters this lane stages -
+    // l and l + 64 from the wave's first -, complete or not.
+    auto pick_up = [&](const long long* words, const int (&index_of)[2], const void* operand, int ld, uint32_t flip,
+                       int32_t (&sums)[2]) {
+      long long word[2] = {0, 0};
+      bool ready = false;
+      for (int looks = 0; !ready && looks < args.row_sums_spin_limit; ++looks) {
+        if (looks) __builtin_amdgcn_s_sleep(8);
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-        word[h] = __hip_atomic_load(args.row_sums + row_of[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      ready = __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
-                    fused_sums::ContributionsIn(word[1]) == share.expected);
-    }
-    if (ready) {
-      edge.sums[0] = fused_sums::SumIn(word[0]);
-      edge.sums[1] = fused_sums::SumIn(word[1]);
-    } else {
+        for (int h = 0; h < 2; ++h)
+          word[h] = __hip_atomic_load(words + index_of[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ready = __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
+                      fused_sums::ContributionsIn(word[1]) == share.expected);
+      }
+      if (ready) {
+        sums[0] = fused_sums::SumIn(word[0]);
+        sums[1] = fused_sums::SumIn(word[1]);
+        return;
+      }
       // (Workgroups that never got to run, on a device shared with somebody
       // else's work, must not be waited for without end.)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const char* from = static_cast<const char*>(args.a) + size_t(row_of[h]) * size_t(args.lda);
+        const char* from = static_cast<const char*>(operand) + size_t(index_of[h]) * size_t(ld);
         int sum = 0;
         for (int k = 0; k < args.k_bytes; k += kGranule) {
           const v4i x = *reinterpret_cast<const v4i*>(from + k);
 #pragma unroll
           for (int d = 0; d < 4; ++d)
-            sum = __builtin_amdgcn_sdot4(kFlip ? x[d] ^ static_cast<int>(args.a_flip) : x[d], 0x01010101, sum, false);
+            sum = __builtin_amdgcn_sdot4(kFlip ? x[d] ^ static_cast<int>(flip) : x[d], 0x01010101, sum, false);
         }
-        edge.sums[h] = sum;
+        sums[h] = sum;
       }
+    };
+    int32_t picked[2];
+    if (args.row_sums_sides & 1) {
+      const int first_row = m0 + wave_m * (WM * 32);
+      const int row_of[2] = {min(first_row + lane, args.M - 1), min(first_row + 64 + lane, args.M - 1)};
+      pick_up(args.row_sums, row_of, args.a, args.lda, args.a_flip, picked);
+      edge.sums[0] = picked[0];
+      edge.sums[1] = picked[1];
+    }
+    if (args.row_sums_sides & 2) {
+      const int first_col = n0 + wave_n * (C::kLogicalWN * 32);
+      const int col_of[2] = {min(first_col + lane, args.n_logical - 1), min(first_col + 64 + lane, args.n_logical - 1)};
+      pick_up(args.row_sums + args.col_sums_offset, col_of, args.b, args.ldb, args.b_flip, picked);
+      edge.sums[2] = picked[0];
+      edge.sums[3] = picked[1];
     }
   }
   Traits::Stage(ep, edge, area, lane);
@@ -2221,6 +2242,15 @@ inline int LeadSumsProducers(const GemmArgs& args, int num_cus, int bm, int bn) 
 inline double LeadSumsMicroseconds(const GemmArgs& args, int num_cus, int bm, int bn) {
   return 0.5 + double(args.M) * args.k_bytes / LeadSumsProducers(args, num_cus, bm, bn) / 100e3;
 }
+// The same for the rows of `b` (the destination's columns), whose words stand
+// behind those of a's rows.
+inline int ColumnSumsOffset(const GemmArgs& args) { return (args.M + 255) / 256 * 256; }
+inline bool LeadColumnSumsApply(const GemmArgs& args) {
+  return (args.sums_wanted & 2) && (args.sums_wanted & 4) && ColumnSumsOffset(args) + args.N <= fused_sums::kMaxRows;
+}
+inline double LeadColumnSumsMicroseconds(const GemmArgs& args, int num_cus, int bm, int bn) {
+  return 0.5 + double(args.N) * args.k_bytes / LeadSumsProducers(args, num_cus, bm, bn) / 100e3;
+}
 inline bool RowSumming128Applies(const GemmArgs& args, int num_cus) {
   const int tiles = ((args.M + 127) / 128) * ((args.N + 127) / 128);
   return (args.sums_wanted & 3) == 1 && tiles <= num_cus && !LeadSumsApply(args, num_cus, 128, 128) &&
@@ -2240,7 +2270,10 @@ inline double PendingSumsMicroseconds(const GemmArgs& args, int num_cus, const T
   const double a_kernel = SumsKernelMicroseconds(double(args.M) * args.k_bytes);
   const double b_kernel = SumsKernelMicroseconds(double(args.N) * args.k_bytes);
   double extra = b ? b_kernel : 0.0;
-  if (a && model.smallest == Tile::k64x64 && t.tile != Tile::k256x256 && LeadSumsApply(args, num_cus, t.bm, t.bn))
+  const bool lead_sums_tile = model.smallest == Tile::k64x64 && t.tile != Tile::k256x256;
+  if (b && lead_sums_tile && LeadColumnSumsApply(args))
+    extra = std::min(b_kernel, LeadColumnSumsMicroseconds(args, num_cus, t.bm, t.bn));
+  if (a && lead_sums_tile && LeadSumsApply(args, num_cus, t.bm, t.bn))
     return extra + std::min(a_kernel, LeadSumsMicroseconds(args, num_cus, t.bm, t.bn));
   if (a) {
     const bool in_launch = t.tile == Tile::k256x256 && (args.sums_wanted & 4) &&

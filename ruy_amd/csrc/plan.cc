@@ -406,10 +406,17 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   // would meet the sums its last run left behind) and not for a call that
   // shares the GPU's static scratch area with other contexts.
   Operand8& kernel_a = swap ? b : a;
+  Operand8& kernel_b = swap ? a : b;
   bool row_sums_in_launch = false;
   PlanDepthSplit(ctx, GemmKind::kInt8, &args);  // (first: what the sums can do depends on it)
-  if (!args.fuse_sums && kernel_a.sums_pending && ctx->row_sums_in_launch && !ctx->capturing && !ctx->no_alloc &&
-      GemmI8CanFormRowSums(args, ctx->multiprocessor_count)) {
+  // (The tiles of 128 and 64 rows form the sums of either operand that way, the
+  // rows shared out over their workgroups; the largest tile those of `a`.)
+  int sides = 0;
+  if (!args.fuse_sums && ctx->row_sums_in_launch && !ctx->capturing && !ctx->no_alloc) {
+    if (kernel_a.sums_pending && GemmI8CanFormRowSums(args, ctx->multiprocessor_count)) sides |= 1;
+    if (kernel_b.sums_pending && GemmI8CanFormColumnSums(args, ctx->multiprocessor_count)) sides |= 2;
+  }
+  if (sides) {
     const int set = ctx->row_sums_next;
     args.row_sums = ctx->row_sums_sets[set];
     args.row_sums_to_zero = ctx->row_sums_sets[set ^ 1];
@@ -422,7 +429,10 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     if (args.split_k == 1 && fused_sums::FirstContributorIsZero(tiles_m, tiles_n))
       args.row_sums_uniform_run = fused_sums::StepsPerWave(
           (args.k_bytes + 127) / 128, std::min(tiles_n, fused_sums::kMaxContributorTiles));
-    kernel_a.sums_pending = false;
+    args.row_sums_sides = sides;
+    args.col_sums_offset = GemmI8ColumnSumsOffset(args);
+    if (sides & 1) kernel_a.sums_pending = false;
+    if (sides & 2) kernel_b.sums_pending = false;
     row_sums_in_launch = true;
   }
   if (!args.fuse_sums) {
@@ -431,7 +441,8 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   }
   args.ep.lhs_sums = (swap ? b : a).sums;
   args.ep.rhs_sums = (swap ? a : b).sums;
-  if (row_sums_in_launch) args.ep.lhs_sums = nullptr;  // the kernel does not look there
+  if (sides & 1) args.ep.lhs_sums = nullptr;  // the kernel does not look there
+  if (sides & 2) args.ep.rhs_sums = nullptr;
   const bool timed = ctx->TimingBegin();
   const hipError_t launched = LaunchGemmI8(ctx->stream, args, ctx->multiprocessor_count);
   if (timed) ctx->TimingEnd();
@@ -443,7 +454,8 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
     // The launch is on the stream: it leaves its own set dirty and the other one clean.
     const int set = ctx->row_sums_next;
     ctx->row_sums_dirty_rows[set ^ 1] = 0;
-    ctx->row_sums_dirty_rows[set] = RoundUp(args.M, fused_sums::kTileRows);
+    ctx->row_sums_dirty_rows[set] =
+        (sides & 2) ? args.col_sums_offset + args.N : RoundUp(args.M, fused_sums::kTileRows);
     ctx->row_sums_next = set ^ 1;
     ++ctx->row_sums_calls;
   }

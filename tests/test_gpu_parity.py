@@ -946,7 +946,8 @@ def test_random_deep_and_weight_streaming_products_every_element(device_ctx):
 @pytest.mark.parametrize("mode", ["in launch", "own", "separate"])
 def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
     """Grids of 128x128, 128x64 or 64x128 tiles: the rows of the `a` operand
-    are dealt out over the workgroups of the grid's first round, which add them
+    (and those of `b`, where the other zero point is set: the cases below have
+    either and both) are dealt out over the workgroups of the grid's first round, which add them
     up from global memory while their first loads are on their way; every wave
     picks up the sums of its rows in front of its write-back. Modes: that; the
     sums never looked for, so that every wave forms those of its rows itself
