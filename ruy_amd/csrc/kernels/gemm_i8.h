@@ -155,11 +155,13 @@ bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus);
 // the depth sums of a's rows (GemmArgs::row_sums).
 bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus);
 // For GemmArgs::row_sums_producers: how many workgroups of the launch share the
-// rows out among themselves (0: the largest tile, which has its own scheme).
+// rows out among themselves (the largest tile: those of b only; a's have
+// their own scheme).
 int GemmI8RowSumsProducers(const GemmArgs& args, int num_cus);
-// Whether the launch should also form the depth sums of b's rows (the tiles of
-// 128 and 64 rows only), and where their words then stand in row_sums.
-bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus);
+// Whether the launch should also form the depth sums of b's rows (the largest
+// tile: only together with those of a's rows), and where their words then
+// stand in row_sums.
+bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus, bool rows_in_launch);
 int GemmI8ColumnSumsOffset(const GemmArgs& args);
 hipError_t LaunchGemmI8(hipStream_t stream, const GemmArgs& args, int num_cus);
 // `count` <= kGemmBatchMax products of the shape and parameters of `args`, each

@@ -434,12 +434,15 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
          tiles_m * fused_sums::kTileRows <= fused_sums::kMaxRows && tile == mfma_gemm::Tile::k256x256;
 }
 
-bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus) {
+bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus, bool rows_in_launch) {
   if (args.split_k > 1 || !mfma_gemm::LeadColumnSumsApply(args)) return false;
   const bool flip = args.a_flip != 0 || args.b_flip != 0;
   if (flip && args.k_bytes % 128 != 0) return false;
   const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
-  for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k128x128, 128, 128},
+  // (The largest tile's kernel with sums in its launch always forms those of a's rows.)
+  if (tile == mfma_gemm::Tile::k256x256 && !rows_in_launch) return false;
+  for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k256x256, 256, 256},
+                                    std::tuple{mfma_gemm::Tile::k128x128, 128, 128},
                                     std::tuple{mfma_gemm::Tile::k128x64, 128, 64},
                                     std::tuple{mfma_gemm::Tile::k64x128, 64, 128}}) {
     if (tile == mid)
@@ -456,6 +459,7 @@ int GemmI8RowSumsProducers(const GemmArgs& args, int num_cus) {
   if (tile == mfma_gemm::Tile::k128x128) return mfma_gemm::LeadSumsProducers(args, num_cus, 128, 128);
   if (tile == mfma_gemm::Tile::k128x64) return mfma_gemm::LeadSumsProducers(args, num_cus, 128, 64);
   if (tile == mfma_gemm::Tile::k64x128) return mfma_gemm::LeadSumsProducers(args, num_cus, 64, 128);
+  if (tile == mfma_gemm::Tile::k256x256) return mfma_gemm::LeadSumsProducers(args, num_cus, 256, 256);
   return 0;
 }
 

@@ -970,6 +970,12 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       for (int l = 0; l < C::kALoads; ++l) issue_one(st, l);
     }
     load_edge_params();
+    // (The rows of `b`, where their sums are wanted too: shared out over the
+    // first round's workgroups like on the smaller tiles.)
+    if constexpr (kRowSums && !kSplitLarge) {
+      if (args.row_sums_sides & 2)
+        add_up_share_of(args.b, args.ldb, args.n_logical, args.b_flip, args.row_sums + args.col_sums_offset);
+    }
     WaitVmcnt<paired_schedule::kLoadsLeftBeforeFirstStep>();
     __syncthreads();
 #pragma unroll
@@ -1467,6 +1473,41 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     }
   }
 
+  // kRowSums: the sums of two rows (columns) that workgroups of this launch
+  // have added up from global memory - those whose parameters a lane stages:
+  // l and l + 64 from the wave's first -, complete or not.
+  auto pick_up = [&](const long long* words, const int (&index_of)[2], const void* operand, int ld, uint32_t flip,
+                     int expected, int32_t (&sums)[2]) {
+    long long word[2] = {0, 0};
+    bool ready = false;
+    for (int looks = 0; !ready && looks < args.row_sums_spin_limit; ++looks) {
+      if (looks) __builtin_amdgcn_s_sleep(8);
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        word[h] = __hip_atomic_load(words + index_of[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      ready = __all(fused_sums::ContributionsIn(word[0]) == expected &&
+                    fused_sums::ContributionsIn(word[1]) == expected);
+    }
+    if (ready) {
+      sums[0] = fused_sums::SumIn(word[0]);
+      sums[1] = fused_sums::SumIn(word[1]);
+      return;
+    }
+    // (Workgroups that never got to run, on a device shared with somebody
+    // else's work, must not be waited for without end.)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const char* from = static_cast<const char*>(operand) + size_t(index_of[h]) * size_t(ld);
+      int sum = 0;
+      for (int k = 0; k < args.k_bytes; k += kGranule) {
+        const v4i x = *reinterpret_cast<const v4i*>(from + k);
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          sum = __builtin_amdgcn_sdot4(kFlip ? x[d] ^ static_cast<int>(flip) : x[d], 0x01010101, sum, false);
+      }
+      sums[h] = sum;
+    }
+  };
   // ---- fused write-back, 16x16 blocks ----
   // The destination is column-major here (rows contiguous; the host swaps the
   // operands for a row-major destination). Lane l holds, of every block,
@@ -1525,6 +1566,17 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
               sum = __builtin_amdgcn_sdot4(kFlip ? x[d] ^ static_cast<int>(args.a_flip) : x[d], 0x01010101, sum, false);
           }
           edge.sums[h] = sum;
+        }
+      }
+      if constexpr (!kSplitLarge) {
+        if (args.row_sums_sides & 2) {
+          const int first_col = n0 + wave_n * (WN * 32);
+          const int col_of[2] = {min(first_col + lane, args.n_logical - 1),
+                                 min(first_col + 64 + lane, args.n_logical - 1)};
+          int32_t picked[2];
+          pick_up(args.row_sums + args.col_sums_offset, col_of, args.b, args.ldb, args.b_flip, 1, picked);
+          edge.sums[2] = picked[0];
+          edge.sums[3] = picked[1];
         }
       }
     }
@@ -1803,50 +1855,18 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   if constexpr (kLeadSums) {
     // The sums of the two rows (columns) whose parameters this lane stages -
     // l and l + 64 from the wave's first -, complete or not.
-    auto pick_up = [&](const long long* words, const int (&index_of)[2], const void* operand, int ld, uint32_t flip,
-                       int32_t (&sums)[2]) {
-      long long word[2] = {0, 0};
-      bool ready = false;
-      for (int looks = 0; !ready && looks < args.row_sums_spin_limit; ++looks) {
-        if (looks) __builtin_amdgcn_s_sleep(8);
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-          word[h] = __hip_atomic_load(words + index_of[h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ready = __all(fused_sums::ContributionsIn(word[0]) == share.expected &&
-                      fused_sums::ContributionsIn(word[1]) == share.expected);
-      }
-      if (ready) {
-        sums[0] = fused_sums::SumIn(word[0]);
-        sums[1] = fused_sums::SumIn(word[1]);
-        return;
-      }
-      // (Workgroups that never got to run, on a device shared with somebody
-      // else's work, must not be waited for without end.)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const char* from = static_cast<const char*>(operand) + size_t(index_of[h]) * size_t(ld);
-        int sum = 0;
-        for (int k = 0; k < args.k_bytes; k += kGranule) {
-          const v4i x = *reinterpret_cast<const v4i*>(from + k);
-#pragma unroll
-          for (int d = 0; d < 4; ++d)
-            sum = __builtin_amdgcn_sdot4(kFlip ? x[d] ^ static_cast<int>(flip) : x[d], 0x01010101, sum, false);
-        }
-        sums[h] = sum;
-      }
-    };
     int32_t picked[2];
     if (args.row_sums_sides & 1) {
       const int first_row = m0 + wave_m * (WM * 32);
       const int row_of[2] = {min(first_row + lane, args.M - 1), min(first_row + 64 + lane, args.M - 1)};
-      pick_up(args.row_sums, row_of, args.a, args.lda, args.a_flip, picked);
+      pick_up(args.row_sums, row_of, args.a, args.lda, args.a_flip, 1, picked);
       edge.sums[0] = picked[0];
       edge.sums[1] = picked[1];
     }
     if (args.row_sums_sides & 2) {
       const int first_col = n0 + wave_n * (C::kLogicalWN * 32);
       const int col_of[2] = {min(first_col + lane, args.n_logical - 1), min(first_col + 64 + lane, args.n_logical - 1)};
-      pick_up(args.row_sums + args.col_sums_offset, col_of, args.b, args.ldb, args.b_flip, picked);
+      pick_up(args.row_sums + args.col_sums_offset, col_of, args.b, args.ldb, args.b_flip, 1, picked);
       edge.sums[2] = picked[0];
       edge.sums[3] = picked[1];
     }
@@ -2226,7 +2246,6 @@ inline double RowSumming128Microseconds(int k_steps) { return 0.6 + 0.103 * k_st
 // `a` added up by the workgroups of their own grid, each taking a share of
 // the rows while its first loads are on their way (kLeadSums in the kernel),
 // where the caller allows sums formed inside a launch (bit 4 of sums_wanted).
-// A workgroup reads its share at some 100 GB/s.
 inline bool LeadSumsApply(const GemmArgs& args, int, int, int) {
   return (args.sums_wanted & 1) && (args.sums_wanted & 4) && args.M <= fused_sums::kMaxRows;
 }
@@ -2236,11 +2255,20 @@ inline bool LeadSumsApply(const GemmArgs& args, int, int, int) {
 inline int LeadSumsProducers(const GemmArgs& args, int num_cus, int bm, int bn) {
   const int tiles = ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
   const int grid = (tiles + 7) / 8 * 8;
-  const int per_cu = tiles <= num_cus ? 1 : (bm == 128 && bn == 128 ? 2 : 3);
+  const int per_cu = tiles <= num_cus || bm == 256 ? 1 : (bm == 128 && bn == 128 ? 2 : 3);
   return std::min(grid, num_cus * per_cu);
 }
+// What a workgroup's share costs it: it adds up eight rows at a time, 4 KiB of
+// each per batch of loads, and a batch takes a round trip to memory - 0.6 us
+// when a workgroup has one or two of them, 1.3 us each when all of them have
+// many in flight (measured: 2048^3 0.9 us, 2048 x 8192 x 2048 1.4 us, the
+// 8192 x 8192 right-hand operand of 8192^3 in 32 rows a workgroup 11 us).
+inline double LeadShareMicroseconds(int rows, int k_bytes, int producers) {
+  const int batches = ((rows + producers - 1) / producers + 7) / 8 * ((k_bytes + 4095) / 4096);
+  return 0.3 + (batches <= 2 ? 0.6 : 1.3) * batches;
+}
 inline double LeadSumsMicroseconds(const GemmArgs& args, int num_cus, int bm, int bn) {
-  return 0.5 + double(args.M) * args.k_bytes / LeadSumsProducers(args, num_cus, bm, bn) / 100e3;
+  return LeadShareMicroseconds(args.M, args.k_bytes, LeadSumsProducers(args, num_cus, bm, bn));
 }
 // The same for the rows of `b` (the destination's columns), whose words stand
 // behind those of a's rows.
@@ -2249,7 +2277,7 @@ inline bool LeadColumnSumsApply(const GemmArgs& args) {
   return (args.sums_wanted & 2) && (args.sums_wanted & 4) && ColumnSumsOffset(args) + args.N <= fused_sums::kMaxRows;
 }
 inline double LeadColumnSumsMicroseconds(const GemmArgs& args, int num_cus, int bm, int bn) {
-  return 0.5 + double(args.N) * args.k_bytes / LeadSumsProducers(args, num_cus, bm, bn) / 100e3;
+  return LeadShareMicroseconds(args.N, args.k_bytes, LeadSumsProducers(args, num_cus, bm, bn));
 }
 inline bool RowSumming128Applies(const GemmArgs& args, int num_cus) {
   const int tiles = ((args.M + 127) / 128) * ((args.N + 127) / 128);
@@ -2271,7 +2299,7 @@ inline double PendingSumsMicroseconds(const GemmArgs& args, int num_cus, const T
   const double b_kernel = SumsKernelMicroseconds(double(args.N) * args.k_bytes);
   double extra = b ? b_kernel : 0.0;
   const bool lead_sums_tile = model.smallest == Tile::k64x64 && t.tile != Tile::k256x256;
-  if (b && lead_sums_tile && LeadColumnSumsApply(args))
+  if (b && model.smallest == Tile::k64x64 && LeadColumnSumsApply(args))
     extra = std::min(b_kernel, LeadColumnSumsMicroseconds(args, num_cus, t.bm, t.bn));
   if (a && lead_sums_tile && LeadSumsApply(args, num_cus, t.bm, t.bn))
     return extra + std::min(a_kernel, LeadSumsMicroseconds(args, num_cus, t.bm, t.bn));

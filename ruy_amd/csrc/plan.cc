@@ -414,7 +414,7 @@ int RunInt8(ruyamd_ctx* ctx, MulCall* call, std::string* err) {
   int sides = 0;
   if (!args.fuse_sums && ctx->row_sums_in_launch && !ctx->capturing && !ctx->no_alloc) {
     if (kernel_a.sums_pending && GemmI8CanFormRowSums(args, ctx->multiprocessor_count)) sides |= 1;
-    if (kernel_b.sums_pending && GemmI8CanFormColumnSums(args, ctx->multiprocessor_count)) sides |= 2;
+    if (kernel_b.sums_pending && GemmI8CanFormColumnSums(args, ctx->multiprocessor_count, (sides & 1) != 0)) sides |= 2;
   }
   if (sides) {
     const int set = ctx->row_sums_next;
