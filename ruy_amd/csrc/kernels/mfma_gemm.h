@@ -362,7 +362,12 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       add_up_share_of(args.b, args.ldb, args.n_logical, args.b_flip, args.row_sums + args.col_sums_offset);
   };
   if (t >= total) {
+    // (A workgroup beyond the last tile still has its share of the rows to add up.)
     if constexpr (kLeadSums) add_up_rows_of_share();
+    if constexpr (kRowSums && !kLeadSums && !kSplitLarge) {
+      if (args.row_sums_sides & 2)
+        add_up_share_of(args.b, args.ldb, args.n_logical, args.b_flip, args.row_sums + args.col_sums_offset);
+    }
     return;
   }
   constexpr int kGroupM = 4;

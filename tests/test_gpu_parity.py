@@ -996,6 +996,45 @@ def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
         ctx.close()
 
 
+def test_sums_shared_out_do_not_wait_for_workgroups_beyond_the_last_tile():
+    """Grids whose number of tiles is not a multiple of eight are launched with
+    a few workgroups beyond the last tile. Where the rows of an operand are
+    shared out over the workgroups of the grid, those have a share too: without
+    it the waves that need the sums look for them until their bound runs out and
+    then form them themselves - right results, milliseconds late. 186 tiles of
+    256x256 (the right-hand operand's sums) and 225 tiles of 128x128 (both),
+    timed by the library's own events."""
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    ctx = api.Context()
+    try:
+        ctx.set_kernel_timing(True)
+        rng = np.random.default_rng(99)
+        for (M, K, N) in [(7936, 2048, 1536), (1900, 2048, 1900)]:
+            p = W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, M, K, N, *cases.RCC, strided=False,
+                                 name="padding workgroups %s" % ((M, K, N),))
+            p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+            p.lhs.zero_point, p.rhs.zero_point = 7, -3
+            announce(p.name)
+            want = O.full_size_expected(p)
+            dp = D.DeviceProblem(p, dst_fill=0)
+            for _ in range(3):
+                dp.run(ctx)
+            ctx.synchronize()
+            ctx.kernel_timing()
+            before = ctx.sums_in_launch_calls()
+            for _ in range(5):
+                dp.run(ctx)
+            ctx.synchronize()
+            ms, launches = ctx.kernel_timing()
+            assert ctx.sums_in_launch_calls() == before + 5
+            assert launches == 5 and ms / launches < 0.5, (ms, launches)
+            if want is not None:
+                assert (dp.dst_t.cpu().numpy() == want).all()
+    finally:
+        ctx.close()
+
+
 def test_row_sums_formed_by_the_128_tile_every_element(device_ctx):
     """A grid of at most one 128x128 tile per CU with a short depth, one
     operand's zero point set and that operand's partner used in place: the
