@@ -1485,7 +1485,11 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
                      int expected, int32_t (&sums)[2]) {
     long long word[2] = {0, 0};
     bool ready = false;
-    for (int looks = 0; !ready && looks < args.row_sums_spin_limit; ++looks) {
+    // (Shares are added up within microseconds of the launch's start, long
+    // before anybody looks here: a few hundred looks, a fraction of a
+    // millisecond, are plenty before giving up on workgroups that do not run.)
+    const int looks_allowed = min(args.row_sums_spin_limit, 512);
+    for (int looks = 0; !ready && looks < looks_allowed; ++looks) {
       if (looks) __builtin_amdgcn_s_sleep(8);
 #pragma unroll
       for (int h = 0; h < 2; ++h)
@@ -2254,13 +2258,13 @@ inline double RowSumming128Microseconds(int k_steps) { return 0.6 + 0.103 * k_st
 inline bool LeadSumsApply(const GemmArgs& args, int, int, int) {
   return (args.sums_wanted & 1) && (args.sums_wanted & 4) && args.M <= fused_sums::kMaxRows;
 }
-// The workgroups that share the rows out: those of the grid's first round (a
-// grid of more tiles than CUs runs on the rings of two stages, two workgroups
-// of the 128x128 tile or three of the 128x64 and 64x128 tiles to a CU).
+// The workgroups that share the rows out: workgroups of the grid's first round,
+// which all run at once (a grid of more tiles than CUs runs on the rings of two
+// stages, of which a CU holds two workgroups at least).
 inline int LeadSumsProducers(const GemmArgs& args, int num_cus, int bm, int bn) {
   const int tiles = ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
   const int grid = (tiles + 7) / 8 * 8;
-  const int per_cu = tiles <= num_cus || bm == 256 ? 1 : (bm == 128 && bn == 128 ? 2 : 3);
+  const int per_cu = tiles <= num_cus || bm == 256 ? 1 : 2;
   return std::min(grid, num_cus * per_cu);
 }
 // What a workgroup's share costs it: it adds up eight rows at a time, 4 KiB of
