@@ -1010,9 +1010,11 @@ def test_sums_shared_out_do_not_wait_for_workgroups_beyond_the_last_tile():
     try:
         ctx.set_kernel_timing(True)
         rng = np.random.default_rng(99)
-        for (M, K, N) in [(7936, 2048, 1536), (1900, 2048, 1900)]:
+        # (the last four: grids of more than one round, whose first round's workgroups must all run at once)
+        for (M, K, N) in [(7936, 2048, 1536), (1900, 2048, 1900), (2560, 2560, 2560), (3000, 1024, 3072),
+                          (4096, 1024, 1000), (8000, 768, 1100)]:
             p = W.random_problem(rng, S.I8, S.I8, S.I32, S.I8, M, K, N, *cases.RCC, strided=False,
-                                 name="padding workgroups %s" % ((M, K, N),))
+                                 name="sums inside the launch, timed %s" % ((M, K, N),))
             p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
             p.lhs.zero_point, p.rhs.zero_point = 7, -3
             announce(p.name)
