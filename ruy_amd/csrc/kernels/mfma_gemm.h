@@ -209,7 +209,8 @@ struct Cfg {
                                                       : kEpilogueBytes + kParamBytes);
 };
 
-// kFusedSums (64x64 tile of the int8 kernel only): the kernel also forms the
+// kFusedSums (64x64 tile of the int8 kernel; the 128x128 tile for the rows of
+// `a` only): the kernel also forms the
 // depth sums of its rows of `a` and columns of `b` - one more matrix
 // instruction each per depth sub-step, against a fragment of ones - and
 // subtracts args.fused_a_factor * rowsum + args.fused_b_factor * colsum from
@@ -222,22 +223,27 @@ struct Cfg {
 // fragment before use, which turns uint8 data used in place into the int8
 // values the arithmetic is defined on.
 //
-// kRowSums (largest int8 tile only): the launch also forms the depth sums of
-// the rows of `a`, dealt out over the first workgroups of every tile row, and
-// every workgroup fetches them shortly before its write-back (fused_sums.h).
+// kRowSums (int8 kernel): the launch also forms depth sums that the write-back
+// needs, in 64-bit words of global memory that carry a sum and the number of
+// contributions to it (fused_sums.h), and every wave picks up those of its
+// rows in front of its write-back. The largest tile forms the sums of the rows
+// of `a` in passing, dealt out over the first workgroups of every tile row,
+// and can have those of the rows of `b` added up from global memory by the
+// workgroups of its first round, a share each; the 128x128, 128x64 and 64x128
+// tiles have either operand's done that second way (args.row_sums_sides).
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false, bool kRowSums = false, bool kSplitLarge = false>
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   static_assert(!kRowSums || !kFusedSums, "one way of forming the sums at a time");
-  // kRowSums on the tiles of 32x32 blocks whose waves share every step (grids
-  // of at most one workgroup per CU): the rows of `a` are dealt out over the
-  // workgroups of the grid, each of which adds up its few rows from global
-  // memory while its first ring stages are on their way (a 1/256 share of the
-  // operand: some tens of bytes a thread) and puts the sums into the rows'
-  // words (fused_sums.h: one contribution completes a word). Every wave looks
-  // at the words of its rows in front of its write-back, microseconds later;
-  // words that are not complete are read again a bounded number of times,
-  // after which the wave forms the sums of its rows itself.
+  // kRowSums on the tiles of 32x32 blocks whose waves share every step: the
+  // rows of an operand are dealt out over the workgroups of the grid's first
+  // round, each of which adds up its few rows from global memory while its
+  // first ring stages are on their way (a 1/256 share of the operand: some
+  // tens of bytes a thread) and puts the sums into the rows' words
+  // (fused_sums.h: one contribution completes a word). Every wave looks at the
+  // words of its rows in front of its write-back, microseconds later; words
+  // that are not complete are read again a bounded number of times, after
+  // which the wave forms the sums of its rows itself.
   constexpr bool kLeadSums = kRowSums && !Traits::kPaired;
   static_assert(!kLeadSums || (Traits::kBlock == 32 && !kDepthWaves && !Traits::kSplitB && !kSplitLarge), "");
   static_assert(!kSplitLarge || Traits::kPaired, "kSplitLarge is the depth split of the paired schedule's tile");
