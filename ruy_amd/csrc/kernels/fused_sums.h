@@ -52,6 +52,12 @@
 // alternates them and tells the kernel how many rows the launch before last
 // left dirty). A launch that is recorded into a graph and replayed would meet
 // its own leftovers, so recorded calls keep the separate kernel.
+//
+// The same words serve the other way of forming sums inside a launch: the
+// rows of an operand shared out over the workgroups of the grid's first round,
+// each of which adds up its share from global memory in its prologue and
+// contributes once per row (the tiles of 128 and 64 rows, either operand; the
+// largest tile, the rows of `b`, whose words stand behind those of a's rows).
 #ifndef RUY_AMD_CSRC_KERNELS_FUSED_SUMS_H_
 #define RUY_AMD_CSRC_KERNELS_FUSED_SUMS_H_
 
