@@ -401,7 +401,8 @@ void GemmTileFor(const GemmArgs& args, int num_cus, GemmKind kind, int* tile_row
 bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
   const mfma_gemm::TileChoice choice = mfma_gemm::ChooseTile(args, num_cus, mfma_gemm::Model::kInt8);
   if (choice.large_parts != 1) return false;
-  if (choice.tile == mfma_gemm::Tile::k64x64) return true;
+  // (The smallest tile: unless sharing the rows out over its workgroups is cheaper.)
+  if (choice.tile == mfma_gemm::Tile::k64x64) return !mfma_gemm::SmallestTileSharesSumsOut(args, num_cus);
   // The 128x128 tile forms the row sums of `a`, and only those, in grids of
   // at most one workgroup per CU.
   return choice.tile == mfma_gemm::Tile::k128x128 && mfma_gemm::RowSumming128Applies(args, num_cus);
@@ -421,6 +422,8 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   // (uint8 data in place needs whole depth steps, which LaunchGemmI8 insists on.)
   if (flip && args.k_bytes % 128 != 0) return false;
   const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
+  if (tile == mfma_gemm::Tile::k64x64)
+    return (args.sums_wanted & 1) && !args.split_large && mfma_gemm::SmallestTileSharesSumsOut(args, num_cus);
   // The tiles in between: by the workgroups of the grid, each for a share of the rows.
   for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k128x128, 128, 128},
                                     std::tuple{mfma_gemm::Tile::k128x64, 128, 64},
@@ -439,6 +442,7 @@ bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus, bool rows_in_lau
   const bool flip = args.a_flip != 0 || args.b_flip != 0;
   if (flip && args.k_bytes % 128 != 0) return false;
   const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
+  if (tile == mfma_gemm::Tile::k64x64) return mfma_gemm::SmallestTileSharesSumsOut(args, num_cus);
   // (The largest tile's kernel with sums in its launch always forms those of a's rows.)
   if (tile == mfma_gemm::Tile::k256x256 && !rows_in_launch) return false;
   for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k256x256, 256, 256},
@@ -460,6 +464,7 @@ int GemmI8RowSumsProducers(const GemmArgs& args, int num_cus) {
   if (tile == mfma_gemm::Tile::k128x64) return mfma_gemm::LeadSumsProducers(args, num_cus, 128, 64);
   if (tile == mfma_gemm::Tile::k64x128) return mfma_gemm::LeadSumsProducers(args, num_cus, 64, 128);
   if (tile == mfma_gemm::Tile::k256x256) return mfma_gemm::LeadSumsProducers(args, num_cus, 256, 256);
+  if (tile == mfma_gemm::Tile::k64x64) return mfma_gemm::LeadSumsProducers(args, num_cus, 64, 64);
   return 0;
 }
 

@@ -245,7 +245,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // that are not complete are read again a bounded number of times, after
   // which the wave forms the sums of its rows itself.
   constexpr bool kLeadSums = kRowSums && !Traits::kPaired;
-  static_assert(!kLeadSums || (Traits::kBlock == 32 && !kDepthWaves && !Traits::kSplitB && !kSplitLarge), "");
+  static_assert(!kLeadSums || (Traits::kBlock == 32 && !Traits::kSplitB && !kSplitLarge), "");
   static_assert(!kSplitLarge || Traits::kPaired, "kSplitLarge is the depth split of the paired schedule's tile");
   // kFusedSums on the 128x128 tile (two by two blocks per wave, waves sharing
   // every step): the row sums of `a` only, one more matrix instruction per
@@ -326,7 +326,8 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     constexpr int kLanesPerRow = 32;
     constexpr int kRowsPerPass = C::kThreads / kLanesPerRow;
     const int producers = args.row_sums_producers;
-    if (int(blockIdx.x) >= producers) return;
+    // (With the depth of the smallest tile split, grid row 0 holds the producers.)
+    if (int(blockIdx.x) >= producers || blockIdx.y != 0) return;
     const int rows_per_group = (rows + producers - 1) / producers;
     const int first = int(blockIdx.x) * rows_per_group;
     const int end = min(rows, first + rows_per_group);
@@ -848,6 +849,7 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
     if (my_steps > 0) issue_step(depth_way, 0);
     if (my_steps > 1) issue_step(depth_way + kDepthWays, 1);
     load_edge_params();
+    if constexpr (kLeadSums) add_up_rows_of_share();
     Frags4 fr[2];
     auto walk_slot = [&](int slot) {
       read4(slot, 0, fr[0]);
@@ -2270,7 +2272,7 @@ inline bool LeadSumsApply(const GemmArgs& args, int, int, int) {
 inline int LeadSumsProducers(const GemmArgs& args, int num_cus, int bm, int bn) {
   const int tiles = ((args.M + bm - 1) / bm) * ((args.N + bn - 1) / bn);
   const int grid = (tiles + 7) / 8 * 8;
-  const int per_cu = tiles <= num_cus || bm == 256 ? 1 : 2;
+  const int per_cu = tiles <= num_cus || bm == 256 || (bm == 64 && bn == 64) ? 1 : 2;
   return std::min(grid, num_cus * per_cu);
 }
 // What a workgroup's share costs it: it adds up eight rows at a time, 4 KiB of
@@ -2278,12 +2280,49 @@ inline int LeadSumsProducers(const GemmArgs& args, int num_cus, int bm, int bn) 
 // when a workgroup has one or two of them, 1.3 us each when all of them have
 // many in flight (measured: 2048^3 0.9 us, 2048 x 8192 x 2048 1.4 us, the
 // 8192 x 8192 right-hand operand of 8192^3 in 32 rows a workgroup 11 us).
+inline int LeadShareBatches(int rows, int k_bytes, int producers) {
+  return ((rows + producers - 1) / producers + 7) / 8 * ((k_bytes + 4095) / 4096);
+}
 inline double LeadShareMicroseconds(int rows, int k_bytes, int producers) {
-  const int batches = ((rows + producers - 1) / producers + 7) / 8 * ((k_bytes + 4095) / 4096);
+  const int batches = LeadShareBatches(rows, k_bytes, producers);
   return 0.3 + (batches <= 2 ? 0.6 : 1.3) * batches;
 }
 inline double LeadSumsMicroseconds(const GemmArgs& args, int num_cus, int bm, int bn) {
   return LeadShareMicroseconds(args.M, args.k_bytes, LeadSumsProducers(args, num_cus, bm, bn));
+}
+// The smallest int8 tile, which otherwise forms both operands' sums with two
+// more matrix instructions per four (measured on 256 tiles: + 1.1 us at a
+// depth of 8 steps, + 1.5 us at 32, + 3.2 us at 64, + 7.0 us at 128 - 15 to
+// 27 % of the launch): shared out where that is cheaper and the depth leaves
+// every wave a step (the depth-per-wave schedule). Measured on 256 tiles with
+// the rows of `a` shared out, against the matrix instructions: 7.8 us for 8.5
+// at 16 steps, 10.4 for 11.3 at 32, 16.5 for 18.3 at 64 - and 42.7 for 32.4
+// at 128 steps, where a workgroup's share takes four batches of loads: two
+// batches a side at most.
+inline int SmallestTileParts(const GemmArgs& args, int num_cus) {
+  const int tiles = ((args.M + 63) / 64) * ((args.N + 63) / 64);
+  return DepthSplitParts(tiles, std::max(1, (args.k_bytes + 127) / 128), num_cus, 16);
+}
+inline double SmallestTileSharedSumsMicroseconds(const GemmArgs& args, int num_cus) {
+  const int tiles = ((args.M + 63) / 64) * ((args.N + 63) / 64);
+  const int producers = std::min((tiles + 7) / 8 * 8, num_cus);
+  double cost = 0;
+  if (args.sums_wanted & 1) cost += LeadShareMicroseconds(args.M, args.k_bytes, producers);
+  if (args.sums_wanted & 2) cost += LeadShareMicroseconds(args.N, args.k_bytes, producers);
+  return cost;
+}
+inline bool SmallestTileSharesSumsOut(const GemmArgs& args, int num_cus) {
+  if (!(args.sums_wanted & 4) || !(args.sums_wanted & 3)) return false;
+  const int rows_of_words = ((args.sums_wanted & 2) ? (args.M + 255) / 256 * 256 + args.N : args.M);
+  if (rows_of_words > fused_sums::kMaxRows) return false;
+  const int k_steps = std::max(1, (args.k_bytes + 127) / 128);
+  const int steps_per_part = depth_split::StepsPerPart(k_steps, SmallestTileParts(args, num_cus));
+  if (steps_per_part < 4) return false;
+  const int tiles = ((args.M + 63) / 64) * ((args.N + 63) / 64);
+  const int producers = std::min((tiles + 7) / 8 * 8, num_cus);
+  if ((args.sums_wanted & 1) && LeadShareBatches(args.M, args.k_bytes, producers) > 2) return false;
+  if ((args.sums_wanted & 2) && LeadShareBatches(args.N, args.k_bytes, producers) > 2) return false;
+  return SmallestTileSharedSumsMicroseconds(args, num_cus) < 0.6 + 0.05 * steps_per_part;
 }
 // The same for the rows of `b` (the destination's columns), whose words stand
 // behind those of a's rows.
@@ -2305,6 +2344,8 @@ inline double PendingSumsMicroseconds(const GemmArgs& args, int num_cus, const T
   const bool a = (args.sums_wanted & 1) != 0, b = (args.sums_wanted & 2) != 0;
   if (!a && !b) return 0.0;
   if (t.tile == model.smallest) {
+    if (model.smallest == Tile::k64x64 && SmallestTileSharesSumsOut(args, num_cus))
+      return SmallestTileSharedSumsMicroseconds(args, num_cus);
     *factor = 1.15;
     return 0.0;
   }
@@ -2511,6 +2552,13 @@ hipError_t LaunchSmallestTile(hipStream_t stream, const GemmArgs& args) {
   constexpr int kDepthWays = 4 / kWN;
   const int k_tiles = (args.k_bytes + 127) / 128;
   const int parts = args.split_k > 1 ? args.split_k : 1;
+  if constexpr (Traits::kModel == Model::kInt8 && !kFusedSums) {
+    // (Sums shared out over the grid's workgroups: the depth-per-wave schedule only.)
+    if (args.row_sums) {
+      if ((k_tiles + parts - 1) / parts < kDepthWays) return hipErrorInvalidValue;
+      return Launch<Traits, 1, kWN, 128, 4, false, kFlip, true, true>(stream, args);
+    }
+  }
   if ((k_tiles + parts - 1) / parts < kDepthWays)
     return Launch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, false>(stream, args);
   return Launch<Traits, 1, kWN, 128, 4, kFusedSums, kFlip, true>(stream, args);

@@ -996,6 +996,52 @@ def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
         ctx.close()
 
 
+@pytest.mark.parametrize("mode", ["in launch", "own"])
+def test_row_sums_shared_out_over_a_grid_of_the_smallest_tile(mode):
+    """Grids of 64x64 tiles whose depth leaves every wave a few steps: the rows
+    of the operands are dealt out over the workgroups of the grid (of its first
+    row, where the depth is split over several) instead of being summed by
+    extra matrix instructions. Either and both operands' sums, uint8 data,
+    ragged edges, operands swapped, a split depth; with the sums picked up,
+    and never looked for (every wave forms its own): every element against the
+    stock library. Shapes beyond what is shared out (a deep share, a depth of
+    few steps) keep the matrix instructions and must come out the same."""
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    ctx = api.Context()
+    try:
+        ctx.set_sums_in_launch(1, 0 if mode == "own" else -1)
+        rng = np.random.default_rng(99)
+        calls = 0
+        for tup, (M, K, N), orders, lzp, rzp in [
+                ((S.I8, S.I8, S.I32, S.I8), (1024, 4096, 1024), cases.RCC, 0, -3),
+                ((S.I8, S.I8, S.I32, S.I8), (1024, 4096, 1024), cases.RCC, 5, 0),
+                ((S.U8, S.U8, S.I32, S.U8), (1000, 8192, 900), cases.RCC, 131, 120),
+                ((S.I8, S.U8, S.I32, S.I16), (768, 4096, 768), (1, 0, 1), 3, 128 + 4),
+                ((S.I8, S.I8, S.I32, S.I32), (512, 4096, 512), cases.RCC, 2, -3),       # the depth in two parts
+                ((S.U8, S.I8, S.I32, S.I8), (300, 6144, 1500), cases.RCC, 128, 9),
+                ((S.I8, S.I8, S.I32, S.I8), (1024, 1024, 1024), cases.RCC, 0, -3),
+                ((S.I8, S.I8, S.I32, S.I8), (640, 2048, 900), (1, 0, 1), 7, -3),
+                ((S.I8, S.I8, S.I32, S.I8), (1024, 16384, 1024), cases.RCC, 0, -3),     # too deep a share
+                ((S.I8, S.I8, S.I32, S.I8), (192, 8192, 192), cases.RCC, 1, 1)]:
+            p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
+                                 name="%s %s %s %s" % (cases.tuple_name(tup), (M, K, N), orders, mode))
+            p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+            p.lhs.zero_point, p.rhs.zero_point = lzp, rzp
+            announce(p.name)
+            want = O.full_size_expected(p)
+            if want is None:
+                pytest.skip("the stock reference library is not built")
+            before = ctx.sums_in_launch_calls()
+            got = D.device_mul(ctx, p, dst_fill=0)
+            calls += ctx.sums_in_launch_calls() - before
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+        assert calls >= 4, calls   # (the planner may give some of the shapes to other tiles)
+    finally:
+        ctx.close()
+
+
 def test_sums_shared_out_do_not_wait_for_workgroups_beyond_the_last_tile():
     """Grids whose number of tiles is not a multiple of eight are launched with
     a few workgroups beyond the last tile. Where the rows of an operand are
