@@ -209,6 +209,18 @@ struct Cfg {
                                                       : kEpilogueBytes + kParamBytes);
 };
 
+// Lanes that add up one row of a workgroup's share of an operand's rows (the
+// sums shared out over a grid, kRowSums below): half a wave, eight rows of the
+// share at a time, 4 KiB of each per batch of loads. A share of four rows or
+// fewer, deeper than two such batches, gets a whole wave to a row, so that all
+// four waves of the workgroup take part and there are half as many batches to
+// wait for one after the other (1024 x 16384 x 1024 on 64x64 tiles: 42.7 us
+// with half waves, 29.2 us with whole ones, 34.2 us with the sums formed by
+// matrix instructions). Kernel and planner agree through this.
+RUYAMD_HOST_DEVICE inline int LeadShareLanesPerRow(int rows_in_share, int k_bytes) {
+  return rows_in_share <= 4 && k_bytes > 8192 ? 64 : 32;
+}
+
 // kFusedSums (64x64 tile of the int8 kernel; the 128x128 tile for the rows of
 // `a` only): the kernel also forms the
 // depth sums of its rows of `a` and columns of `b` - one more matrix
@@ -230,7 +242,8 @@ struct Cfg {
 // of `a` in passing, dealt out over the first workgroups of every tile row,
 // and can have those of the rows of `b` added up from global memory by the
 // workgroups of its first round, a share each; the 128x128, 128x64 and 64x128
-// tiles have either operand's done that second way (args.row_sums_sides).
+// tiles, and the 64x64 tile on its depth-per-wave schedule, have either
+// operand's done that second way (args.row_sums_sides).
 template <typename Traits, int WM, int WN, int BK, int STAGES, bool kFusedSums = false, bool kFlip = false,
           bool kDepthWaves = false, bool kRowSums = false, bool kSplitLarge = false>
 __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
@@ -322,15 +335,10 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
   // (workgroups beyond the last tile have a share too): the first
   // args.row_sums_producers workgroups, which the hardware starts first and
   // which all fit the device at once, deal the rows out among themselves.
-  auto add_up_share_of = [&](const void* operand, int ld, int rows, uint32_t flip, long long* words) {
-    constexpr int kLanesPerRow = 32;
+  auto add_up_share_with = [&](auto lanes_constant, const void* operand, int ld, int first, int end, uint32_t flip,
+                               long long* words) {
+    constexpr int kLanesPerRow = decltype(lanes_constant)::value;
     constexpr int kRowsPerPass = C::kThreads / kLanesPerRow;
-    const int producers = args.row_sums_producers;
-    // (With the depth of the smallest tile split, grid row 0 holds the producers.)
-    if (int(blockIdx.x) >= producers || blockIdx.y != 0) return;
-    const int rows_per_group = (rows + producers - 1) / producers;
-    const int first = int(blockIdx.x) * rows_per_group;
-    const int end = min(rows, first + rows_per_group);
     const int lane_in_row = threadIdx.x % kLanesPerRow;
     for (int row = first + int(threadIdx.x) / kLanesPerRow; row < end; row += kRowsPerPass) {
       const char* from = static_cast<const char*>(operand) + size_t(row) * size_t(ld);
@@ -362,6 +370,20 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
       if (lane_in_row == 0)
         __hip_atomic_fetch_add(words + row, fused_sums::Contribution(sum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+  };
+  auto add_up_share_of = [&](const void* operand, int ld, int rows, uint32_t flip, long long* words) {
+    const int producers = args.row_sums_producers;
+    // (With the depth of the smallest tile split, grid row 0 holds the producers.)
+    if (int(blockIdx.x) >= producers || blockIdx.y != 0) return;
+    const int rows_per_group = (rows + producers - 1) / producers;
+    const int first = int(blockIdx.x) * rows_per_group;
+    const int end = min(rows, first + rows_per_group);
+    // Half a wave to a row, eight rows at a time; a few long rows get a whole
+    // wave each (LeadShareLanesPerRow).
+    if (LeadShareLanesPerRow(rows_per_group, args.k_bytes) == 64)
+      add_up_share_with(std::integral_constant<int, 64>(), operand, ld, first, end, flip, words);
+    else
+      add_up_share_with(std::integral_constant<int, 32>(), operand, ld, first, end, flip, words);
   };
   auto add_up_rows_of_share = [&]() {
     if (args.row_sums_sides & 1) add_up_share_of(args.a, args.lda, args.M, args.a_flip, args.row_sums);
@@ -2276,12 +2298,16 @@ inline int LeadSumsProducers(const GemmArgs& args, int num_cus, int bm, int bn) 
   return std::min(grid, num_cus * per_cu);
 }
 // What a workgroup's share costs it: it adds up eight rows at a time, 4 KiB of
-// each per batch of loads, and a batch takes a round trip to memory - 0.6 us
+// each per batch of loads (or four rows, 8 KiB of each: LeadShareLanesPerRow),
+// and a batch takes a round trip to memory - 0.6 us
 // when a workgroup has one or two of them, 1.3 us each when all of them have
 // many in flight (measured: 2048^3 0.9 us, 2048 x 8192 x 2048 1.4 us, the
 // 8192 x 8192 right-hand operand of 8192^3 in 32 rows a workgroup 11 us).
 inline int LeadShareBatches(int rows, int k_bytes, int producers) {
-  return ((rows + producers - 1) / producers + 7) / 8 * ((k_bytes + 4095) / 4096);
+  const int share = (rows + producers - 1) / producers;
+  const int lanes = LeadShareLanesPerRow(share, k_bytes);
+  const int rows_per_pass = 256 / lanes, bytes_per_batch = lanes * 128;
+  return (share + rows_per_pass - 1) / rows_per_pass * ((k_bytes + bytes_per_batch - 1) / bytes_per_batch);
 }
 inline double LeadShareMicroseconds(int rows, int k_bytes, int producers) {
   const int batches = LeadShareBatches(rows, k_bytes, producers);
@@ -2297,8 +2323,8 @@ inline double LeadSumsMicroseconds(const GemmArgs& args, int num_cus, int bm, in
 // every wave a step (the depth-per-wave schedule). Measured on 256 tiles with
 // the rows of `a` shared out, against the matrix instructions: 7.8 us for 8.5
 // at 16 steps, 10.4 for 11.3 at 32, 16.5 for 18.3 at 64 - and 42.7 for 32.4
-// at 128 steps, where a workgroup's share takes four batches of loads: two
-// batches a side at most.
+// at 128 steps, where a workgroup's share took four batches of loads: two
+// batches a side at most (which whole waves to a row make of those four).
 inline int SmallestTileParts(const GemmArgs& args, int num_cus) {
   const int tiles = ((args.M + 63) / 64) * ((args.N + 63) / 64);
   return DepthSplitParts(tiles, std::max(1, (args.k_bytes + 127) / 128), num_cus, 16);

@@ -974,7 +974,8 @@ def test_row_sums_formed_by_the_workgroups_of_a_mid_tile_grid(mode):
                 # more tiles than CUs (rings of two stages): the first round's workgroups share the rows out
                 ((S.I8, S.I8, S.I32, S.I8), (2560, 2560, 2560), cases.RCC, 0, -3),       # 400 tiles, one round
                 ((S.U8, S.I8, S.I32, S.I8), (3000, 1024, 3072), cases.RCC, 128, 9),      # 576 tiles, two rounds
-                ((S.I8, S.I8, S.I32, S.I16), (4096, 1024, 1000), (1, 0, 1), 4, 0)]:      # swapped, a wide grid
+                ((S.I8, S.I8, S.I32, S.I16), (4096, 1024, 1000), (1, 0, 1), 4, 0),       # swapped, a wide grid
+                ((S.I8, S.U8, S.I32, S.I8), (1024, 16384, 2048), cases.RCC, 2, 125)]:    # few long rows a workgroup
             p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
                                  name="%s %s %s %s" % (cases.tuple_name(tup), (M, K, N), orders, mode))
             p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
@@ -1022,7 +1023,10 @@ def test_row_sums_shared_out_over_a_grid_of_the_smallest_tile(mode):
                 ((S.U8, S.I8, S.I32, S.I8), (300, 6144, 1500), cases.RCC, 128, 9),
                 ((S.I8, S.I8, S.I32, S.I8), (1024, 1024, 1024), cases.RCC, 0, -3),
                 ((S.I8, S.I8, S.I32, S.I8), (640, 2048, 900), (1, 0, 1), 7, -3),
-                ((S.I8, S.I8, S.I32, S.I8), (1024, 16384, 1024), cases.RCC, 0, -3),     # too deep a share
+                # a few long rows a workgroup: a whole wave to each
+                ((S.I8, S.I8, S.I32, S.I8), (1024, 16384, 1024), cases.RCC, 0, -3),
+                ((S.U8, S.U8, S.I32, S.I16), (1000, 12288 + 64, 700), (1, 0, 1), 128, 128 + 6),
+                ((S.I8, S.I8, S.I32, S.I8), (768, 16384, 768), cases.RCC, 0, -3),       # too deep a share
                 ((S.I8, S.I8, S.I32, S.I8), (192, 8192, 192), cases.RCC, 1, 1)]:
             p = W.random_problem(rng, *tup, M, K, N, *orders, strided=False,
                                  name="%s %s %s %s" % (cases.tuple_name(tup), (M, K, N), orders, mode))
