@@ -408,6 +408,17 @@ bool GemmI8CanFuseSums(const GemmArgs& args, int num_cus) {
   return choice.tile == mfma_gemm::Tile::k128x128 && mfma_gemm::RowSumming128Applies(args, num_cus);
 }
 
+// The smallest tile, asked after the depth split has been planned: the
+// planner's answer, and every wave of the depth-per-wave schedule must have a
+// step of the parts as they are.
+static bool SmallestTileCanShareSumsOut(const GemmArgs& args, int num_cus) {
+  if (args.split_large || !mfma_gemm::SmallestTileSharesSumsOut(args, num_cus)) return false;
+  const int k_steps = std::max(1, (args.k_bytes + 127) / 128);
+  const int parts = std::max(1, args.split_k);
+  return parts <= k_steps && depth_split::StepsPerPart(k_steps, parts) >= 4 &&
+         depth_split::NoEmptyPart(k_steps, parts);
+}
+
 bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   const bool flip = args.a_flip != 0 || args.b_flip != 0;
   const int tiles_m = (args.M + fused_sums::kTileRows - 1) / fused_sums::kTileRows;
@@ -423,7 +434,7 @@ bool GemmI8CanFormRowSums(const GemmArgs& args, int num_cus) {
   if (flip && args.k_bytes % 128 != 0) return false;
   const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
   if (tile == mfma_gemm::Tile::k64x64)
-    return (args.sums_wanted & 1) && !args.split_large && mfma_gemm::SmallestTileSharesSumsOut(args, num_cus);
+    return (args.sums_wanted & 1) && SmallestTileCanShareSumsOut(args, num_cus);
   // The tiles in between: by the workgroups of the grid, each for a share of the rows.
   for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k128x128, 128, 128},
                                     std::tuple{mfma_gemm::Tile::k128x64, 128, 64},
@@ -442,7 +453,7 @@ bool GemmI8CanFormColumnSums(const GemmArgs& args, int num_cus, bool rows_in_lau
   const bool flip = args.a_flip != 0 || args.b_flip != 0;
   if (flip && args.k_bytes % 128 != 0) return false;
   const mfma_gemm::Tile tile = mfma_gemm::PickTile(args, num_cus, mfma_gemm::Model::kInt8);
-  if (tile == mfma_gemm::Tile::k64x64) return mfma_gemm::SmallestTileSharesSumsOut(args, num_cus);
+  if (tile == mfma_gemm::Tile::k64x64) return SmallestTileCanShareSumsOut(args, num_cus);
   // (The largest tile's kernel with sums in its launch always forms those of a's rows.)
   if (tile == mfma_gemm::Tile::k256x256 && !rows_in_launch) return false;
   for (const auto& [mid, bm, bn] : {std::tuple{mfma_gemm::Tile::k256x256, 256, 256},
