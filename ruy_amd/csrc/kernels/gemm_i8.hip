@@ -31,6 +31,7 @@ __device__ __forceinline__ int32_t Median3(int32_t x, int32_t lo, int32_t hi) {
 }
 
 struct Int8Traits16;
+struct Int8Traits16StreamingA;
 
 struct Int8Traits {
   using Acc = v16i;
@@ -43,6 +44,7 @@ struct Int8Traits {
   static constexpr bool kPaired = false;
   // The 256x256 tile runs on 16x16 blocks (below).
   using LargeTile = Int8Traits16;
+  using LargeTileStreamingA = Int8Traits16StreamingA;
   static constexpr bool kSplitB = false;
   static constexpr mfma_gemm::Model kModel = mfma_gemm::Model::kInt8;
   static __device__ __forceinline__ int Bits(int x, int) { return x; }
@@ -319,6 +321,12 @@ struct Int8Traits16 : Int8Traits {
       vals[q] = Median3(v, ep.clamp_min_i, ep.clamp_max_i);
     }
   }
+};
+
+// The same kernel fetching `a` with the non-temporal cache policy
+// (mfma_gemm::StreamsLargeA says for which launches).
+struct Int8Traits16StreamingA : Int8Traits16 {
+  static constexpr bool kStreamA = true;
 };
 
 // int8 x int16 (ruy/kernel_avx512.cc:55-626 instantiated for a 16-bit RHS,

@@ -141,6 +141,16 @@ __device__ __forceinline__ void SetLdsTargetAt(uint32_t lds_base) {
 __device__ __forceinline__ void LoadToLdsTarget16(uint32_t voffset, uint32_t soffset, v4i rsrc) {
   asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
 }
+// The same with the non-temporal cache policy: for an operand that the launch
+// reads exactly once, so that it does not push the other one out of L2.
+__device__ __forceinline__ void LoadToLdsTarget16Streaming(uint32_t voffset, uint32_t soffset, v4i rsrc) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen nt lds" : : "v"(voffset), "s"(rsrc), "s"(soffset) : "memory");
+}
+// Whether a Traits asks for that on the `a` operand (a member kStreamA; absent: no).
+template <class T, class = void>
+struct StreamsA : std::false_type {};
+template <class T>
+struct StreamsA<T, std::void_t<decltype(T::kStreamA)>> : std::bool_constant<T::kStreamA> {};
 
 // f(std::integral_constant<int, 0>()), ..., f(std::integral_constant<int, N - 1>()).
 template <class F, int... Is>
@@ -1112,7 +1122,9 @@ __device__ __forceinline__ void MfmaGemmBody(const GemmArgs args) {
               wave_targets);
         constexpr ps::Load load = ps::LoadBehind(n);
         if constexpr (load.valid) {
-          if constexpr (decltype(full)::value)
+          if constexpr (decltype(full)::value && !load.is_b && StreamsA<Traits>::value)
+            LoadToLdsTarget16Streaming(a_goff[load.index], refill_offset, a_rsrc);
+          else if constexpr (decltype(full)::value)
             LoadToLdsTarget16(load.is_b ? b_goff[load.index] : a_goff[load.index], refill_offset,
                               load.is_b ? b_rsrc : a_rsrc);
           else
@@ -2431,6 +2443,18 @@ inline bool ShallowRing(const GemmArgs& args, int num_cus, int bm, int bn) {
   return TileCount(args, bm, bn) > num_cus;
 }
 
+// Whether the 256x256 tile's split kernel should fetch `a` with the
+// non-temporal policy: a single column of tiles, so that no second workgroup
+// ever asks for the same bytes, and an operand too large to stay in any cache.
+// Measured, same card, default policy -> non-temporal: 16384 x 16384 x 256 in
+// four parts 104 -> 81 us, 32768 x 8192 x 256 in two 99 -> 80 us, 24576 x
+// 16384 x 256 in two 144 -> 126 us, 16384 x 32768 x 256 in four 183 -> 169 us;
+// operands of 128 MiB lose 2 % by it (8192 x 16384 x 256 56.7 -> 58.2 us), and
+// where the operand is reused the policy costs 4 % (8192^3).
+inline bool StreamsLargeA(const GemmArgs& args) {
+  return args.N <= 256 && double(args.M) * args.k_bytes >= 192.0 * 1024 * 1024;
+}
+
 // The depth split of the 256x256 int8 tile (a kernel of its own, kSplitLarge):
 // for destinations of so few tiles that the 256x256 grid leaves most CUs idle,
 // with depths so long that a part still has kLargeSplitMinSteps ring steps.
@@ -2449,7 +2473,7 @@ constexpr double kLargeSplitFixed = 1.5, kLargeSplitPerMiB = 0.18;
 // The modelled time of the split into `parts` (a whole number of rounds is not
 // needed: the parts all run at once).
 inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps, int parts, int num_cus,
-                                     double operand_bytes) {
+                                     double operand_bytes, bool streams_a = false) {
   const double fraction = double(tiles * parts) / num_cus;
   // (A workgroup moves its own (2 - 1/parts) * 256 KiB at 60 GB/s or so: what
   // the exchange costs at least, however few workgroups there are.)
@@ -2461,19 +2485,20 @@ inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps
   const double main_loop = (t.last_round + (1 - t.last_round) * fraction) * t.step *
                            (t.overhead + depth_split::StepsPerPart(k_steps, parts));
   // (... with a workgroup on every CU; fewer of them stream less: 2.8 TB/s with 128.)
-  const double streaming = operand_bytes / (3.5e6 * std::sqrt(std::min(1.0, fraction)));
+  // (3.8 TB/s with the non-temporal policy on `a`, StreamsLargeA.)
+  const double streaming = operand_bytes / ((streams_a ? 3.8e6 : 3.5e6) * std::sqrt(std::min(1.0, fraction)));
   return t.fixed + std::max(main_loop, streaming) + kLargeSplitFixed + exchange;
 }
 // The best number of parts (2, 4, 8) by that model among those that fit the
 // CUs at once and leave every part kLargeSplitMinSteps steps; 1 if none does.
 inline int LargeSplitPartsWanted(const TileTiming& t, int tiles, int k_steps, int num_cus, double operand_bytes,
-                                 double* time) {
+                                 double* time, bool streams_a = false) {
   if (tiles <= 0 || tiles * depth_split::kLargeWordsPerTile > kSplitCounters) return 1;
   const int most = std::min(num_cus / tiles, k_steps / kLargeSplitMinSteps);
   int best = 1;
   for (int parts = 2; parts <= depth_split::kLargeMaxParts; parts *= 2) {
     if (parts > most || !depth_split::NoEmptyPart(k_steps, parts)) continue;
-    const double modelled = LargeSplitMicroseconds(t, tiles, k_steps, parts, num_cus, operand_bytes);
+    const double modelled = LargeSplitMicroseconds(t, tiles, k_steps, parts, num_cus, operand_bytes, streams_a);
     if (best == 1 || modelled < *time) {
       best = parts;
       *time = modelled;
@@ -2515,8 +2540,8 @@ inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
     const TileTiming& t = model.tiles[0];
     const int tiles = TileCount(args, t.bm, t.bn);
     double time = 0;
-    const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus,
-                                            (double(args.M) + args.N) * args.k_bytes, &time);
+    const double operand_bytes = (double(args.M) + args.N) * args.k_bytes;
+    const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus, operand_bytes, &time, StreamsLargeA(args));
     double unused_factor;
     time += PendingSumsMicroseconds(args, num_cus, model, t, &unused_factor);
     // What the split is held against. The smallest tile's step was fitted to
@@ -2531,6 +2556,20 @@ inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
       const int small_parts = DepthSplitParts(small_tiles, k_steps, num_cus, model.min_steps_per_part);
       const double busy = std::min(1.0, double(small_tiles) * small_parts / num_cus);
       if (busy >= 0.75) against += 0.06 * depth_split::StepsPerPart(k_steps, small_parts) * busy;
+    }
+    // One column of large tiles over a long `a`: every byte of it is read
+    // once, from memory, and the unsplit tiles then run at the rate they stream
+    // it at, which their fitted steps (operands mostly found in L2) do not
+    // show: 2.1 TB/s on 128x128 tiles (16384 x 16384 x 256: 127 us, 16384 x
+    // 8192 x 256: 66 us, 24576 x 16384 x 256: 199 us), 3.5 TB/s on a full grid
+    // of the largest (32768 x 16384 x 256, 128 workgroups: 217 us). (Not so for
+    // a long `b` under one row of tiles: 256 x 16384 x 16384 takes 78 us on
+    // 128x128 tiles and 100 us in four parts of the largest.)
+    if (args.N <= 256 && operand_bytes >= 64.0 * 1024 * 1024 && (best == Tile::k128x128 || best == Tile::k256x256)) {
+      const int bm = best == Tile::k128x128 ? 128 : 256;
+      const double busy = std::min(1.0, double(TileCount(args, bm, bm)) / num_cus);
+      const double rate = best == Tile::k128x128 ? 2.1e6 : 3.5e6;
+      against = std::max(against, operand_bytes / (rate * std::sqrt(busy)));
     }
     if (parts > 1 && time < against) large_parts = parts;
   }
@@ -2612,6 +2651,17 @@ template <typename Traits, bool kFlip = false>
 hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int num_cus) {
   switch (tile) {
     case Tile::k256x256:
+      // One column of tiles over a large `a`: every byte of it is read once,
+      // with the cache policy for that (StreamsLargeA).
+      if constexpr (Traits::LargeTile::kPaired && !kFlip) {
+        if (args.split_k > 1 && StreamsLargeA(args)) {
+          if (args.row_sums)
+            return Launch<typename Traits::LargeTileStreamingA, 4, 4, 128, 2, false, false, false, true, true>(stream,
+                                                                                                              args);
+          return Launch<typename Traits::LargeTileStreamingA, 4, 4, 128, 2, false, false, false, false, true>(stream,
+                                                                                                             args);
+        }
+      }
       if constexpr (Traits::LargeTile::kPaired) {
         if (args.row_sums && args.split_k > 1)
           return Launch<typename Traits::LargeTile, 4, 4, 128, 2, false, kFlip, false, true, true>(stream, args);

@@ -1046,6 +1046,35 @@ def test_row_sums_shared_out_over_a_grid_of_the_smallest_tile(mode):
         ctx.close()
 
 
+def test_long_operand_under_one_column_of_large_tiles(device_ctx):
+    """A destination of 256 columns or fewer under a left-hand operand of
+    hundreds of MiB: one column of 256x256 tiles with the depth in parts, the
+    long operand fetched with the non-temporal cache policy (int8 data; uint8
+    data used in place keeps the default one). With and without zero points,
+    a ragged width, a raw int32 destination: every element against the stock
+    library."""
+    from ruy_amd import api
+    from ruy_amd import device_problem as D
+    rng = np.random.default_rng(2718)
+    for tup, (M, K, N), lzp, rzp in [
+            ((S.I8, S.I8, S.I32, S.I8), (16384, 16384, 256), 0, -3),
+            ((S.I8, S.I8, S.I32, S.I32), (32768, 8192, 256), 0, 0),
+            ((S.I8, S.U8, S.I32, S.I16), (16384, 12288 + 128, 200), 5, 128 + 2),
+            ((S.U8, S.I8, S.I32, S.U8), (24576, 8192, 250), 131, 0)]:
+        assert api.tile_for(0, M, K, N)[:2] == (256, 256) and api.tile_for(0, M, K, N)[2] > 1
+        p = W.random_problem(rng, *tup, M, K, N, *cases.RCC, strided=False,
+                             name="%s %s" % (cases.tuple_name(tup), (M, K, N)))
+        p.lhs.cache_policy = p.rhs.cache_policy = S.CACHE_NEVER
+        p.lhs.zero_point, p.rhs.zero_point = lzp, rzp
+        announce(p.name)
+        want = O.full_size_expected(p)
+        if want is None:
+            pytest.skip("the stock reference library is not built")
+        got = D.device_mul(device_ctx, p, dst_fill=0)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "%s: %d of %d elements differ, first at %d" % (p.name, bad.size, got.size, bad[0])
+
+
 def test_sums_shared_out_do_not_wait_for_workgroups_beyond_the_last_tile():
     """Grids whose number of tiles is not a multiple of eight are launched with
     a few workgroups beyond the last tile. Where the rows of an operand are
