@@ -2653,12 +2653,12 @@ hipError_t LaunchTile(hipStream_t stream, const GemmArgs& args, Tile tile, int n
     case Tile::k256x256:
       // One column of tiles over a large `a`: every byte of it is read once,
       // with the cache policy for that (StreamsLargeA).
-      if constexpr (Traits::LargeTile::kPaired && !kFlip) {
+      if constexpr (Traits::LargeTile::kPaired) {
         if (args.split_k > 1 && StreamsLargeA(args)) {
           if (args.row_sums)
-            return Launch<typename Traits::LargeTileStreamingA, 4, 4, 128, 2, false, false, false, true, true>(stream,
+            return Launch<typename Traits::LargeTileStreamingA, 4, 4, 128, 2, false, kFlip, false, true, true>(stream,
                                                                                                               args);
-          return Launch<typename Traits::LargeTileStreamingA, 4, 4, 128, 2, false, false, false, false, true>(stream,
+          return Launch<typename Traits::LargeTileStreamingA, 4, 4, 128, 2, false, kFlip, false, false, true>(stream,
                                                                                                              args);
         }
       }

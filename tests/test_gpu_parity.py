@@ -1049,8 +1049,8 @@ def test_row_sums_shared_out_over_a_grid_of_the_smallest_tile(mode):
 def test_long_operand_under_one_column_of_large_tiles(device_ctx):
     """A destination of 256 columns or fewer under a left-hand operand of
     hundreds of MiB: one column of 256x256 tiles with the depth in parts, the
-    long operand fetched with the non-temporal cache policy (int8 data; uint8
-    data used in place keeps the default one). With and without zero points,
+    long operand fetched with the non-temporal cache policy (int8 data, and
+    uint8 data used in place). With and without zero points,
     a ragged width, a raw int32 destination: every element against the stock
     library."""
     from ruy_amd import api
