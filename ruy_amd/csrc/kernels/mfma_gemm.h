@@ -2473,7 +2473,7 @@ constexpr double kLargeSplitFixed = 1.5, kLargeSplitPerMiB = 0.18;
 // The modelled time of the split into `parts` (a whole number of rounds is not
 // needed: the parts all run at once).
 inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps, int parts, int num_cus,
-                                     double operand_bytes, bool streams_a = false) {
+                                     double operand_bytes, double streaming_rate = 3.5e6) {
   const double fraction = double(tiles * parts) / num_cus;
   // (A workgroup moves its own (2 - 1/parts) * 256 KiB at 60 GB/s or so: what
   // the exchange costs at least, however few workgroups there are.)
@@ -2485,20 +2485,22 @@ inline double LargeSplitMicroseconds(const TileTiming& t, int tiles, int k_steps
   const double main_loop = (t.last_round + (1 - t.last_round) * fraction) * t.step *
                            (t.overhead + depth_split::StepsPerPart(k_steps, parts));
   // (... with a workgroup on every CU; fewer of them stream less: 2.8 TB/s with 128.)
-  // (3.8 TB/s with the non-temporal policy on `a`, StreamsLargeA.)
-  const double streaming = operand_bytes / ((streams_a ? 3.8e6 : 3.5e6) * std::sqrt(std::min(1.0, fraction)));
+  // (`streaming_rate`: what ChooseTile knows better for one column of tiles;
+  // measured with a workgroup on three CUs of four or more.)
+  const double rate = fraction >= 0.75 ? streaming_rate : std::min(streaming_rate, 3.5e6);
+  const double streaming = operand_bytes / (rate * std::sqrt(std::min(1.0, fraction)));
   return t.fixed + std::max(main_loop, streaming) + kLargeSplitFixed + exchange;
 }
 // The best number of parts (2, 4, 8) by that model among those that fit the
 // CUs at once and leave every part kLargeSplitMinSteps steps; 1 if none does.
 inline int LargeSplitPartsWanted(const TileTiming& t, int tiles, int k_steps, int num_cus, double operand_bytes,
-                                 double* time, bool streams_a = false) {
+                                 double* time, double streaming_rate = 3.5e6) {
   if (tiles <= 0 || tiles * depth_split::kLargeWordsPerTile > kSplitCounters) return 1;
   const int most = std::min(num_cus / tiles, k_steps / kLargeSplitMinSteps);
   int best = 1;
   for (int parts = 2; parts <= depth_split::kLargeMaxParts; parts *= 2) {
     if (parts > most || !depth_split::NoEmptyPart(k_steps, parts)) continue;
-    const double modelled = LargeSplitMicroseconds(t, tiles, k_steps, parts, num_cus, operand_bytes, streams_a);
+    const double modelled = LargeSplitMicroseconds(t, tiles, k_steps, parts, num_cus, operand_bytes, streaming_rate);
     if (best == 1 || modelled < *time) {
       best = parts;
       *time = modelled;
@@ -2541,7 +2543,13 @@ inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
     const int tiles = TileCount(args, t.bm, t.bn);
     double time = 0;
     const double operand_bytes = (double(args.M) + args.N) * args.k_bytes;
-    const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus, operand_bytes, &time, StreamsLargeA(args));
+    // One column of tiles: the long operand streams at 3.8 TB/s with the
+    // non-temporal policy (StreamsLargeA), and one of up to 160 MB at 4.5 TB/s
+    // (16384 x 8192 x 256 in four parts: 53 us, 12288 x 8192 x 256: 47 us).
+    const double streaming_rate = StreamsLargeA(args)                       ? 3.8e6
+                                  : args.N <= 256 && operand_bytes <= 160e6 ? 4.5e6
+                                                                            : 3.5e6;
+    const int parts = LargeSplitPartsWanted(t, tiles, k_steps, num_cus, operand_bytes, &time, streaming_rate);
     double unused_factor;
     time += PendingSumsMicroseconds(args, num_cus, model, t, &unused_factor);
     // What the split is held against. The smallest tile's step was fitted to
@@ -2565,11 +2573,18 @@ inline TileChoice ChooseTile(const GemmArgs& args, int num_cus, Model which) {
     // of the largest (32768 x 16384 x 256, 128 workgroups: 217 us). (Not so for
     // a long `b` under one row of tiles: 256 x 16384 x 16384 takes 78 us on
     // 128x128 tiles and 100 us in four parts of the largest.)
-    if (args.N <= 256 && operand_bytes >= 64.0 * 1024 * 1024 && (best == Tile::k128x128 || best == Tile::k256x256)) {
-      const int bm = best == Tile::k128x128 ? 128 : 256;
-      const double busy = std::min(1.0, double(TileCount(args, bm, bm)) / num_cus);
-      const double rate = best == Tile::k128x128 ? 2.1e6 : 3.5e6;
-      against = std::max(against, operand_bytes / (rate * std::sqrt(busy)));
+    // (The tiles of 64 rows or columns the same where they take more than two
+    // tile columns: 16384 x 8192 x 256 on 128x64 tiles 66 us, 16384 x 16384 x
+    // 256 133 us.)
+    const bool mid_tile_floor = best == Tile::k128x128 || (args.N > 128 && best != Tile::k256x256);
+    if (args.N <= 256 && operand_bytes >= 64.0 * 1024 * 1024 && best != model.smallest &&
+        (mid_tile_floor || best == Tile::k256x256)) {
+      for (int i = 0; i < model.count; ++i) {
+        if (model.tiles[i].tile != best) continue;
+        const double busy = std::min(1.0, double(TileCount(args, model.tiles[i].bm, model.tiles[i].bn)) / num_cus);
+        const double rate = best == Tile::k256x256 ? 3.5e6 : 2.1e6;
+        against = std::max(against, operand_bytes / (rate * std::sqrt(busy)));
+      }
     }
     if (parts > 1 && time < against) large_parts = parts;
   }
